@@ -1,0 +1,106 @@
+/* C ABI of libnq_gfx950.so: the binary low-rank linear layer on AMD gfx950 (MI355X).
+ *
+ * Every entry point takes raw device pointers, sizes and a HIP stream, enqueues its kernels on that
+ * stream and returns without synchronising.  Nothing here allocates or frees device memory and no
+ * pointer is kept after return; scratch buffers are passed in by the caller.  Return value: NQ_OK or
+ * a negative nq_status; nq_status_string() gives the message (the messages of argument errors are
+ * the ones the reference's host wrappers raise).
+ *
+ * Reference paths are relative to the reference checkout; "kernel/" = src/nanoquant/kernel/.
+ * Operand naming follows the mathematics, not the reference's swapped argument names:
+ *   vt_bits [r, ceil(n/32)]  first-stage factor  (reference op argument `Ubits`, module attr V_int8)
+ *   u_bits  [m, ceil(r/32)]  second-stage factor (reference op argument `Vbits`, module attr U_int8)
+ * Packed words use the row-major "half2" order of kernel/utils.py:99-104: element k of a 32-group
+ * sits at bit 15 - (k>>1) + 16*(k&1); bit 1 encodes -1, bit 0 encodes +1.
+ */
+#ifndef NQ_GFX950_H
+#define NQ_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum nq_dtype { NQ_F16 = 0, NQ_BF16 = 1 } nq_dtype;
+
+typedef enum nq_status {
+    NQ_OK = 0,
+    NQ_ERR_DTYPE = -1,        /* "Support only Half or BFloat16" (kernel/cuda/gemv_kernel.cu:318) */
+    NQ_ERR_NULL = -2,         /* a required pointer is NULL */
+    NQ_ERR_SHAPE = -3,        /* a size is negative or inconsistent */
+    NQ_ERR_K_MISMATCH = -4,   /* "k dimension mismatch" (kernel/cuda/gemm.cpp:48) */
+    NQ_ERR_PROB_SHAPE = -5,   /* "Problem shape incompatible" (kernel/cuda/gemm.cpp:93) */
+    NQ_ERR_WORKSPACE = -6,    /* "workspace too small" (kernel/cuda/gemm.cpp:52) */
+    NQ_ERR_ORDER = -7,        /* unknown word order id */
+    NQ_ERR_ALIGN = -8,        /* a prefill operand is not 16-byte aligned */
+    NQ_ERR_HIP = -100         /* a HIP call failed; see nq_last_hip_error() */
+} nq_status;
+
+typedef enum nq_word_order { NQ_ORDER_LSB_FIRST = 0, NQ_ORDER_HALF2 = 1 } nq_word_order;
+
+typedef enum nq_device_attr { NQ_ATTR_CU_COUNT = 0, NQ_ATTR_LDS_BYTES = 1, NQ_ATTR_WAVE_SIZE = 2 } nq_device_attr;
+
+const char* nq_status_string(int status);
+int nq_last_hip_error(void);          /* hipError_t of the most recent NQ_ERR_HIP on this thread */
+int nq_abi_version(void);
+int nq_device_query(int attr, int* value);   /* current device */
+
+/* Decode path, one term:  y = s_out * (U (s_mid * (Vt (s_in * x)))).
+ * Replaces nanoquant_dyn_forward (kernel/cuda/gemv_kernel.cu:308-429; schema kernel/pybind.cpp:86-90).
+ *   x [batch, n], s_in [n], s_mid [r] or NULL, s_out [m], y [batch, m]: all of `dtype`, contiguous.
+ *   h_scratch: fp32 [batch, r] owned by the caller (the reference allocates `interm` itself, :345).
+ * Any batch >= 1 is accepted; every packed word is read once per 16 batch rows. */
+int nq_gemv_forward(const void* x, const void* s_in, const uint32_t* vt_bits, const void* s_mid,
+                    const uint32_t* u_bits, const void* s_out, float* h_scratch, void* y,
+                    int batch, int n, int r, int m, int dtype, void* stream);
+
+/* Decode path, sum of `nterms` terms that share x (the mixture-of-rank layer; no counterpart in the
+ * reference's code, defined as the sum of single-term layers).  Arrays hold one pointer / rank per
+ * term; s_mid[t] may be NULL.  h_scratch: fp32 [batch, max r]; y_scratch: fp32 [batch, m]. */
+int nq_gemv_mixture(const void* x, const void* const* s_in, const uint32_t* const* vt_bits,
+                    const void* const* s_mid, const uint32_t* const* u_bits, const void* const* s_out,
+                    const int* r, int nterms, float* h_scratch, float* y_scratch, void* y,
+                    int batch, int n, int m, int dtype, void* stream);
+
+/* One matmul-free stage: out[b,row] = s_row[row] * sum_c sgn(bits[row,c]) * in[b,c] * s_col[c].
+ * Replaces nanoquant_stage1_dyn_kernel / nanoquant_stage2_dyn_kernel launches
+ * (kernel/cuda/gemv_kernel.cu:283-301).  in/out are `dtype`; s_col, s_row may be NULL. */
+int nq_gemv_stage(const void* in, const void* s_col, const uint32_t* bits, const void* s_row, void* out,
+                  int batch, int cols, int rows, int dtype, void* stream);
+
+/* Prefill path, single matrix:  y[t, j] = s_out[j] * sum_k (x[t, k] * s_in[k]) * sgn(W)[j, k].
+ * Replaces marlin_onebit_cuda (kernel/cuda/gemm.cpp:59-98; schema kernel/pybind.cpp:93-98).
+ *   x [tokens, k], y [tokens, rows], s_in [k] or NULL, s_out [rows] or NULL: `dtype`, contiguous.
+ *   tiles: k*rows/32 words in the 32-row x 256-k tile layout of the package's prefill packer (the
+ *   layout is private to packer and kernel, as the reference's Marlin layout is).
+ *   Requires k % 256 == 0 and rows % 32 == 0 (else NQ_ERR_PROB_SHAPE, the reference's error class
+ *   for shapes its tiles do not cover).  scratch: nq_gemm_scratch_bytes(tokens, k, rows) bytes of
+ *   device memory (may be NULL when that is 0); it holds fp32 partial sums when k is split. */
+size_t nq_gemm_scratch_bytes(int tokens, int k, int rows);
+int nq_gemm_onebit(const void* x, const uint32_t* tiles, const void* s_in, const void* s_out, void* y,
+                   void* scratch, size_t scratch_bytes, int tokens, int k, int rows, int dtype, void* stream);
+
+/* Prefill path, one term: two chained one-bit GEMMs with the intermediate h [tokens, r] (`dtype`,
+ * caller-owned) between them.  Replaces marlin_nanoquant_cuda (kernel/cuda/gemm.cpp:112-122; schema
+ * kernel/pybind.cpp:99-104).  vt_tiles: first stage [r rows x n], u_tiles: second stage [m rows x r];
+ * r is the padded rank (multiple of 256, padded entries carry a zero s_mid).
+ * scratch: max of nq_gemm_scratch_bytes(tokens, n, r) and nq_gemm_scratch_bytes(tokens, r, m). */
+int nq_gemm_nanoquant(const void* x, const uint32_t* vt_tiles, const uint32_t* u_tiles, const void* s_in,
+                      const void* s_mid, const void* s_out, void* h, void* y, void* scratch,
+                      size_t scratch_bytes, int tokens, int n, int r, int m, int dtype, void* stream);
+
+/* Word-order conversion on the device, in place allowed (dst == src): the checkpoint format
+ * ("lsb_first", modules/linear.py:298) to the kernel format ("half2", modules/linear.py:171-172)
+ * without the dense round trip of utils/load_utils.py:269-293.  order ids: nq_word_order. */
+int nq_repack_words(const uint32_t* src, uint32_t* dst, size_t nwords, int src_order, int dst_order, void* stream);
+
+/* Plain device copy kernel of known traffic (bytes read + bytes written); used to calibrate the
+ * memory counters of a profiler.  bytes must be a multiple of 16. */
+int nq_stream_copy(void* dst, const void* src, size_t bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NQ_GFX950_H */

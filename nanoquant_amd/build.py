@@ -1,0 +1,33 @@
+"""hipcc build of libnq_gfx950.so (the only native artefact of the package)."""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(_HERE, "csrc")
+LIB_PATH = os.path.join(_HERE, "libnq_gfx950.so")
+SOURCES = ("nq_gemv.hip", "nq_gemm.hip", "nq_util.hip", "nq_api.hip")
+# -packed-fp32-ops off: hipcc may otherwise fuse scalar float code into packed-fp32 instructions.
+FLAGS = ("--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-munsafe-fp-atomics",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops")
+
+
+def build(verbose: bool = False) -> str:
+    """Compile every HIP source for gfx950 and link the shared library in-tree.  Always recompiles."""
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    tmp = LIB_PATH + ".tmp"
+    cmd = [hipcc, *FLAGS, *srcs, "-o", tmp]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + res.stdout + res.stderr)
+    if verbose and res.stderr:
+        print(res.stderr)
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

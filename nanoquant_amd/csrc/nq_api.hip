@@ -1,0 +1,148 @@
+// extern "C" surface of libnq_gfx950.so: argument checks, then kernel launches on the caller's
+// stream.  No allocation, no synchronisation, no retained pointers.
+#include "../../include/nq_gfx950.h"
+#include "nq_kernels.h"
+
+namespace {
+thread_local int g_last_hip_error = 0;
+
+int hip_status(hipError_t e) {
+    if (e == hipSuccess) return NQ_OK;
+    g_last_hip_error = (int)e;
+    (void)hipGetLastError();  // clear the sticky launch error so later calls report their own
+    return NQ_ERR_HIP;
+}
+
+inline int words_of(int cols) { return (cols + 31) / 32; }
+}  // namespace
+
+extern "C" {
+
+const char* nq_status_string(int status) {
+    switch (status) {
+        case NQ_OK: return "ok";
+        case NQ_ERR_DTYPE: return "Support only Half or BFloat16";
+        case NQ_ERR_NULL: return "required pointer is null";
+        case NQ_ERR_SHAPE: return "invalid or inconsistent sizes";
+        case NQ_ERR_K_MISMATCH: return "k dimension mismatch";
+        case NQ_ERR_PROB_SHAPE: return "Problem shape incompatible";
+        case NQ_ERR_WORKSPACE: return "workspace too small";
+        case NQ_ERR_ORDER: return "unknown word order";
+        case NQ_ERR_ALIGN: return "prefill operands must be 16-byte aligned";
+        case NQ_ERR_HIP: return "HIP runtime error";
+        default: return "unknown status";
+    }
+}
+
+int nq_last_hip_error(void) { return g_last_hip_error; }
+
+int nq_abi_version(void) { return 1; }
+
+int nq_device_query(int attr, int* value) {
+    if (!value) return NQ_ERR_NULL;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_status(e);
+    hipDeviceAttribute_t which;
+    switch (attr) {
+        case NQ_ATTR_CU_COUNT: which = hipDeviceAttributeMultiprocessorCount; break;
+        case NQ_ATTR_LDS_BYTES: which = hipDeviceAttributeMaxSharedMemoryPerBlock; break;
+        case NQ_ATTR_WAVE_SIZE: which = hipDeviceAttributeWarpSize; break;
+        default: return NQ_ERR_SHAPE;
+    }
+    return hip_status(hipDeviceGetAttribute(value, which, dev));
+}
+
+int nq_gemv_forward(const void* x, const void* s_in, const uint32_t* vt_bits, const void* s_mid,
+                    const uint32_t* u_bits, const void* s_out, float* h_scratch, void* y,
+                    int batch, int n, int r, int m, int dtype, void* stream) {
+    if (dtype != NQ_F16 && dtype != NQ_BF16) return NQ_ERR_DTYPE;
+    if (batch < 0 || n < 0 || r < 0 || m < 0) return NQ_ERR_SHAPE;
+    if (batch == 0 || m == 0) return NQ_OK;
+    if (!x || !s_in || !vt_bits || !u_bits || !s_out || !h_scratch || !y) return NQ_ERR_NULL;
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e = nq::gemv_stage(dtype, true, vt_bits, x, s_in, s_mid, nullptr, h_scratch, true, batch, r,
+                                  words_of(n), n, n, r, st);
+    if (e != hipSuccess) return hip_status(e);
+    e = nq::gemv_stage(dtype, false, u_bits, h_scratch, nullptr, s_out, nullptr, y, false, batch, m,
+                       words_of(r), r, r, m, st);
+    return hip_status(e);
+}
+
+int nq_gemv_mixture(const void* x, const void* const* s_in, const uint32_t* const* vt_bits,
+                    const void* const* s_mid, const uint32_t* const* u_bits, const void* const* s_out,
+                    const int* r, int nterms, float* h_scratch, float* y_scratch, void* y,
+                    int batch, int n, int m, int dtype, void* stream) {
+    if (dtype != NQ_F16 && dtype != NQ_BF16) return NQ_ERR_DTYPE;
+    if (batch < 0 || n < 0 || m < 0 || nterms < 1) return NQ_ERR_SHAPE;
+    if (!x || !s_in || !vt_bits || !s_mid || !u_bits || !s_out || !r || !h_scratch || !y) return NQ_ERR_NULL;
+    if (nterms > 1 && !y_scratch) return NQ_ERR_NULL;
+    for (int t = 0; t < nterms; ++t) {
+        if (r[t] < 0) return NQ_ERR_SHAPE;
+        if (!s_in[t] || !vt_bits[t] || !u_bits[t] || !s_out[t]) return NQ_ERR_NULL;
+    }
+    if (batch == 0 || m == 0) return NQ_OK;
+    hipStream_t st = (hipStream_t)stream;
+    for (int t = 0; t < nterms; ++t) {
+        hipError_t e = nq::gemv_stage(dtype, true, vt_bits[t], x, s_in[t], s_mid[t], nullptr, h_scratch, true,
+                                      batch, r[t], words_of(n), n, n, r[t], st);
+        if (e != hipSuccess) return hip_status(e);
+        const bool last = (t == nterms - 1);
+        // Partial sums over terms stay in fp32; only the last term rounds to the activation type.
+        e = nq::gemv_stage(dtype, false, u_bits[t], h_scratch, nullptr, s_out[t], t ? y_scratch : nullptr,
+                           last ? y : (void*)y_scratch, !last, batch, m, words_of(r[t]), r[t], r[t], m, st);
+        if (e != hipSuccess) return hip_status(e);
+    }
+    return NQ_OK;
+}
+
+int nq_gemv_stage(const void* in, const void* s_col, const uint32_t* bits, const void* s_row, void* out,
+                  int batch, int cols, int rows, int dtype, void* stream) {
+    if (dtype != NQ_F16 && dtype != NQ_BF16) return NQ_ERR_DTYPE;
+    if (batch < 0 || cols < 0 || rows < 0) return NQ_ERR_SHAPE;
+    if (batch == 0 || rows == 0) return NQ_OK;
+    if (!in || !bits || !out) return NQ_ERR_NULL;
+    return hip_status(nq::gemv_stage(dtype, true, bits, in, s_col, s_row, nullptr, out, false, batch, rows,
+                                     words_of(cols), cols, cols, rows, (hipStream_t)stream));
+}
+
+size_t nq_gemm_scratch_bytes(int tokens, int k, int rows) { return nq::gemm_scratch_bytes(tokens, k, rows); }
+
+int nq_gemm_onebit(const void* x, const uint32_t* tiles, const void* s_in, const void* s_out, void* y,
+                   void* scratch, size_t scratch_bytes, int tokens, int k, int rows, int dtype, void* stream) {
+    if (dtype != NQ_F16 && dtype != NQ_BF16) return NQ_ERR_DTYPE;
+    if (tokens < 0 || k < 0 || rows < 0) return NQ_ERR_SHAPE;
+    if (k % 256 != 0 || rows % 32 != 0) return NQ_ERR_PROB_SHAPE;
+    if (tokens == 0 || rows == 0 || k == 0) return NQ_OK;
+    if (!x || !tiles || !y) return NQ_ERR_NULL;
+    if (((uintptr_t)x | (uintptr_t)tiles | (uintptr_t)y | (uintptr_t)s_in | (uintptr_t)scratch) & 15u) return NQ_ERR_ALIGN;
+    const size_t need = nq::gemm_scratch_bytes(tokens, k, rows);
+    if (need > 0 && (!scratch || scratch_bytes < need)) return NQ_ERR_WORKSPACE;
+    return hip_status(nq::gemm_onebit(dtype, x, tiles, s_in, s_out, y, (float*)scratch, tokens, k, rows,
+                                      (hipStream_t)stream));
+}
+
+int nq_gemm_nanoquant(const void* x, const uint32_t* vt_tiles, const uint32_t* u_tiles, const void* s_in,
+                      const void* s_mid, const void* s_out, void* h, void* y, void* scratch,
+                      size_t scratch_bytes, int tokens, int n, int r, int m, int dtype, void* stream) {
+    if (!h) return (tokens == 0 || m == 0) ? NQ_OK : NQ_ERR_NULL;
+    int st = nq_gemm_onebit(x, vt_tiles, s_in, s_mid, h, scratch, scratch_bytes, tokens, n, r, dtype, stream);
+    if (st != NQ_OK) return st;
+    return nq_gemm_onebit(h, u_tiles, nullptr, s_out, y, scratch, scratch_bytes, tokens, r, m, dtype, stream);
+}
+
+int nq_repack_words(const uint32_t* src, uint32_t* dst, size_t nwords, int src_order, int dst_order, void* stream) {
+    if ((src_order != 0 && src_order != 1) || (dst_order != 0 && dst_order != 1)) return NQ_ERR_ORDER;
+    if (nwords == 0) return NQ_OK;
+    if (!src || !dst) return NQ_ERR_NULL;
+    return hip_status(nq::repack_words(src, dst, nwords, src_order, dst_order, (hipStream_t)stream));
+}
+
+int nq_stream_copy(void* dst, const void* src, size_t bytes, void* stream) {
+    if (bytes % 16 != 0) return NQ_ERR_SHAPE;
+    if (bytes == 0) return NQ_OK;
+    if (!src || !dst) return NQ_ERR_NULL;
+    return hip_status(nq::stream_copy(dst, src, bytes, (hipStream_t)stream));
+}
+
+}  // extern "C"

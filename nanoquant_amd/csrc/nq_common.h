@@ -1,0 +1,88 @@
+// Shared device helpers for the gfx950 binary low-rank kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace nq {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf162_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf168_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+constexpr int kWave = 64;
+constexpr uint32_t kSignPair = 0x80008000u;
+
+// Element traits.  DT = 0: IEEE fp16, DT = 1: bfloat16.  Values travel as raw 16-bit patterns so
+// that the sign can be flipped with integer logic, as the packed "half2" word order intends.
+template <int DT>
+struct Elem;
+
+template <>
+struct Elem<0> {
+    static constexpr uint32_t kOnePair = 0x3C003C00u;  // (1.0h, 1.0h)
+    static constexpr uint32_t kOne = 0x3C00u;
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b), c, false);
+    }
+    static __device__ __forceinline__ float to_float(uint16_t v) {
+        return (float)__builtin_bit_cast(_Float16, v);
+    }
+    static __device__ __forceinline__ uint16_t from_float(float f) {
+        return __builtin_bit_cast(uint16_t, (_Float16)f);
+    }
+    // Final store of the decode path: clamp as the reference does (kernel/cuda/cuda_utils.cuh:83-86).
+    static __device__ __forceinline__ uint16_t from_float_clamped(float f) {
+        return from_float(fminf(fmaxf(f, -64504.0f), 64504.0f));
+    }
+    // Final store of the prefill path: saturate to the largest finite fp16.
+    static __device__ __forceinline__ uint16_t from_float_sat(float f) {
+        return from_float(fminf(fmaxf(f, -65504.0f), 65504.0f));
+    }
+};
+
+template <>
+struct Elem<1> {
+    static constexpr uint32_t kOnePair = 0x3F803F80u;  // (1.0bf, 1.0bf)
+    static constexpr uint32_t kOne = 0x3F80u;
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf162_t, a), __builtin_bit_cast(bf162_t, b), c,
+                                               false);
+    }
+    static __device__ __forceinline__ float to_float(uint16_t v) {
+        return __builtin_bit_cast(float, (uint32_t)v << 16);
+    }
+    static __device__ __forceinline__ uint16_t from_float(float f) {
+        return __builtin_bit_cast(uint16_t, (__bf16)f);
+    }
+    static __device__ __forceinline__ uint16_t from_float_clamped(float f) {
+        return from_float(fminf(fmaxf(f, -3.3895313892515355e+38f), 3.3895313892515355e+38f));
+    }
+    static __device__ __forceinline__ uint16_t from_float_sat(float f) { return from_float_clamped(f); }
+};
+
+// ---- cross-lane sums on a 64-wide wavefront -------------------------------------------------
+// DPP control words (gfx9 encoding): quad_perm = 4 x 2-bit selects; 0x140 row_mirror;
+// 0x141 row_half_mirror.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false);
+    return v + __builtin_bit_cast(float, moved);
+}
+
+// Sum over aligned groups of `group` consecutive lanes (group = 1,2,4,...,64; wave-uniform).  Every
+// lane of a group ends up with the group's total.  Steps inside a 16-lane row are DPP moves; the
+// two cross-row steps go through the LDS crossbar (ds_bpermute), no LDS memory involved.
+__device__ __forceinline__ float group_sum(float v, int group) {
+    if (group >= 2) v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+    if (group >= 4) v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+    if (group >= 8) v = dpp_add<0x141>(v);  // row_half_mirror: lane i <-> 7-i within 8
+    if (group >= 16) v = dpp_add<0x140>(v); // row_mirror: lane i <-> 15-i within 16
+    if (group >= 32) v += __shfl_xor(v, 16, kWave);
+    if (group >= 64) v += __shfl_xor(v, 32, kWave);
+    return v;
+}
+
+}  // namespace nq

@@ -1,0 +1,273 @@
+"""Quantized-linear module interface of the reference, inference side.
+
+`NanoQuantLinear` keeps the attribute names and call protocol of
+src/nanoquant/modules/linear.py (forward :106-150, _prepare_kernel :152-204, _compute_forward
+:248-257, pack_weights/state_dict :288-321): dense +-1 factors `V` [rank, in] and `U` [out, rank]
+with scales `scale_pre` [1, in], `scale_mid` [1, rank] (optional) and `scale_post` [1, out]; after
+`_prepare_kernel(kernel_type, dtype)` the dense factors are replaced by packed words and `forward`
+calls the `torch.ops.binary_kernels` operator.  The quantizer-side parts (latent weights, STE,
+finalize) are not part of this package.
+
+`MixtureOfRankLinear` sums several such terms (the sub-1-bit mixture-of-rank layout); the reference
+describes it but ships no code for it, so its definition here is the sum of single-term layers.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import ops
+from .packing import (binary_packer, binary_unpacker, marlin_nanoquant_packer, repack_words)
+
+
+def _sign_pm1(x: torch.Tensor) -> torch.Tensor:
+    y = x.sign()
+    y[y == 0] = 1
+    return y
+
+
+class NanoQuantLinear(nn.Module):
+    def __init__(self, in_features: int, out_features: int, rank: int, bias: bool = False,
+                 has_scale_mid: bool = True, device=None, dtype: torch.dtype = torch.bfloat16):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.rank = rank
+        self.do_train = False
+        self._binarized = True
+        self.dtype = dtype
+        self.register_parameter("weight", None)
+        if bias:
+            self.bias = nn.Parameter(torch.zeros(out_features, device=device, dtype=dtype), requires_grad=False)
+        else:
+            self.register_parameter("bias", None)
+        self._alloc(has_scale_mid, device)
+
+    # ---- construction ------------------------------------------------------------------------
+    def _alloc(self, has_scale_mid: bool, device) -> None:
+        def p(*shape):
+            return nn.Parameter(torch.empty(*shape, device=device, dtype=self.dtype), requires_grad=False)
+
+        self.scale_pre = p(1, self.in_features)
+        self.scale_post = p(1, self.out_features)
+        self.V = p(self.rank, self.in_features)
+        self.U = p(self.out_features, self.rank)
+        if has_scale_mid:
+            self.scale_mid = p(1, self.rank)
+
+    def init_for_inference(self, rank: int, has_scale_mid: bool = False) -> None:
+        """Re-shape the module for a given rank (reference: linear.py:86-99)."""
+        self.rank = rank
+        self.do_train = False
+        self._binarized = True
+        self.dtype = torch.bfloat16
+        device = self.bias.device if self.bias is not None else None
+        if hasattr(self, "scale_mid"):
+            delattr(self, "scale_mid")
+        self._alloc(has_scale_mid, device)
+
+    @classmethod
+    def from_factors(cls, V: torch.Tensor, U: torch.Tensor, scale_pre: torch.Tensor,
+                     scale_mid: Optional[torch.Tensor], scale_post: torch.Tensor,
+                     bias: Optional[torch.Tensor] = None, dtype: torch.dtype = torch.bfloat16) -> "NanoQuantLinear":
+        """V [rank, in] and U [out, rank] hold +-1 (any dtype); scales are 1-D or [1, D]."""
+        rank, in_f = V.shape
+        out_f = U.shape[0]
+        mod = cls(in_f, out_f, rank, bias=bias is not None, has_scale_mid=scale_mid is not None,
+                  device=V.device, dtype=dtype)
+        with torch.no_grad():
+            mod.V.copy_(_sign_pm1(V.float()))
+            mod.U.copy_(_sign_pm1(U.float()))
+            mod.scale_pre.copy_(scale_pre.reshape(1, -1))
+            mod.scale_post.copy_(scale_post.reshape(1, -1))
+            if scale_mid is not None:
+                mod.scale_mid.copy_(scale_mid.reshape(1, -1))
+            if bias is not None:
+                mod.bias.copy_(bias)
+        return mod
+
+    # ---- forward -----------------------------------------------------------------------------
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if getattr(self, "do_kernel_inference", False):
+            orig_dtype = x.dtype
+            if x.dtype != self.dtype:
+                x = x.to(self.dtype)
+            original_shape = None
+            if x.ndim == 3:
+                original_shape = x.shape
+                x = x.contiguous().view(-1, x.size(-1))
+            elif x.ndim == 2:
+                x = x.contiguous()
+            else:
+                raise ValueError(f"Expected 2D or 3D input tensor, got {x.ndim}D")
+
+            if self.kernel_type == "gemv":
+                y = self.kernel_forward(x, self.scale_pre, self.V_int8, self.scale_mid, self.U_int8,
+                                        self.scale_post, **self.kernel_kwargs)
+            elif self.kernel_type == "gemm":
+                y = self.kernel_forward(x, self.V_int8, self.U_int8, self.s1, self.s2, self.s3, self.workspace)
+            else:
+                raise ValueError(f"Unknown kernel_type: {self.kernel_type}")
+            if original_shape is not None:
+                y = y.view(original_shape[0], original_shape[1], -1)
+            # As in the reference (linear.py:121-141), the kernel paths do not add the bias.
+            return y.to(orig_dtype) if y.dtype != orig_dtype else y
+
+        s_mid = getattr(self, "scale_mid", None)
+        y = self._compute_forward(x, self.V, self.U, self.scale_pre, s_mid, self.scale_post)
+        if self.bias is not None:
+            y += self.bias
+        return y
+
+    def _compute_forward(self, x, V, U, scale_pre, scale_mid, scale_post):
+        """Dense definition of the layer (reference: linear.py:248-257)."""
+        y = F.linear(x * scale_pre, V)
+        if scale_mid is not None:
+            y = y * scale_mid
+        y = F.linear(y, U)
+        return y * scale_post
+
+    # ---- kernel preparation --------------------------------------------------------------------
+    def _prepare_kernel(self, kernel_type: str = "gemv", dtype: torch.dtype = torch.float16) -> None:
+        if kernel_type == "gemlite":
+            raise NotImplementedError("the GemLite/Triton backend is not part of the gfx950 implementation")
+        if kernel_type not in ("gemv", "gemm"):
+            raise ValueError("kernel_type must be one of ['gemv', 'gemm', 'gemlite'].")
+        self.do_kernel_inference = True
+        self.kernel_type = kernel_type
+        self.dtype = dtype
+
+        self.scale_pre = nn.Parameter(self.scale_pre.to(dtype).squeeze(0), requires_grad=False)
+        self.scale_post = nn.Parameter(self.scale_post.to(dtype).squeeze(0), requires_grad=False)
+        self.scale_mid = getattr(self, "scale_mid", None)
+        if self.scale_mid is not None:
+            self.scale_mid = nn.Parameter(self.scale_mid.to(dtype).squeeze(0), requires_grad=False)
+
+        if kernel_type == "gemv":
+            self.U_int8 = binary_packer(self.U.to(torch.int8), method="half2")
+            self.V_int8 = binary_packer(self.V.to(torch.int8), method="half2")
+            delattr(self, "U")
+            delattr(self, "V")
+            self.kernel_forward = ops.get_kernel_function("nanoquant", dtype, kernel_type="dynamic")
+            # Tuning hints of the CUDA kernels, passed through unchanged (linear.py:176-185); the
+            # gfx950 op validates and ignores them.
+            self.kernel_kwargs = {
+                "num_thread_stage1": 128, "num_thread_stage2": 128,
+                "num_row_per_warp_stage1": 2, "num_row_per_warp_stage2": 2,
+                "num_acc_stage1": 1, "num_acc_stage2": 1,
+                "num_pipeline_stage1": 8, "num_pipeline_stage2": 8,
+            }
+        else:
+            if self.scale_mid is None:
+                self.scale_mid = nn.Parameter(torch.ones(self.rank, device=self.scale_pre.device, dtype=dtype),
+                                              requires_grad=False)
+            (self.V_int8, self.U_int8, self.s1, self.s2, self.s3, self.workspace) = marlin_nanoquant_packer(
+                self.V.to(torch.int8).T, self.U.to(torch.int8).T, self.scale_pre.data, self.scale_mid.data,
+                self.scale_post.data)
+            for key in ["U", "V", "scale_pre", "scale_mid", "scale_post"]:
+                delattr(self, key)
+            self.kernel_forward = torch.ops.binary_kernels.marlin_nanoquant_forward
+
+    # ---- packed checkpoint format ----------------------------------------------------------------
+    def pack_weights(self) -> dict:
+        """{V,U}_packed int32 `lsb_first` words + {V,U}_shape (reference: linear.py:288-305)."""
+        packed = {}
+        for name in ("V", "U"):
+            param = getattr(self, name, None)
+            if param is None:
+                continue
+            packed[f"{name}_packed"] = binary_packer(_sign_pm1(param.data.float()).to(torch.int8))
+            packed[f"{name}_shape"] = torch.tensor(param.shape, dtype=torch.long)
+        return packed
+
+    def state_dict(self, *args, **kwargs):
+        state = super().state_dict(*args, **kwargs)
+        prefix = kwargs.get("prefix", "")
+        for k in [k for k in state.keys() if k in (prefix + "V", prefix + "U")]:
+            del state[k]
+        for k, v in self.pack_weights().items():
+            state[prefix + k] = v
+        return state
+
+    def load_packed(self, state: dict, prefix: str = "", kernel_type: str = "gemv",
+                    dtype: torch.dtype = torch.float16) -> None:
+        """Load a packed checkpoint entry.  For the decode path the `lsb_first` words are permuted to the
+        kernel's `half2` order word by word -- the dense +-1 matrices of the reference's loader
+        (src/nanoquant/utils/load_utils.py:269-293) are never materialised."""
+        dev = self.scale_pre.device
+        v_shape = tuple(int(v) for v in state[prefix + "V_shape"])
+        u_shape = tuple(int(v) for v in state[prefix + "U_shape"])
+        self.rank = v_shape[0]
+        for name in ("scale_pre", "scale_post", "scale_mid"):
+            key = prefix + name
+            if key in state:
+                setattr(self, name, nn.Parameter(state[key].to(dev, self.dtype).reshape(1, -1), requires_grad=False))
+            elif name == "scale_mid" and hasattr(self, "scale_mid"):
+                delattr(self, "scale_mid")
+        v_words = state[prefix + "V_packed"].to(dev)
+        u_words = state[prefix + "U_packed"].to(dev)
+        if kernel_type == "gemv":
+            for name in ("V", "U"):
+                if hasattr(self, name):
+                    delattr(self, name)
+            self._prepare_scales_only(dtype)
+            self.V_int8 = repack_words(v_words, "lsb_first", "half2")
+            self.U_int8 = repack_words(u_words, "lsb_first", "half2")
+        else:
+            self.V = nn.Parameter(binary_unpacker(v_words, v_shape).to(self.dtype), requires_grad=False)
+            self.U = nn.Parameter(binary_unpacker(u_words, u_shape).to(self.dtype), requires_grad=False)
+            self._prepare_kernel(kernel_type, dtype)
+
+    def _prepare_scales_only(self, dtype: torch.dtype) -> None:
+        self.do_kernel_inference = True
+        self.kernel_type = "gemv"
+        self.dtype = dtype
+        self.scale_pre = nn.Parameter(self.scale_pre.to(dtype).squeeze(0), requires_grad=False)
+        self.scale_post = nn.Parameter(self.scale_post.to(dtype).squeeze(0), requires_grad=False)
+        self.scale_mid = getattr(self, "scale_mid", None)
+        if self.scale_mid is not None:
+            self.scale_mid = nn.Parameter(self.scale_mid.to(dtype).squeeze(0), requires_grad=False)
+        self.kernel_forward = ops.get_kernel_function("nanoquant", dtype, kernel_type="dynamic")
+        self.kernel_kwargs = {
+            "num_thread_stage1": 128, "num_thread_stage2": 128,
+            "num_row_per_warp_stage1": 2, "num_row_per_warp_stage2": 2,
+            "num_acc_stage1": 1, "num_acc_stage2": 1,
+            "num_pipeline_stage1": 8, "num_pipeline_stage2": 8,
+        }
+
+
+class MixtureOfRankLinear(nn.Module):
+    """y = sum_t term_t(x): several binary low-rank terms with their own scale vectors."""
+
+    def __init__(self, terms: Sequence[NanoQuantLinear]):
+        super().__init__()
+        if len(terms) == 0:
+            raise ValueError("at least one term is required")
+        self.terms = nn.ModuleList(terms)
+        self.in_features = terms[0].in_features
+        self.out_features = terms[0].out_features
+        for t in terms:
+            if t.in_features != self.in_features or t.out_features != self.out_features:
+                raise ValueError("all terms must share in_features and out_features")
+        self.kernel_type = None
+
+    def _prepare_kernel(self, kernel_type: str = "gemv", dtype: torch.dtype = torch.float16) -> None:
+        for t in self.terms:
+            t._prepare_kernel(kernel_type, dtype)
+        self.kernel_type = kernel_type
+        self.dtype = dtype
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.kernel_type == "gemv":
+            orig_dtype = x.dtype
+            xk = x.to(self.dtype).contiguous()
+            y = ops.gemv_mixture_forward(
+                xk, [(t.scale_pre, t.V_int8, t.scale_mid, t.U_int8, t.scale_post) for t in self.terms])
+            return y.to(orig_dtype) if y.dtype != orig_dtype else y
+        y = self.terms[0](x)
+        for t in self.terms[1:]:
+            y = y + t(x)
+        return y

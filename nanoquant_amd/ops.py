@@ -1,0 +1,336 @@
+"""`torch.ops.binary_kernels.*`: the operator boundary of the reference, served by libnq_gfx950.so.
+
+Schemas are the reference's, character for character (src/nanoquant/kernel/pybind.cpp:83-105).  The
+device implementations are registered under the CUDA dispatch key (ROCm tensors dispatch there) and
+shape-only implementations under Meta, as the reference does (pybind.cpp:108-124), so the ops trace
+under torch.compile(fullgraph=True).  There is no CPU registration and no fallback: without the
+built library, or on CPU tensors, the ops raise.
+
+Argument checks and their messages follow the reference's host wrappers:
+  nanoquant_dyn_forward     src/nanoquant/kernel/cuda/gemv_kernel.cu:308-346, cuda/meta_utils.h:14-38
+  marlin_onebit_forward     src/nanoquant/kernel/cuda/gemm.cpp:36-98
+  marlin_nanoquant_forward  src/nanoquant/kernel/cuda/gemm.cpp:112-122
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+_NS = "binary_kernels"
+
+_SCHEMAS = (
+    "nanoquant_dyn_forward("
+    "Tensor x, Tensor scale_g, Tensor Ubits, Tensor? scale_l, Tensor Vbits, Tensor scale_h, "
+    "int num_thread_stage1=128, int num_thread_stage2=128, int num_row_per_warp_stage1=2, "
+    "int num_row_per_warp_stage2=2, int num_acc_stage1=4, int num_acc_stage2=4, "
+    "int num_pipeline_stage1=2, int num_pipeline_stage2=2) -> Tensor",
+    "marlin_onebit_forward("
+    "Tensor x, "
+    "Tensor weight, "
+    "Tensor? scale_g, Tensor? scale_h, "
+    "Tensor(a!) workspace) -> Tensor",
+    "marlin_nanoquant_forward("
+    "Tensor x, "
+    "Tensor weight_u, Tensor weight_v, "
+    "Tensor? scale_g, Tensor? scale_l, Tensor? scale_h, "
+    "Tensor(a!) workspace) -> Tensor",
+)
+
+MARLIN_MIN_MAX_PAR = 32
+
+# Legal values of the CUDA tuning hints (gemv_kernel.cu:351-354).  They select template instances in
+# the reference; here they are validated and otherwise ignored -- the gfx950 launch shape is derived
+# from the problem.  4 is added to the accumulator set because it is the schema's own default.
+_SWEEPS = {
+    "n_th": (64, 128, 256),
+    "n_rpw": (1, 2, 4, 8),
+    "n_acc": (1, 2, 4),
+    "n_pipe": (1, 2, 4, 8, 16),
+}
+
+
+def _dtype_id(t: torch.Tensor) -> int:
+    if t.dtype == torch.float16:
+        return _lib.NQ_F16
+    if t.dtype == torch.bfloat16:
+        return _lib.NQ_BF16
+    raise RuntimeError("Support only Half or BFloat16")
+
+
+def _check_dev_cont(t: torch.Tensor, name: str, dtype: torch.dtype, what: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if t.dtype != dtype:
+        raise RuntimeError(f"{name} {what}")
+
+
+_FLOAT_WHAT = {torch.float16: "must be float16 tensor", torch.bfloat16: "must be bfloat16 tensor"}
+
+
+def _sweep(name: str, value: int) -> None:
+    legal = _SWEEPS[name.rstrip("12")]
+    if value not in legal:
+        choices = ", ".join(str(v) for v in legal)
+        raise ValueError(f"{name} should be one of [{choices}], but {value} was given")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(dev: torch.device):
+    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+# ---------------------------------------------------------------------------------------------
+# decode op
+# ---------------------------------------------------------------------------------------------
+def _check_gemv_args(x, scale_g, Ubits, scale_l, Vbits, scale_h):
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("Support only Half or BFloat16")
+    what = _FLOAT_WHAT[x.dtype]
+    _check_dev_cont(x, "x", x.dtype, what)
+    _check_dev_cont(scale_g, "scale_g", x.dtype, what)
+    _check_dev_cont(scale_h, "scale_h", x.dtype, what)
+    _check_dev_cont(Ubits, "Ubits", torch.int32, "tensor dtype must be int32")
+    _check_dev_cont(Vbits, "Vbits", torch.int32, "tensor dtype must be int32")
+    if scale_l is not None:
+        _check_dev_cont(scale_l, "(*scale_l)", x.dtype, what)
+        if scale_l.size(0) != Ubits.size(0):
+            raise RuntimeError("scale_l size mismatch")
+    if x.dim() < 1:
+        raise RuntimeError("x must have at least one dimension")
+    n = x.size(-1)
+    r = Ubits.size(0)
+    m = scale_h.size(0)
+    # The reference trusts these and indexes out of bounds otherwise; the launch needs them to hold.
+    if Ubits.dim() != 2 or Vbits.dim() != 2:
+        raise RuntimeError("Ubits and Vbits must be 2-D packed word matrices")
+    if Ubits.size(1) != (n + 31) // 32:
+        raise RuntimeError(f"Ubits has {Ubits.size(1)} words per row, expected {(n + 31) // 32} for {n} input columns")
+    if scale_g.numel() != n:
+        raise RuntimeError("scale_g size mismatch")
+    if Vbits.size(0) != m or Vbits.size(1) != (r + 31) // 32:
+        raise RuntimeError(f"Vbits must be [{m}, {(r + 31) // 32}], got {list(Vbits.shape)}")
+    return n, r, m
+
+
+def nanoquant_dyn_forward(x, scale_g, Ubits, scale_l, Vbits, scale_h,
+                          num_thread_stage1=128, num_thread_stage2=128,
+                          num_row_per_warp_stage1=2, num_row_per_warp_stage2=2,
+                          num_acc_stage1=4, num_acc_stage2=4,
+                          num_pipeline_stage1=2, num_pipeline_stage2=2):
+    """y = scale_h * (Vbits (scale_l * (Ubits (scale_g * x)))): `Ubits` [r, n/32] is the FIRST stage,
+    `Vbits` [m, r/32] the second (the reference's argument names, pybind.cpp:86-90)."""
+    n, r, m = _check_gemv_args(x, scale_g, Ubits, scale_l, Vbits, scale_h)
+    _sweep("n_th1", num_thread_stage1)
+    _sweep("n_rpw1", num_row_per_warp_stage1)
+    _sweep("n_acc1", num_acc_stage1)
+    _sweep("n_pipe1", num_pipeline_stage1)
+    _sweep("n_th2", num_thread_stage2)
+    _sweep("n_rpw2", num_row_per_warp_stage2)
+    _sweep("n_acc2", num_acc_stage2)
+    _sweep("n_pipe2", num_pipeline_stage2)
+    lead = x.shape[:-1]
+    batch = 1
+    for d in lead:
+        batch *= d
+    y = torch.empty((batch, m), dtype=x.dtype, device=x.device)
+    if batch > 0 and m > 0:
+        h = torch.empty((batch, max(r, 1)), dtype=torch.float32, device=x.device)
+        with torch.cuda.device(x.device):
+            _lib.check(_lib.lib().nq_gemv_forward(_ptr(x), _ptr(scale_g), _ptr(Ubits), _ptr(scale_l), _ptr(Vbits),
+                                                  _ptr(scale_h), _ptr(h), _ptr(y), batch, n, r, m, _dtype_id(x),
+                                                  _stream(x.device)))
+    return y.reshape(*lead, m)
+
+
+def _nanoquant_dyn_forward_meta(x, scale_g, Ubits, scale_l, Vbits, scale_h, *hints, **kw):
+    shape = list(x.shape)
+    shape[-1] = scale_h.size(0)
+    return x.new_empty(shape)
+
+
+# ---------------------------------------------------------------------------------------------
+# prefill ops
+# ---------------------------------------------------------------------------------------------
+def _onebit_check(A, B, s_in, s_out, workspace):
+    """marlin_onebit_check_and_alloc (gemm.cpp:36-56): returns (m, n, k)."""
+    prob_m = A.size(0)
+    prob_n = B.size(1) * 2
+    prob_k = A.size(1)
+    if prob_k != B.size(0) * 16:
+        raise RuntimeError("k dimension mismatch")
+    if s_in is not None and s_in.size(0) != prob_k:
+        raise RuntimeError("s_in size mismatch")
+    if s_out is not None and s_out.size(0) != prob_n:
+        raise RuntimeError("s_out size mismatch")
+    if workspace.numel() < prob_n // 128 * MARLIN_MIN_MAX_PAR:
+        raise RuntimeError("workspace too small")
+    return prob_m, prob_n, prob_k
+
+
+def _gemm_dtype(A):
+    if A.dtype == torch.float16:
+        return _lib.NQ_F16
+    if A.dtype == torch.bfloat16:
+        return _lib.NQ_BF16
+    raise RuntimeError("Unsupported dtype: Marlin only supports Half and BFloat16")
+
+
+def _check_gemm_tensor(t, name, dtype=None):
+    if t is None:
+        return
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise RuntimeError(f"{name} must have dtype {dtype}")
+
+
+def _scratch(tokens, k, rows, device):
+    nbytes = int(_lib.lib().nq_gemm_scratch_bytes(tokens, k, rows))
+    if nbytes == 0:
+        return None, 0
+    return torch.empty(nbytes // 4, dtype=torch.float32, device=device), nbytes
+
+
+def marlin_onebit_forward(x, weight, scale_g, scale_h, workspace):
+    """C[m, n] = s_out[n] * sum_k (x[m, k] * s_in[k]) * sgn(weight)[n, k]; weight from marlin_onebit_packer."""
+    dt = _gemm_dtype(x)
+    m, n, k = _onebit_check(x, weight, scale_g, scale_h, workspace)
+    _check_gemm_tensor(x, "x")
+    _check_gemm_tensor(weight, "weight", torch.int32)
+    _check_gemm_tensor(scale_g, "scale_g", x.dtype)
+    _check_gemm_tensor(scale_h, "scale_h", x.dtype)
+    C = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    if m == 0 or n == 0:
+        return C
+    scratch, nbytes = _scratch(m, k, n, x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().nq_gemm_onebit(_ptr(x), _ptr(weight), _ptr(scale_g), _ptr(scale_h), _ptr(C),
+                                             _ptr(scratch), nbytes, m, k, n, dt, _stream(x.device)))
+    return C
+
+
+def _marlin_onebit_meta(x, weight, scale_g, scale_h, workspace):
+    m, n, _ = _onebit_check(x, weight, scale_g, scale_h, workspace)
+    return x.new_empty((m, n))
+
+
+def marlin_nanoquant_forward(x, weight_u, weight_v, scale_g, scale_l, scale_h, workspace):
+    """Two chained one-bit GEMMs (gemm.cpp:112-122): `weight_u` is the FIRST stage [n -> r],
+    `weight_v` the second [r -> m] (the order marlin_nanoquant_packer returns them)."""
+    dt = _gemm_dtype(x)
+    t, r, n = _onebit_check(x, weight_u, scale_g, scale_l, workspace)
+    _check_gemm_tensor(x, "x")
+    _check_gemm_tensor(weight_u, "weight_u", torch.int32)
+    _check_gemm_tensor(weight_v, "weight_v", torch.int32)
+    for name, s in (("scale_g", scale_g), ("scale_l", scale_l), ("scale_h", scale_h)):
+        _check_gemm_tensor(s, name, x.dtype)
+    imm = torch.empty((t, r), dtype=x.dtype, device=x.device)
+    _, m, _ = _onebit_check(imm, weight_v, None, scale_h, workspace)
+    out = torch.empty((t, m), dtype=x.dtype, device=x.device)
+    if t == 0 or m == 0:
+        return out
+    s1, b1 = _scratch(t, n, r, x.device)
+    s2, b2 = _scratch(t, r, m, x.device)
+    scratch, nbytes = (s1, b1) if b1 >= b2 else (s2, b2)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().nq_gemm_nanoquant(_ptr(x), _ptr(weight_u), _ptr(weight_v), _ptr(scale_g), _ptr(scale_l),
+                                                _ptr(scale_h), _ptr(imm), _ptr(out), _ptr(scratch), nbytes,
+                                                t, n, r, m, dt, _stream(x.device)))
+    return out
+
+
+def _marlin_nanoquant_meta(x, weight_u, weight_v, scale_g, scale_l, scale_h, workspace):
+    t, r, _ = _onebit_check(x, weight_u, scale_g, scale_l, workspace)
+    imm = x.new_empty((t, r))
+    _, m, _ = _onebit_check(imm, weight_v, None, scale_h, workspace)
+    return x.new_empty((t, m))
+
+
+# ---------------------------------------------------------------------------------------------
+# extras above the reference's surface (plain functions, not dispatcher ops)
+# ---------------------------------------------------------------------------------------------
+def gemv_mixture_forward(x, terms):
+    """Sum of several binary low-rank terms sharing x.  terms: sequence of
+    (scale_g, Ubits, scale_l | None, Vbits, scale_h) with the operand meaning of nanoquant_dyn_forward."""
+    if len(terms) == 0:
+        raise ValueError("at least one term is required")
+    ranks, m = [], None
+    for (scale_g, Ubits, scale_l, Vbits, scale_h) in terms:
+        n, r, mm = _check_gemv_args(x, scale_g, Ubits, scale_l, Vbits, scale_h)
+        if m is not None and mm != m:
+            raise RuntimeError("all terms must have the same output size")
+        m = mm
+        ranks.append(r)
+    lead = x.shape[:-1]
+    batch = 1
+    for d in lead:
+        batch *= d
+    y = torch.empty((batch, m), dtype=x.dtype, device=x.device)
+    if batch == 0 or m == 0:
+        return y.reshape(*lead, m)
+    nt = len(terms)
+    h = torch.empty((batch, max(max(ranks), 1)), dtype=torch.float32, device=x.device)
+    yacc = torch.empty((batch, m), dtype=torch.float32, device=x.device) if nt > 1 else None
+
+    def ptr_array(idx):
+        arr = (ctypes.c_void_p * nt)()
+        for i, term in enumerate(terms):
+            t = term[idx]
+            arr[i] = None if t is None else t.data_ptr()
+        return arr
+
+    rank_arr = (ctypes.c_int * nt)(*ranks)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().nq_gemv_mixture(_ptr(x), ptr_array(0), ptr_array(1), ptr_array(2), ptr_array(3),
+                                              ptr_array(4), rank_arr, nt, _ptr(h), _ptr(yacc), _ptr(y),
+                                              batch, n, m, _dtype_id(x), _stream(x.device)))
+    return y.reshape(*lead, m)
+
+
+def repack_words_device(packed: torch.Tensor, src: str, dst: str) -> torch.Tensor:
+    for name in (src, dst):
+        if name not in _lib.ORDER_IDS:
+            raise ValueError(f"Unsupported method: '{name}'. Supported methods are 'lsb_first', 'half2'.")
+    packed = packed.contiguous()
+    out = torch.empty_like(packed)
+    with torch.cuda.device(packed.device):
+        _lib.check(_lib.lib().nq_repack_words(_ptr(packed), _ptr(out), packed.numel(), _lib.ORDER_IDS[src],
+                                              _lib.ORDER_IDS[dst], _stream(packed.device)))
+    return out
+
+
+def get_kernel_function(namespace: str, dtype: torch.dtype, kernel_type: str):
+    """Operator lookup with the reference's naming rule (src/nanoquant/kernel/utils.py:33-48)."""
+    mid = "_dyn" if kernel_type != "fixed" else ""
+    op_name = f"{namespace}{mid}_forward"
+    try:
+        return getattr(torch.ops.binary_kernels, op_name)
+    except AttributeError as exc:
+        have = dir(torch.ops.binary_kernels) if hasattr(torch.ops, "binary_kernels") else []
+        raise AttributeError(f"Dispatcher op `{namespace}::{op_name}` not found. "
+                             f"Available in torch.ops.binary_kernels: {have}") from exc
+
+
+# ---------------------------------------------------------------------------------------------
+# registration
+# ---------------------------------------------------------------------------------------------
+_library = torch.library.Library(_NS, "DEF")
+for _schema in _SCHEMAS:
+    _library.define(_schema)
+_library.impl("nanoquant_dyn_forward", nanoquant_dyn_forward, "CUDA")
+_library.impl("marlin_onebit_forward", marlin_onebit_forward, "CUDA")
+_library.impl("marlin_nanoquant_forward", marlin_nanoquant_forward, "CUDA")
+_library.impl("nanoquant_dyn_forward", _nanoquant_dyn_forward_meta, "Meta")
+_library.impl("marlin_onebit_forward", _marlin_onebit_meta, "Meta")
+_library.impl("marlin_nanoquant_forward", _marlin_nanoquant_meta, "Meta")
