@@ -1,0 +1,273 @@
+#!/usr/bin/env python3
+"""Benchmark of the binary low-rank linear layer on one MI355X.
+
+Headline workload (N=1): the decode GEMV over one Llama-2-7B-shaped decoder layer at 1.0 bpw --
+q/k/v/o 4096x4096 (r=2048), gate/up 11008x4096 and down 4096x11008 (r = round(mn/(m+n)) = 2985) --
+batch 1, fp16 activations.  One "step" is one pass over the 7 linears of the layer.  Successive steps
+walk over distinct copies of the layer's weights (more than the 256 MB Infinity Cache in total), so
+the packed words come from HBM, not from cache.  `value` is algorithmic bytes / time.
+
+Prints ONE JSON line.  Extra keys report the same layer at batch 4 and 16 and the 128-token prefill
+GEMM; `roofline` is for the decode kernel, `cpu_baseline` is the reference's dense CPU path (two
+F.linear on unpacked +-1 factors) timed on this host.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+LLAMA2_7B_LAYER = (("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096),
+                   ("gate", 11008, 4096), ("up", 11008, 4096), ("down", 4096, 11008))
+
+
+def nominal_rank(m, n):
+    return int(round(m * n / (m + n)))
+
+
+def gemv_bytes(m, n, r, batch):
+    """Algorithmic bytes of one decode call: packed bits at the nominal rank + fp16 scales + x + y."""
+    return r * (m + n) / 8 + 2 * (n + r + m) + 2 * batch * (n + m)
+
+
+def gemm_flops(m, n, r, tokens):
+    return 2.0 * tokens * r * (m + n)
+
+
+class SynthLinear:
+    """Random packed factors of one linear, resident on the GPU (decode layout)."""
+
+    def __init__(self, torch, dev, m, n, r, gen):
+        self.m, self.n, self.r = m, n, r
+        self.rp = (r + 31) // 32 * 32          # rank padded to whole words; padding has s_mid = 0
+        i32 = torch.iinfo(torch.int32)
+        self.vt_bits = torch.randint(i32.min, i32.max, (self.rp, n // 32), dtype=torch.int32, device=dev, generator=gen)
+        self.u_bits = torch.randint(i32.min, i32.max, (m, self.rp // 32), dtype=torch.int32, device=dev, generator=gen)
+
+        def scale(k):
+            return (torch.randn(k, device=dev, generator=gen).abs() * 0.02 + 1e-3).to(torch.float16)
+
+        self.s_in, self.s_mid, self.s_out = scale(n), scale(self.rp), scale(m)
+        if self.rp > r:
+            self.s_mid[r:] = 0
+
+
+def build_layers(torch, dev, shapes, copies, seed):
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    return [[SynthLinear(torch, dev, m, n, nominal_rank(m, n), gen) for (_, m, n) in shapes] for _ in range(copies)]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=520)
+    ap.add_argument("--warmup", type=int, default=52)
+    ap.add_argument("--copies", type=int, default=26, help="distinct weight copies of the layer (26 x 25.3 MB > 256 MB)")
+    ap.add_argument("--no-extra", action="store_true", help="skip batch 4/16, prefill and CPU legs")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the layer is a single-GPU hot path); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import nanoquant_amd  # noqa: F401
+    from nanoquant_amd import _lib, packing
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    lib = _lib.lib()
+    vp = ctypes.c_void_p
+
+    layers = build_layers(torch, dev, LLAMA2_7B_LAYER, args.copies, seed=0)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1)
+
+    def make_io(batch):
+        xs = [torch.randn(batch, lin.n, device=dev, generator=gen).to(torch.float16) for lin in layers[0]]
+        hs = [torch.empty(batch, lin.rp, dtype=torch.float32, device=dev) for lin in layers[0]]
+        ys = [torch.empty(batch, lin.m, dtype=torch.float16, device=dev) for lin in layers[0]]
+        return xs, hs, ys
+
+    def layer_pass(layer, io, batch, stream):
+        xs, hs, ys = io
+        for lin, x, h, y in zip(layer, xs, hs, ys):
+            st = lib.nq_gemv_forward(vp(x.data_ptr()), vp(lin.s_in.data_ptr()), vp(lin.vt_bits.data_ptr()),
+                                     vp(lin.s_mid.data_ptr()), vp(lin.u_bits.data_ptr()), vp(lin.s_out.data_ptr()),
+                                     vp(h.data_ptr()), vp(y.data_ptr()), batch, lin.n, lin.rp, lin.m, _lib.NQ_F16, stream)
+            if st != 0:
+                raise RuntimeError(_lib.status_message(st))
+
+    def capture_graphs(io, batch):
+        """One HIP graph per weight copy, each holding the launches of one layer pass."""
+        side = torch.cuda.Stream()
+        graphs = []
+        with torch.cuda.stream(side):
+            layer_pass(layers[0], io, batch, vp(side.cuda_stream))  # warm (module load, attributes)
+        side.synchronize()
+        for layer in layers:
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=side):
+                layer_pass(layer, io, batch, vp(torch.cuda.current_stream().cuda_stream))
+            graphs.append(g)
+        return graphs
+
+    def timed(graphs, steps, warmup):
+        for i in range(warmup):
+            graphs[i % len(graphs)].replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(steps):
+            graphs[(warmup + i) % len(graphs)].replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps  # ms per step
+
+    def layer_bytes(batch):
+        return sum(gemv_bytes(lin.m, lin.n, lin.r, batch) for lin in layers[0])
+
+    # ---- headline: batch 1 -------------------------------------------------------------------
+    io1 = make_io(1)
+    graphs1 = capture_graphs(io1, 1)
+    ms = timed(graphs1, args.steps, args.warmup)
+    bytes1 = layer_bytes(1)
+    gbs = bytes1 / (ms * 1e-3) / 1e9
+    launches_per_step = 2 * len(LLAMA2_7B_LAYER)
+    launch_us = ms * 1e3 / launches_per_step
+    result = {
+        "metric": "batch-1 binary GEMV sustained GB/s over one Llama-2-7B decoder layer (1.0 bpw)",
+        "value": round(gbs, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16 operands, f32 accumulate",
+        "data": "synthetic",
+        "config": {
+            "workload": "cfg1: decode GEMV over the 7 linears of one Llama-2-7B decoder layer, batch 1, 1.0 bpw "
+                        "(q/k/v/o 4096x4096 r2048; gate/up 11008x4096, down 4096x11008 r2985 padded to 3008 with "
+                        "zero mid scale); %d rotating weight copies (%.0f MB) so words come from HBM"
+                        % (args.copies, args.copies * sum(lin.r * (lin.m + lin.n) / 8 for lin in layers[0]) / 1e6),
+            "batch": 1,
+            "algorithmic_bytes_per_step": int(bytes1),
+            "launches_per_step": launches_per_step,
+        },
+        "us_per_layer": round(ms * 1e3, 3),
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "gemv_stage_kernel (one launch per stage, 14 per layer)",
+            "achieved": round(bytes1 / launches_per_step / (launch_us * 1e-6) / 1e9, 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(bytes1 / launches_per_step / (launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "bytes_per_launch": int(bytes1 / launches_per_step),
+            "avg_launch_us": round(launch_us, 3),
+        },
+    }
+
+    if not args.no_extra:
+        extra = {}
+        for b in (4, 16):
+            io = make_io(b)
+            graphs = capture_graphs(io, b)
+            msb = timed(graphs, max(args.steps // 4, 26), 26)
+            extra[f"batch{b}"] = {"us_per_layer": round(msb * 1e3, 3),
+                                  "GBps": round(layer_bytes(b) / (msb * 1e-3) / 1e9, 2)}
+            del graphs
+        # ---- 128-token prefill over the same layer shapes ----
+        tokens = 128
+        pre = []
+        g2 = torch.Generator(device=dev)
+        g2.manual_seed(2)
+        for (_, m, n) in LLAMA2_7B_LAYER[3:]:  # o (4096^2), gate, up, down: the three distinct shapes + one repeat
+            r = nominal_rank(m, n)
+            v = (torch.randint(0, 2, (n, r), device=dev, generator=g2, dtype=torch.int8) * 2 - 1)
+            u = (torch.randint(0, 2, (r, m), device=dev, generator=g2, dtype=torch.int8) * 2 - 1)
+            sc = lambda k: (torch.randn(k, device=dev, generator=g2).abs() * 0.02 + 1e-3).to(torch.float16)
+            packed = packing.marlin_nanoquant_packer(v, u, sc(n), sc(r), sc(m))
+            x = torch.randn(tokens, n, device=dev, generator=g2).to(torch.float16)
+            pre.append((m, n, r, x, packed))
+        op = torch.ops.binary_kernels.marlin_nanoquant_forward
+        gemm_lines = {}
+        for (m, n, r, x, packed) in pre:
+            for _ in range(5):
+                op(x, *packed)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            iters = 50
+            e0.record()
+            for _ in range(iters):
+                op(x, *packed)
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / iters
+            tf = gemm_flops(m, n, r, tokens) / (us * 1e-6) / 1e12
+            gemm_lines[f"{m}x{n}_r{r}"] = {"us": round(us, 2), "TFLOPs": round(tf, 2),
+                                           "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+        extra["prefill_128_tokens"] = gemm_lines
+        result["extra"] = extra
+
+        # ---- CPU baseline: the reference's dense path on this host (bounded sample) ----
+        from oracle import nq_oracle as oracle
+
+        torch.set_num_threads(os.cpu_count() or 1)
+        cpu_terms = []
+        gcpu = torch.Generator().manual_seed(3)
+        for (_, m, n) in LLAMA2_7B_LAYER:
+            r = nominal_rank(m, n)
+            vt = (torch.randint(0, 2, (r, n), generator=gcpu) * 2 - 1).float()
+            u = (torch.randint(0, 2, (m, r), generator=gcpu) * 2 - 1).float()
+            sc = lambda k: torch.randn(k, generator=gcpu).abs() * 0.02 + 1e-3
+            cpu_terms.append((torch.randn(1, n, generator=gcpu), vt, u, sc(n), sc(r), sc(m)))
+
+        def cpu_pass():
+            for (x, vt, u, s_in, s_mid, s_out) in cpu_terms:
+                oracle.torch_dense_forward(x, vt, u, s_in, s_mid, s_out)
+
+        for _ in range(3):
+            cpu_pass()
+        times = []
+        t_end = time.perf_counter() + args.cpu_seconds
+        while len(times) < 20 or (time.perf_counter() < t_end and len(times) < 200):
+            t0 = time.perf_counter()
+            cpu_pass()
+            times.append(time.perf_counter() - t0)
+            if time.perf_counter() > t_end + 20:
+                break
+        times.sort()
+        med = times[len(times) // 2]
+        result["cpu_baseline"] = {
+            "value": round(bytes1 / med / 1e9, 3),
+            "unit": "GB/s",
+            "us_per_layer": round(med * 1e6, 1),
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": "same 7-linear layer, batch 1, fp32 dense +-1 factors through two F.linear per linear "
+                      "(the reference's CPU path), median of %d passes; GB/s counts the same algorithmic bytes" % len(times),
+        }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -204,9 +204,11 @@ static hipError_t launch_gemm(const GemmArgs& a, const GemmPlan& p, hipStream_t 
     dim3 grid(p.gx, p.gy, p.ksplit);
     if (p.ksplit > 1) {
         auto kern = gemm_onebit_kernel<DT, TT, true>;
-        if (lds > 64 * 1024) {
+        static bool attr_done = false;
+        if (lds > 64 * 1024 && !attr_done) {
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             if (e != hipSuccess) return e;
+            attr_done = true;
         }
         const size_t n4 = (size_t)a.T * a.R / 4;
         size_t zb = (n4 + 255) / 256;
@@ -217,9 +219,11 @@ static hipError_t launch_gemm(const GemmArgs& a, const GemmPlan& p, hipStream_t 
                            a.s_out, (uint16_t*)a.y, a.R, n4);
     } else {
         auto kern = gemm_onebit_kernel<DT, TT, false>;
-        if (lds > 64 * 1024) {
+        static bool attr_done = false;
+        if (lds > 64 * 1024 && !attr_done) {
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             if (e != hipSuccess) return e;
+            attr_done = true;
         }
         hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);
     }

@@ -109,7 +109,9 @@ def test_all_plus_one_closed_form(dev):
     y = torch.ops.binary_kernels.nanoquant_dyn_forward(f(x), f(s_in), zeros_v, f(s_mid), zeros_u, f(s_out), **HINTS)
     expect = (x.astype(np.float64) * s_in.astype(np.float64)).sum(1, keepdims=True) * s_mid.astype(np.float64).sum() \
         * s_out.astype(np.float64)[None, :]
-    assert oracle.max_rel_err(y.float().cpu().numpy(), expect) < 1e-3
+    # With identical signs nothing averages out: the three 16-bit roundings (x*s_in, h, y) of 2^-11
+    # each add up coherently, so the bound is their sum rather than the random-sign budget of 1e-3.
+    assert oracle.max_rel_err(y.float().cpu().numpy(), expect) < 3 * 2.0**-11 + 1e-4
 
 
 def test_bit_index_exactness_single_minus_one(dev):
