@@ -64,6 +64,48 @@ int nq_gemv_mixture(const void* x, const void* const* s_in, const uint32_t* cons
                     const int* r, int nterms, float* h_scratch, float* y_scratch, void* y,
                     int batch, int n, int m, int dtype, void* stream);
 
+/* Decode path, run-list form: a whole list of linears (a decoder layer, a decoder stack) in ONE
+ * persistent kernel launch.  No counterpart in the reference, which launches two kernels per linear
+ * from Python (modules/linear.py:121-130 -> kernel/cuda/gemv_kernel.cu:406-425); it exists because a
+ * 1-bit linear is worth well under a microsecond of HBM time and launch boundaries would dominate.
+ *
+ * nq_linear describes one linear with the operand meaning of nq_gemv_forward; h is its private fp32
+ * [batch, r] intermediate.  x_from >= 0 says that x is the y of that earlier entry of the list (the
+ * kernel then orders the two); y_from >= 0 says that `addend` is the fp32 y of that earlier entry.
+ * With out_f32 the result y is stored as fp32 (used for sums over terms); addend (fp32 [batch, m])
+ * is added before the store.
+ *
+ * nq_runlist_build writes the stage table into `workspace` (device memory of at least
+ * nq_runlist_workspace_bytes(nlinears) bytes, 256-byte aligned) -- it copies from host memory, so it
+ * synchronises with the host and must not be captured in a graph.  `interleave` >= 1 is how many
+ * first stages of independent linears are placed between a linear's two stages, which hides the
+ * device-wide hand-over of h; linears inside that window need distinct h buffers.
+ * nq_runlist_run enqueues the single launch; it allocates nothing and can be graph-captured.  Runs of
+ * the same workspace must not overlap in time.  batch must be 1, 2, 4, 8 or 16.
+ * nq_runlist_status copies the error word back (synchronises): 0 ok, 1 = a bounded dependency wait
+ * expired (the results of that run are invalid; call nq_runlist_build again before reuse). */
+typedef struct nq_linear {
+    const void* x;
+    const void* s_in;
+    const uint32_t* vt_bits;
+    const void* s_mid;      /* may be NULL */
+    const uint32_t* u_bits;
+    const void* s_out;
+    float* h;
+    void* y;
+    const float* addend;    /* may be NULL */
+    int n, r, m;
+    int x_from;             /* -1: x is an external input */
+    int y_from;             /* -1: addend (if any) is an external input */
+    int out_f32;
+} nq_linear;
+
+size_t nq_runlist_workspace_bytes(int nlinears);
+int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtype, int interleave,
+                     void* workspace, size_t workspace_bytes, void* stream);
+int nq_runlist_run(const void* workspace, int nlinears, int batch, int dtype, void* stream);
+int nq_runlist_status(const void* workspace, int* status_out, void* stream);
+
 /* One matmul-free stage: out[b,row] = s_row[row] * sum_c sgn(bits[row,c]) * in[b,c] * s_col[c].
  * Replaces nanoquant_stage1_dyn_kernel / nanoquant_stage2_dyn_kernel launches
  * (kernel/cuda/gemv_kernel.cu:283-301).  in/out are `dtype`; s_col, s_row may be NULL. */

@@ -8,9 +8,10 @@ from .packing import (binary_packer, binary_unpacker, marlin_nanoquant_packer, m
                       pack_binary_gemv, pack_binary_marlin, pack_binary_marlin_fused, repack_words,
                       unpack_binary_gemv)
 from .ops import get_kernel_function
+from .runlist import DecodeRunList
 
 __all__ = [
     "NanoQuantLinear", "MixtureOfRankLinear", "binary_packer", "binary_unpacker", "marlin_nanoquant_packer",
     "marlin_onebit_packer", "pack_binary_gemv", "unpack_binary_gemv", "pack_binary_marlin",
-    "pack_binary_marlin_fused", "repack_words", "get_kernel_function",
+    "pack_binary_marlin_fused", "repack_words", "get_kernel_function", "DecodeRunList",
 ]

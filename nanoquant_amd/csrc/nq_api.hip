@@ -3,6 +3,8 @@
 #include "../../include/nq_gfx950.h"
 #include "nq_kernels.h"
 
+#include <vector>
+
 namespace {
 thread_local int g_last_hip_error = 0;
 
@@ -104,6 +106,121 @@ int nq_gemv_stage(const void* in, const void* s_col, const uint32_t* bits, const
     if (!in || !bits || !out) return NQ_ERR_NULL;
     return hip_status(nq::gemv_stage(dtype, true, bits, in, s_col, s_row, nullptr, out, false, batch, rows,
                                      words_of(cols), cols, cols, rows, (hipStream_t)stream));
+}
+
+// ---- run list ---------------------------------------------------------------------------------
+// workspace layout: [0,256): status word; [256, 256 + 4*(2n+1) rounded to 256): counters (one per
+// stage + the exit counter); then 2n RunStage records.
+static size_t runlist_counter_bytes(int n) { return ((size_t)(2 * n + 1) * 4 + 255) / 256 * 256; }
+
+size_t nq_runlist_workspace_bytes(int nlinears) {
+    if (nlinears <= 0) return 0;
+    return 256 + runlist_counter_bytes(nlinears) + (size_t)2 * nlinears * sizeof(nq::RunStage);
+}
+
+static inline bool al16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtype, int interleave,
+                     void* workspace, size_t workspace_bytes, void* stream) {
+    if (dtype != NQ_F16 && dtype != NQ_BF16) return NQ_ERR_DTYPE;
+    if (nlinears <= 0 || interleave < 1) return NQ_ERR_SHAPE;
+    if (batch != 1 && batch != 2 && batch != 4 && batch != 8 && batch != 16) return NQ_ERR_SHAPE;
+    if (!linears || !workspace) return NQ_ERR_NULL;
+    if (((uintptr_t)workspace & 255u) != 0) return NQ_ERR_ALIGN;
+    if (workspace_bytes < nq_runlist_workspace_bytes(nlinears)) return NQ_ERR_WORKSPACE;
+    for (int i = 0; i < nlinears; ++i) {
+        const nq_linear& l = linears[i];
+        if (l.n <= 0 || l.r <= 0 || l.m <= 0) return NQ_ERR_SHAPE;
+        if (!l.x || !l.s_in || !l.vt_bits || !l.u_bits || !l.s_out || !l.h || !l.y) return NQ_ERR_NULL;
+        if (l.x_from >= i || l.y_from >= i) return NQ_ERR_SHAPE;
+    }
+    // Order of stages: first stages run ahead of second stages by up to `interleave` linears, unless a
+    // dependency (or a shared h buffer) forces a second stage out earlier.
+    std::vector<nq::RunStage> table;
+    std::vector<int> first_idx(nlinears, -1), second_idx(nlinears, -1);
+    std::vector<int> pending;
+    auto emit_second = [&](int i) {
+        const nq_linear& l = linears[i];
+        nq::RunStage st{};
+        st.bits = l.u_bits; st.in = l.h; st.s_col = nullptr; st.s_row = (const uint16_t*)l.s_out;
+        st.out = l.y; st.addend = l.addend;
+        st.rows = l.m; st.K = l.r; st.words = (l.r + 31) / 32; st.units = (st.words + 3) / 4;
+        st.in_stride = l.r; st.out_stride = l.m; st.in_f32 = 1; st.out_f32 = l.out_f32 ? 1 : 0;
+        st.dep = first_idx[i];
+        st.dep2 = (l.addend && l.y_from >= 0) ? second_idx[l.y_from] : -1;
+        st.signal = 0;
+        st.vec_bits = (st.words % 4 == 0) && al16(l.u_bits);
+        st.vec_in = al16(l.h) && ((size_t)l.r * 4) % 16 == 0;
+        second_idx[i] = (int)table.size();
+        table.push_back(st);
+    };
+    auto flush_until = [&](int upto_linear) {   // emit pending second stages in order up to `upto_linear`
+        while (!pending.empty()) {
+            const int i = pending.front();
+            emit_second(i);
+            pending.erase(pending.begin());
+            if (i == upto_linear) break;
+        }
+    };
+    for (int i = 0; i < nlinears; ++i) {
+        const nq_linear& l = linears[i];
+        int need = -1;
+        for (int j : pending) {
+            if (j == l.x_from || j == l.y_from || linears[j].h == l.h) need = j;
+        }
+        if (need >= 0) flush_until(need);
+        nq::RunStage st{};
+        st.bits = l.vt_bits; st.in = l.x; st.s_col = (const uint16_t*)l.s_in; st.s_row = (const uint16_t*)l.s_mid;
+        st.out = l.h; st.addend = nullptr;
+        st.rows = l.r; st.K = l.n; st.words = (l.n + 31) / 32; st.units = (st.words + 3) / 4;
+        st.in_stride = l.n; st.out_stride = l.r; st.in_f32 = 0; st.out_f32 = 1;
+        st.dep = l.x_from >= 0 ? second_idx[l.x_from] : -1;
+        st.dep2 = -1;
+        st.signal = 1;
+        st.vec_bits = (st.words % 4 == 0) && al16(l.vt_bits);
+        st.vec_in = al16(l.x) && ((size_t)l.n * 2) % 16 == 0 && al16(l.s_in);
+        first_idx[i] = (int)table.size();
+        table.push_back(st);
+        pending.push_back(i);
+        if ((int)pending.size() >= interleave) flush_until(pending.front());
+    }
+    flush_until(-1);
+    for (auto& st : table) {
+        if (st.dep >= 0) table[st.dep].signal = 1;
+        if (st.dep2 >= 0) table[st.dep2].signal = 1;
+    }
+    hipStream_t hs = (hipStream_t)stream;
+    char* base = (char*)workspace;
+    hipError_t e = hipMemsetAsync(base, 0, 256 + runlist_counter_bytes(nlinears), hs);
+    if (e != hipSuccess) return hip_status(e);
+    e = hipMemcpyAsync(base + 256 + runlist_counter_bytes(nlinears), table.data(), table.size() * sizeof(nq::RunStage),
+                       hipMemcpyHostToDevice, hs);
+    if (e != hipSuccess) return hip_status(e);
+    return hip_status(hipStreamSynchronize(hs));   // `table` is host stack memory: finish before it dies
+}
+
+int nq_runlist_run(const void* workspace, int nlinears, int batch, int dtype, void* stream) {
+    if (dtype != NQ_F16 && dtype != NQ_BF16) return NQ_ERR_DTYPE;
+    if (nlinears <= 0) return NQ_ERR_SHAPE;
+    if (batch != 1 && batch != 2 && batch != 4 && batch != 8 && batch != 16) return NQ_ERR_SHAPE;
+    if (!workspace) return NQ_ERR_NULL;
+    static int nwg = 0;
+    if (nwg == 0) nwg = nq::stream_max_workgroups();
+    if (nwg <= 0) return NQ_ERR_HIP;
+    char* base = (char*)workspace;
+    return hip_status(nq::gemv_stream(dtype, batch, (const nq::RunStage*)(base + 256 + runlist_counter_bytes(nlinears)),
+                                      2 * nlinears, (unsigned*)(base + 256), (unsigned*)base, nwg,
+                                      (hipStream_t)stream));
+}
+
+int nq_runlist_status(const void* workspace, int* status_out, void* stream) {
+    if (!workspace || !status_out) return NQ_ERR_NULL;
+    unsigned v = 0;
+    hipError_t e = hipMemcpyAsync(&v, workspace, sizeof(v), hipMemcpyDeviceToHost, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_status(e);
+    e = hipStreamSynchronize((hipStream_t)stream);
+    *status_out = (int)v;
+    return hip_status(e);
 }
 
 size_t nq_gemm_scratch_bytes(int tokens, int k, int rows) { return nq::gemm_scratch_bytes(tokens, k, rows); }

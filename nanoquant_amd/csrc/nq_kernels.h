@@ -12,6 +12,26 @@ hipError_t gemv_stage(int dtype, bool first, const uint32_t* bits, const void* i
                       const void* s_row, const float* addend, void* out, bool out_f32, int batch, int rows,
                       int words, int K, int in_stride, int out_stride, hipStream_t stream);
 
+// nq_stream.hip: one persistent launch over a table of stages (see the file header).
+struct RunStage {
+    const uint32_t* bits;   // [rows, words] packed signs, row-major "half2" order
+    const void* in;         // [batch, in_stride]: 16-bit activations, or fp32 when in_f32
+    const uint16_t* s_col;  // [K] per-column scale applied to a 16-bit input, may be null
+    const uint16_t* s_row;  // [rows] per-row scale, may be null
+    void* out;              // [batch, out_stride]: fp32 when out_f32, else 16-bit (clamped)
+    const float* addend;    // fp32 [batch, out_stride] added before the store, may be null
+    int rows, words, K, units;
+    int in_stride, out_stride;
+    int in_f32, out_f32;
+    int dep, dep2;          // stage indices that must be complete before `in` / `addend` are read, or -1
+    int signal;             // a later stage waits on this one
+    int vec_bits, vec_in;
+    int pad_;
+};
+int stream_max_workgroups();
+hipError_t gemv_stream(int dtype, int batch, const RunStage* stages, int nstages, unsigned* counters,
+                       unsigned* status, int nwg, hipStream_t stream);
+
 // nq_gemm.hip: C[T,R] = s_out * ((x * s_in) . sgn(W)^T) with W in the 32x256 tile layout.
 // scratch: fp32 [T,R] when gemm_scratch_bytes(T,K,R) > 0.
 size_t gemm_scratch_bytes(int T, int K, int R);

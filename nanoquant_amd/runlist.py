@@ -1,0 +1,117 @@
+"""Host side of the run-list decode path: many linears, one persistent kernel launch.
+
+`DecodeRunList` owns the device workspace (stage table + completion counters) and the fp32
+intermediates of a list of linears; `run()` enqueues the single launch on the current stream and can
+be captured in a HIP graph.  The reference has no such object: its decode path is one Python op call,
+two allocations and two launches per linear (src/nanoquant/modules/linear.py:121-130,
+src/nanoquant/kernel/cuda/gemv_kernel.cu:340-425).
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import _lib
+
+
+class NqLinear(ctypes.Structure):
+    """Mirror of `nq_linear` in include/nq_gfx950.h."""
+    _fields_ = [
+        ("x", ctypes.c_void_p), ("s_in", ctypes.c_void_p), ("vt_bits", ctypes.c_void_p), ("s_mid", ctypes.c_void_p),
+        ("u_bits", ctypes.c_void_p), ("s_out", ctypes.c_void_p), ("h", ctypes.c_void_p), ("y", ctypes.c_void_p),
+        ("addend", ctypes.c_void_p),
+        ("n", ctypes.c_int), ("r", ctypes.c_int), ("m", ctypes.c_int),
+        ("x_from", ctypes.c_int), ("y_from", ctypes.c_int), ("out_f32", ctypes.c_int),
+    ]
+
+
+class DecodeRunList:
+    BATCHES = (1, 2, 4, 8, 16)
+
+    def __init__(self, batch: int, dtype: torch.dtype = torch.float16, device=None, interleave: int = 2):
+        if batch not in self.BATCHES:
+            raise ValueError(f"run-list batch must be one of {self.BATCHES}, got {batch}")
+        if dtype not in (torch.float16, torch.bfloat16):
+            raise RuntimeError("Support only Half or BFloat16")
+        self.batch = batch
+        self.dtype = dtype
+        self.device = torch.device(device if device is not None else "cuda")
+        self.interleave = interleave
+        self._entries: List[dict] = []
+        self._keep: list = []          # tensors referenced by raw pointers stay alive here
+        self._workspace: Optional[torch.Tensor] = None
+
+    # ---- building -----------------------------------------------------------------------------
+    def add(self, x: torch.Tensor, scale_pre: torch.Tensor, V_int8: torch.Tensor, scale_mid: Optional[torch.Tensor],
+            U_int8: torch.Tensor, scale_post: torch.Tensor, y: Optional[torch.Tensor] = None,
+            x_from: int = -1, addend: Optional[torch.Tensor] = None, y_from: int = -1,
+            out_f32: bool = False) -> int:
+        """Append one linear (operands as `NanoQuantLinear` holds them after `_prepare_kernel('gemv')`:
+        V_int8 [r, n/32] first stage, U_int8 [m, r/32] second stage).  Returns its index; `y` is
+        allocated when not given and is available as `outputs[index]`."""
+        n = x.shape[-1]
+        r, m = V_int8.shape[0], U_int8.shape[0]
+        for name, t, dt in (("x", x, self.dtype), ("scale_pre", scale_pre, self.dtype), ("scale_post", scale_post, self.dtype),
+                            ("V_int8", V_int8, torch.int32), ("U_int8", U_int8, torch.int32)):
+            if not t.is_cuda or not t.is_contiguous() or t.dtype != dt:
+                raise RuntimeError(f"{name} must be a contiguous {dt} tensor on the GPU")
+        if x.numel() != self.batch * n:
+            raise RuntimeError(f"x must hold {self.batch} rows of {n}")
+        if V_int8.shape[1] != (n + 31) // 32 or U_int8.shape[1] != (r + 31) // 32:
+            raise RuntimeError("packed factor shapes do not match x / each other")
+        if scale_pre.numel() != n or scale_post.numel() != m or (scale_mid is not None and scale_mid.numel() != r):
+            raise RuntimeError("scale size mismatch")
+        if y is None:
+            y = torch.empty((self.batch, m), dtype=torch.float32 if out_f32 else self.dtype, device=self.device)
+        h = torch.empty((self.batch, r), dtype=torch.float32, device=self.device)
+        self._keep += [x, scale_pre, V_int8, scale_mid, U_int8, scale_post, y, h, addend]
+        self._entries.append(dict(x=x, s_in=scale_pre, vt=V_int8, s_mid=scale_mid, u=U_int8, s_out=scale_post, h=h, y=y,
+                                  addend=addend, n=n, r=r, m=m, x_from=x_from, y_from=y_from, out_f32=int(out_f32)))
+        self._workspace = None
+        return len(self._entries) - 1
+
+    @property
+    def outputs(self) -> Sequence[torch.Tensor]:
+        return [e["y"] for e in self._entries]
+
+    def build(self) -> None:
+        n = len(self._entries)
+        if n == 0:
+            raise ValueError("empty run list")
+        arr = (NqLinear * n)()
+        p = lambda t: None if t is None else t.data_ptr()
+        for i, e in enumerate(self._entries):
+            arr[i] = NqLinear(p(e["x"]), p(e["s_in"]), p(e["vt"]), p(e["s_mid"]), p(e["u"]), p(e["s_out"]), p(e["h"]),
+                              p(e["y"]), p(e["addend"]), e["n"], e["r"], e["m"], e["x_from"], e["y_from"], e["out_f32"])
+        lib = _lib.lib()
+        nbytes = int(lib.nq_runlist_workspace_bytes(n))
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+        with torch.cuda.device(self.device):
+            stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+            _lib.check(lib.nq_runlist_build(arr, n, self.batch, self._dtype_id(), self.interleave,
+                                            ctypes.c_void_p(ws.data_ptr()), nbytes, stream))
+        self._workspace = ws
+
+    def _dtype_id(self) -> int:
+        return _lib.NQ_F16 if self.dtype == torch.float16 else _lib.NQ_BF16
+
+    # ---- running --------------------------------------------------------------------------------
+    def run(self) -> Sequence[torch.Tensor]:
+        """Enqueue the launch on the current stream (no allocation, no synchronisation)."""
+        if self._workspace is None:
+            self.build()
+        with torch.cuda.device(self.device):
+            stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+            _lib.check(_lib.lib().nq_runlist_run(ctypes.c_void_p(self._workspace.data_ptr()), len(self._entries),
+                                                 self.batch, self._dtype_id(), stream))
+        return self.outputs
+
+    def status(self) -> int:
+        """Synchronises.  0 = ok; 1 = a dependency wait ran into its bound (results invalid)."""
+        out = ctypes.c_int(0)
+        with torch.cuda.device(self.device):
+            stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+            _lib.check(_lib.lib().nq_runlist_status(ctypes.c_void_p(self._workspace.data_ptr()), ctypes.byref(out), stream))
+        return out.value

@@ -1,0 +1,146 @@
+"""Run-list decode path (one persistent launch over many linears) against the oracle and against
+the per-linear entry point."""
+import numpy as np
+import pytest
+import torch
+
+import nanoquant_amd  # noqa: F401
+from nanoquant_amd import DecodeRunList, packing
+from oracle import nq_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+TIGHT = 1e-3   # fp16, ranks >= 256: the fp32-accumulate budget (max|y-y_ref| / max|y_ref|)
+
+
+def _term(dev, m, n, r, seed):
+    vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, seed)
+    f = lambda a: torch.from_numpy(a).to(dev)
+    ops = (f(s_in), packing.binary_packer(torch.from_numpy(vt), "half2").to(dev), f(s_mid),
+           packing.binary_packer(torch.from_numpy(u), "half2").to(dev), f(s_out))
+    return (vt, u, s_in, s_mid, s_out), ops
+
+
+@pytest.mark.parametrize("batch", [1, 4, 16])
+@pytest.mark.parametrize("interleave", [1, 2, 3])
+def test_independent_linears(dev, batch, interleave):
+    shapes = [(512, 1024, 256), (1376, 512, 384), (512, 1376, 352), (96, 160, 64), (2048, 2048, 1024)]
+    rl = DecodeRunList(batch, torch.float16, dev, interleave=interleave)
+    refs = []
+    for i, (m, n, r) in enumerate(shapes):
+        npt, ops = _term(dev, m, n, r, seed=100 + i)
+        x = oracle.synth_x(batch, n, 100 + i)
+        rl.add(torch.from_numpy(x).to(dev), *ops)
+        refs.append(oracle.layer_forward(x.astype(np.float64), *npt, dtype=np.float64))
+    print(f"runlist independent B={batch} interleave={interleave}", flush=True)
+    for rep in range(3):                       # repeated runs: the counters must come back to zero
+        for y in rl.outputs:
+            y.zero_()
+        ys = rl.run()
+        torch.cuda.synchronize()
+        assert rl.status() == 0
+        for (m, n, r), y, ref in zip(shapes, ys, refs):
+            err = oracle.max_rel_err(y.float().cpu().numpy(), ref)
+            assert err < (TIGHT if r >= 256 else 1e-2), (rep, m, n, r, err)
+
+
+def test_matches_per_linear_entry_point_bitwise(dev):
+    # same arithmetic per 16-byte unit, different summation tree across units: agreement to fp32
+    # rounding of the row sums, i.e. far below one fp16 ulp of the output for almost all elements
+    m, n, r, batch = 1024, 4096, 512, 2
+    npt, ops = _term(dev, m, n, r, seed=7)
+    x = torch.from_numpy(oracle.synth_x(batch, n, 7)).to(dev)
+    rl = DecodeRunList(batch, torch.float16, dev)
+    rl.add(x, *ops)
+    y_rl = rl.run()[0].float()
+    y_op = torch.ops.binary_kernels.nanoquant_dyn_forward(x, *ops, 128, 128, 2, 2, 1, 1, 8, 8).float()
+    torch.cuda.synchronize()
+    assert torch.allclose(y_rl, y_op, rtol=2e-3, atol=0)
+    assert (y_rl == y_op).float().mean() > 0.9
+
+
+def test_chained_linears_depend_on_each_other(dev):
+    # y of linear i is x of linear i+1: the in-kernel dependency counters order them
+    dims = [768, 512, 1024, 256]
+    batch = 2
+    rl = DecodeRunList(batch, torch.float16, dev, interleave=3)
+    x0 = oracle.synth_x(batch, dims[0], 3)
+    cur = torch.from_numpy(x0).to(dev)
+    ref = x0.astype(np.float64)
+    for i in range(len(dims) - 1):
+        n, m = dims[i], dims[i + 1]
+        npt, ops = _term(dev, m, n, 256, seed=40 + i)
+        # big scales so that values stay O(1) through the chain
+        scale_up = torch.tensor(8.0, dtype=torch.float16, device=dev)
+        ops = (ops[0] * scale_up, ops[1], ops[2] * scale_up, ops[3], ops[4] * scale_up)
+        npt = (npt[0], npt[1], (ops[0].float().cpu().numpy()), ops[2].float().cpu().numpy(), ops[4].float().cpu().numpy())
+        idx = rl.add(cur, *ops, x_from=i - 1)
+        cur = rl.outputs[idx]
+        ref = oracle.layer_forward(ref, *npt, dtype=np.float64)
+        ref = ref.astype(np.float16).astype(np.float64)     # y is stored as fp16 between linears
+    for rep in range(2):
+        ys = rl.run()
+        torch.cuda.synchronize()
+        assert rl.status() == 0
+        err = oracle.max_rel_err(ys[-1].float().cpu().numpy(), ref)
+        assert err < 5e-3, err
+
+
+def test_mixture_through_addend(dev):
+    m, n, batch = 512, 1024, 4
+    x = oracle.synth_x(batch, n, 5)
+    xt = torch.from_numpy(x).to(dev)
+    t0, ops0 = _term(dev, m, n, 320, seed=60)
+    t1, ops1 = _term(dev, m, n, 128, seed=61)
+    rl = DecodeRunList(batch, torch.float16, dev, interleave=2)
+    i0 = rl.add(xt, *ops0, out_f32=True)
+    i1 = rl.add(xt, *ops1, addend=rl.outputs[i0], y_from=i0)
+    y = rl.run()[i1]
+    torch.cuda.synchronize()
+    ref = oracle.mixture_forward(x.astype(np.float64), [t0, t1], dtype=np.float64)
+    assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < TIGHT
+
+
+def test_bf16_and_ragged_shapes(dev):
+    rl = DecodeRunList(1, torch.bfloat16, dev)
+    refs = []
+    for i, (m, n, r) in enumerate([(100, 1000, 70), (33, 4100, 2985), (300, 96, 32)]):
+        vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, 200 + i)
+        x = oracle.synth_x(1, n, 200 + i)
+        bf = lambda a: torch.from_numpy(a.astype(np.float32)).to(torch.bfloat16)
+        xt, si, sm, so = bf(x), bf(s_in), bf(s_mid), bf(s_out)
+        rl.add(xt.to(dev), si.to(dev), packing.binary_packer(torch.from_numpy(vt), "half2").to(dev), sm.to(dev),
+               packing.binary_packer(torch.from_numpy(u), "half2").to(dev), so.to(dev))
+        refs.append(oracle.layer_forward(xt.float().numpy(), vt, u, si.float().numpy(), sm.float().numpy(),
+                                         so.float().numpy(), dtype=np.float64))
+    ys = rl.run()
+    torch.cuda.synchronize()
+    assert rl.status() == 0
+    for y, ref in zip(ys, refs):
+        assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < 1e-2
+
+
+def test_graph_replay_of_a_run_list(dev):
+    # the launch allocates nothing and can be replayed; replays must equal the eager result
+    batch = 1
+    rl = DecodeRunList(batch, torch.float16, dev, interleave=2)
+    xs = []
+    for i, (m, n, r) in enumerate([(1024, 1024, 512), (1024, 2048, 512), (2048, 1024, 512)]):
+        _, ops = _term(dev, m, n, r, seed=300 + i)
+        x = torch.from_numpy(oracle.synth_x(batch, n, 300 + i)).to(dev)
+        xs.append(x)
+        rl.add(x, *ops)
+    eager = [y.clone() for y in rl.run()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        rl.run()
+    for rep in range(4):
+        for y in rl.outputs:
+            y.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert rl.status() == 0
+        for y, e in zip(rl.outputs, eager):
+            assert torch.equal(y, e), rep
