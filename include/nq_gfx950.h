@@ -65,7 +65,7 @@ int nq_gemv_mixture(const void* x, const void* const* s_in, const uint32_t* cons
                     int batch, int n, int m, int dtype, void* stream);
 
 /* Decode path, run-list form: a whole list of linears (a decoder layer, a decoder stack) in ONE
- * persistent kernel launch.  No counterpart in the reference, which launches two kernels per linear
+ * kernel launch.  No counterpart in the reference, which launches two kernels per linear
  * from Python (modules/linear.py:121-130 -> kernel/cuda/gemv_kernel.cu:406-425); it exists because a
  * 1-bit linear is worth well under a microsecond of HBM time and launch boundaries would dominate.
  *
@@ -76,12 +76,14 @@ int nq_gemv_mixture(const void* x, const void* const* s_in, const uint32_t* cons
  * is added before the store.
  *
  * nq_runlist_build writes the stage table into `workspace` (device memory of at least
- * nq_runlist_workspace_bytes(nlinears) bytes, 256-byte aligned) -- it copies from host memory, so it
+ * nq_runlist_workspace_bytes(linears, nlinears) bytes, 256-byte aligned) -- it copies from host memory, so it
  * synchronises with the host and must not be captured in a graph.  `interleave` >= 1 is how many
  * first stages of independent linears are placed between a linear's two stages, which hides the
  * device-wide hand-over of h; linears inside that window need distinct h buffers.
  * nq_runlist_run enqueues the single launch; it allocates nothing and can be graph-captured.  Runs of
  * the same workspace must not overlap in time.  batch must be 1, 2, 4, 8 or 16.
+ * Inside the launch a stage waits for the stages it depends on through device-scope counters; the
+ * waits are bounded.
  * nq_runlist_status copies the error word back (synchronises): 0 ok, 1 = a bounded dependency wait
  * expired (the results of that run are invalid; call nq_runlist_build again before reuse). */
 typedef struct nq_linear {
@@ -100,10 +102,15 @@ typedef struct nq_linear {
     int out_f32;
 } nq_linear;
 
-size_t nq_runlist_workspace_bytes(int nlinears);
+/* Launch geometry of a built run list; filled by nq_runlist_build, passed back to nq_runlist_run. */
+typedef struct nq_runlist_plan {
+    int nlinears, nstages, total_workgroups, max_units, batch, dtype;
+} nq_runlist_plan;
+
+size_t nq_runlist_workspace_bytes(const nq_linear* linears, int nlinears);
 int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtype, int interleave,
-                     void* workspace, size_t workspace_bytes, void* stream);
-int nq_runlist_run(const void* workspace, int nlinears, int batch, int dtype, void* stream);
+                     void* workspace, size_t workspace_bytes, nq_runlist_plan* plan_out, void* stream);
+int nq_runlist_run(const void* workspace, const nq_runlist_plan* plan, void* stream);
 int nq_runlist_status(const void* workspace, int* status_out, void* stream);
 
 /* One matmul-free stage: out[b,row] = s_row[row] * sum_c sgn(bits[row,c]) * in[b,c] * s_col[c].

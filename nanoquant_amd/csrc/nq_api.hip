@@ -109,31 +109,46 @@ int nq_gemv_stage(const void* in, const void* s_col, const uint32_t* bits, const
 }
 
 // ---- run list ---------------------------------------------------------------------------------
-// workspace layout: [0,256): status word; [256, 256 + 4*(2n+1) rounded to 256): counters (one per
-// stage + the exit counter); then 2n RunStage records.
-static size_t runlist_counter_bytes(int n) { return ((size_t)(2 * n + 1) * 4 + 255) / 256 * 256; }
+// workspace layout: [0,256): status word; counters (one per stage + the exit counter, rounded to
+// 256 bytes); 2n RunStage records (rounded to 256 bytes); one int per workgroup naming its stage.
+static size_t round256(size_t v) { return (v + 255) / 256 * 256; }
+static size_t runlist_counter_bytes(int n) { return round256(nq::stream_counter_bytes(2 * n)); }
+static size_t runlist_table_bytes(int n) { return round256((size_t)2 * n * sizeof(nq::RunStage)); }
 
-size_t nq_runlist_workspace_bytes(int nlinears) {
-    if (nlinears <= 0) return 0;
-    return 256 + runlist_counter_bytes(nlinears) + (size_t)2 * nlinears * sizeof(nq::RunStage);
+static int stage_workgroups(int rows, int cols) {
+    const int units = ((cols + 31) / 32 + 3) / 4;
+    const int per = nq::stream_rows_per_item(units);
+    return (rows + per - 1) / per;
+}
+
+size_t nq_runlist_workspace_bytes(const nq_linear* linears, int nlinears) {
+    if (nlinears <= 0 || !linears) return 0;
+    size_t wgs = 0;
+    for (int i = 0; i < nlinears; ++i) {
+        if (linears[i].n <= 0 || linears[i].r <= 0 || linears[i].m <= 0) return 0;
+        wgs += (size_t)stage_workgroups(linears[i].r, linears[i].n) + (size_t)stage_workgroups(linears[i].m, linears[i].r);
+    }
+    return 256 + runlist_counter_bytes(nlinears) + runlist_table_bytes(nlinears) + round256(wgs * sizeof(int));
 }
 
 static inline bool al16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtype, int interleave,
-                     void* workspace, size_t workspace_bytes, void* stream) {
+                     void* workspace, size_t workspace_bytes, nq_runlist_plan* plan_out, void* stream) {
+    if (!plan_out) return NQ_ERR_NULL;
     if (dtype != NQ_F16 && dtype != NQ_BF16) return NQ_ERR_DTYPE;
     if (nlinears <= 0 || interleave < 1) return NQ_ERR_SHAPE;
     if (batch != 1 && batch != 2 && batch != 4 && batch != 8 && batch != 16) return NQ_ERR_SHAPE;
     if (!linears || !workspace) return NQ_ERR_NULL;
     if (((uintptr_t)workspace & 255u) != 0) return NQ_ERR_ALIGN;
-    if (workspace_bytes < nq_runlist_workspace_bytes(nlinears)) return NQ_ERR_WORKSPACE;
     for (int i = 0; i < nlinears; ++i) {
         const nq_linear& l = linears[i];
         if (l.n <= 0 || l.r <= 0 || l.m <= 0) return NQ_ERR_SHAPE;
         if (!l.x || !l.s_in || !l.vt_bits || !l.u_bits || !l.s_out || !l.h || !l.y) return NQ_ERR_NULL;
         if (l.x_from >= i || l.y_from >= i) return NQ_ERR_SHAPE;
+        if (l.y_from >= 0 && !linears[l.y_from].out_f32) return NQ_ERR_SHAPE;   // addends are fp32 results
     }
+    if (workspace_bytes < nq_runlist_workspace_bytes(linears, nlinears)) return NQ_ERR_WORKSPACE;
     // Order of stages: first stages run ahead of second stages by up to `interleave` linears, unless a
     // dependency (or a shared h buffer) forces a second stage out earlier.
     std::vector<nq::RunStage> table;
@@ -147,6 +162,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         st.rows = l.m; st.K = l.r; st.words = (l.r + 31) / 32; st.units = (st.words + 3) / 4;
         st.in_stride = l.r; st.out_stride = l.m; st.in_f32 = 1; st.out_f32 = l.out_f32 ? 1 : 0;
         st.dep = first_idx[i];
+        st.in_coherent = 1;
         st.dep2 = (l.addend && l.y_from >= 0) ? second_idx[l.y_from] : -1;
         st.signal = 0;
         st.vec_bits = (st.words % 4 == 0) && al16(l.u_bits);
@@ -175,8 +191,12 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         st.rows = l.r; st.K = l.n; st.words = (l.n + 31) / 32; st.units = (st.words + 3) / 4;
         st.in_stride = l.n; st.out_stride = l.r; st.in_f32 = 0; st.out_f32 = 1;
         st.dep = l.x_from >= 0 ? second_idx[l.x_from] : -1;
+        if (st.dep >= 0) {                       // 16-bit y of an earlier linear is this linear's x
+            st.heavy_acquire = 1;
+            table[st.dep].heavy_release = 1;
+        }
         st.dep2 = -1;
-        st.signal = 1;
+        st.signal = 0;
         st.vec_bits = (st.words % 4 == 0) && al16(l.vt_bits);
         st.vec_in = al16(l.x) && ((size_t)l.n * 2) % 16 == 0 && al16(l.s_in);
         first_idx[i] = (int)table.size();
@@ -185,32 +205,53 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         if ((int)pending.size() >= interleave) flush_until(pending.front());
     }
     flush_until(-1);
+    for (auto& st : table) st.signal = 0;
+    int total_wgs = 0, max_units = 1;
     for (auto& st : table) {
+        if (st.units > max_units) max_units = st.units;
         if (st.dep >= 0) table[st.dep].signal = 1;
         if (st.dep2 >= 0) table[st.dep2].signal = 1;
+        st.rows_item = nq::stream_rows_per_item(st.units);
+        st.wg_begin = total_wgs;
+        st.wg_count = (st.rows + st.rows_item - 1) / st.rows_item;
+        total_wgs += st.wg_count;
     }
+    std::vector<int> wg_stage((size_t)total_wgs);
+    for (size_t si = 0; si < table.size(); ++si)
+        for (int w = 0; w < table[si].wg_count; ++w) wg_stage[(size_t)table[si].wg_begin + w] = (int)si;
     hipStream_t hs = (hipStream_t)stream;
     char* base = (char*)workspace;
-    hipError_t e = hipMemsetAsync(base, 0, 256 + runlist_counter_bytes(nlinears), hs);
+    const size_t off_table = 256 + runlist_counter_bytes(nlinears);
+    const size_t off_map = off_table + runlist_table_bytes(nlinears);
+    hipError_t e = hipMemsetAsync(base, 0, off_table, hs);
     if (e != hipSuccess) return hip_status(e);
-    e = hipMemcpyAsync(base + 256 + runlist_counter_bytes(nlinears), table.data(), table.size() * sizeof(nq::RunStage),
-                       hipMemcpyHostToDevice, hs);
+    e = hipMemcpyAsync(base + off_table, table.data(), table.size() * sizeof(nq::RunStage), hipMemcpyHostToDevice, hs);
     if (e != hipSuccess) return hip_status(e);
-    return hip_status(hipStreamSynchronize(hs));   // `table` is host stack memory: finish before it dies
+    e = hipMemcpyAsync(base + off_map, wg_stage.data(), wg_stage.size() * sizeof(int), hipMemcpyHostToDevice, hs);
+    if (e != hipSuccess) return hip_status(e);
+    plan_out->nlinears = nlinears;
+    plan_out->nstages = (int)table.size();
+    plan_out->total_workgroups = total_wgs;
+    plan_out->max_units = max_units;
+    plan_out->batch = batch;
+    plan_out->dtype = dtype;
+    return hip_status(hipStreamSynchronize(hs));   // `table` is host memory: finish before it dies
 }
 
-int nq_runlist_run(const void* workspace, int nlinears, int batch, int dtype, void* stream) {
-    if (dtype != NQ_F16 && dtype != NQ_BF16) return NQ_ERR_DTYPE;
-    if (nlinears <= 0) return NQ_ERR_SHAPE;
+int nq_runlist_run(const void* workspace, const nq_runlist_plan* plan, void* stream) {
+    if (!workspace || !plan) return NQ_ERR_NULL;
+    if (plan->dtype != NQ_F16 && plan->dtype != NQ_BF16) return NQ_ERR_DTYPE;
+    if (plan->nlinears <= 0 || plan->nstages != 2 * plan->nlinears || plan->total_workgroups <= 0 ||
+        plan->max_units <= 0)
+        return NQ_ERR_SHAPE;
+    const int batch = plan->batch;
     if (batch != 1 && batch != 2 && batch != 4 && batch != 8 && batch != 16) return NQ_ERR_SHAPE;
-    if (!workspace) return NQ_ERR_NULL;
-    static int nwg = 0;
-    if (nwg == 0) nwg = nq::stream_max_workgroups();
-    if (nwg <= 0) return NQ_ERR_HIP;
     char* base = (char*)workspace;
-    return hip_status(nq::gemv_stream(dtype, batch, (const nq::RunStage*)(base + 256 + runlist_counter_bytes(nlinears)),
-                                      2 * nlinears, (unsigned*)(base + 256), (unsigned*)base, nwg,
-                                      (hipStream_t)stream));
+    const size_t off_table = 256 + runlist_counter_bytes(plan->nlinears);
+    const size_t off_map = off_table + runlist_table_bytes(plan->nlinears);
+    return hip_status(nq::gemv_stream(plan->dtype, batch, (const nq::RunStage*)(base + off_table), plan->nstages,
+                                      (const int*)(base + off_map), (unsigned long long*)(base + 256), (unsigned*)base,
+                                      plan->total_workgroups, plan->max_units, (hipStream_t)stream));
 }
 
 int nq_runlist_status(const void* workspace, int* status_out, void* stream) {

@@ -12,7 +12,7 @@ hipError_t gemv_stage(int dtype, bool first, const uint32_t* bits, const void* i
                       const void* s_row, const float* addend, void* out, bool out_f32, int batch, int rows,
                       int words, int K, int in_stride, int out_stride, hipStream_t stream);
 
-// nq_stream.hip: one persistent launch over a table of stages (see the file header).
+// nq_stream.hip: one launch over a table of stages (see the file header).
 struct RunStage {
     const uint32_t* bits;   // [rows, words] packed signs, row-major "half2" order
     const void* in;         // [batch, in_stride]: 16-bit activations, or fp32 when in_f32
@@ -26,11 +26,16 @@ struct RunStage {
     int dep, dep2;          // stage indices that must be complete before `in` / `addend` are read, or -1
     int signal;             // a later stage waits on this one
     int vec_bits, vec_in;
-    int pad_;
+    int wg_begin, wg_count; // this stage's work items are workgroups [wg_begin, wg_begin + wg_count)
+    int rows_item;          // rows per work item
+    int in_coherent;        // fp32 input written by another stage of the same launch
+    int heavy_release;      // 16-bit output read by a later stage: full device-scope release on completion
+    int heavy_acquire;      // 16-bit input written by an earlier stage: full device-scope acquire after the wait
 };
-int stream_max_workgroups();
-hipError_t gemv_stream(int dtype, int batch, const RunStage* stages, int nstages, unsigned* counters,
-                       unsigned* status, int nwg, hipStream_t stream);
+int stream_rows_per_item(int units);
+size_t stream_counter_bytes(int nstages);
+hipError_t gemv_stream(int dtype, int batch, const RunStage* stages, int nstages, const int* wg_stage,
+                       unsigned long long* counters, unsigned* status, int total_wgs, int max_units, hipStream_t stream);
 
 // nq_gemm.hip: C[T,R] = s_out * ((x * s_in) . sgn(W)^T) with W in the 32x256 tile layout.
 // scratch: fp32 [T,R] when gemm_scratch_bytes(T,K,R) > 0.

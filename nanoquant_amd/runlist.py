@@ -1,4 +1,4 @@
-"""Host side of the run-list decode path: many linears, one persistent kernel launch.
+"""Host side of the run-list decode path: many linears, one kernel launch.
 
 `DecodeRunList` owns the device workspace (stage table + completion counters) and the fp32
 intermediates of a list of linears; `run()` enqueues the single launch on the current stream and can
@@ -25,6 +25,12 @@ class NqLinear(ctypes.Structure):
         ("n", ctypes.c_int), ("r", ctypes.c_int), ("m", ctypes.c_int),
         ("x_from", ctypes.c_int), ("y_from", ctypes.c_int), ("out_f32", ctypes.c_int),
     ]
+
+
+class NqRunlistPlan(ctypes.Structure):
+    """Mirror of `nq_runlist_plan`."""
+    _fields_ = [("nlinears", ctypes.c_int), ("nstages", ctypes.c_int), ("total_workgroups", ctypes.c_int),
+                ("max_units", ctypes.c_int), ("batch", ctypes.c_int), ("dtype", ctypes.c_int)]
 
 
 class DecodeRunList:
@@ -86,12 +92,14 @@ class DecodeRunList:
             arr[i] = NqLinear(p(e["x"]), p(e["s_in"]), p(e["vt"]), p(e["s_mid"]), p(e["u"]), p(e["s_out"]), p(e["h"]),
                               p(e["y"]), p(e["addend"]), e["n"], e["r"], e["m"], e["x_from"], e["y_from"], e["out_f32"])
         lib = _lib.lib()
-        nbytes = int(lib.nq_runlist_workspace_bytes(n))
+        nbytes = int(lib.nq_runlist_workspace_bytes(arr, n))
         ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
         with torch.cuda.device(self.device):
             stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+            plan = NqRunlistPlan()
             _lib.check(lib.nq_runlist_build(arr, n, self.batch, self._dtype_id(), self.interleave,
-                                            ctypes.c_void_p(ws.data_ptr()), nbytes, stream))
+                                            ctypes.c_void_p(ws.data_ptr()), nbytes, ctypes.byref(plan), stream))
+        self._plan = plan
         self._workspace = ws
 
     def _dtype_id(self) -> int:
@@ -104,8 +112,8 @@ class DecodeRunList:
             self.build()
         with torch.cuda.device(self.device):
             stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
-            _lib.check(_lib.lib().nq_runlist_run(ctypes.c_void_p(self._workspace.data_ptr()), len(self._entries),
-                                                 self.batch, self._dtype_id(), stream))
+            _lib.check(_lib.lib().nq_runlist_run(ctypes.c_void_p(self._workspace.data_ptr()),
+                                                 ctypes.byref(self._plan), stream))
         return self.outputs
 
     def status(self) -> int:
