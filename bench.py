@@ -74,7 +74,7 @@ def main():
     ap.add_argument("--steps", type=int, default=520)
     ap.add_argument("--warmup", type=int, default=52)
     ap.add_argument("--copies", type=int, default=26, help="distinct weight copies of the layer (26 x 25.3 MB > 256 MB)")
-    ap.add_argument("--interleave", type=int, default=2, help="first stages run ahead of second stages by this many linears")
+    ap.add_argument("--interleave", type=int, default=7, help="first stages run ahead of second stages by this many linears")
     ap.add_argument("--no-extra", action="store_true", help="skip batch 4/16, prefill and CPU legs")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()

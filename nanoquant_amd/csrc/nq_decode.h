@@ -25,6 +25,8 @@
 
 namespace nq {
 
+constexpr int kXsumStride = 576;   // floats of unit sums per batch row: >= largest staged chunk (| 1), multiple of 4
+
 __device__ __forceinline__ uint32_t comp_d(const uint4& v, int i) {
     return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
 }

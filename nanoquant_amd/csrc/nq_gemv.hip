@@ -12,11 +12,10 @@
 //
 // Mapping: a workgroup of 4 wavefronts stages the scaled input vector(s) once in LDS as 16-bit pairs.
 // A wavefront is split into 64/G lane groups; a lane group owns RPW rows and its G lanes stride over
-// the row's 16-byte units (4 words = 128 columns).  The sign of pair j of a word is the word shifted
-// left by j and masked to bits 15 and 31, OR-ed onto the pair (1.0, 1.0): that +-1 pair is the second
-// operand of v_dot2_f32_{f16,bf16}, so one instruction adds two signed activations into an fp32
-// accumulator.  Row sums are finished with DPP moves inside a 16-lane row and two ds_bpermute steps.
-#include "nq_common.h"
+// the row's 16-byte units (4 words = 128 columns).  The arithmetic of a unit (masked words used
+// directly as the second operand of v_dot2_f32_{f16,bf16}, fp32 accumulators) is in nq_decode.h.
+// Row sums are finished with DPP moves inside a 16-lane row and two ds_bpermute steps.
+#include "nq_decode.h"
 #include "nq_kernels.h"
 
 namespace nq {
@@ -37,68 +36,6 @@ struct StageArgs {
     const float* addend;    // [batch, out_stride] fp32 added before the store (sum over terms), may be null
     int out_f32;            // store fp32 instead of the 16-bit activation type
 };
-
-__device__ __forceinline__ uint32_t comp(const uint4& v, int i) {
-    return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
-}
-
-// Stage the scaled input of units [c0, c0+cu_n) into LDS.  Layout: 16-byte chunk (b, i, cu) at
-// lds[(b*16 + i)*upad + cu] holds the 8 consecutive columns 128*(c0+cu) + 8*i .. +7.  For a fixed i
-// the lanes of a group read consecutive 16-byte chunks (conflict-free); upad is odd so that the
-// staging writes, which run along i, spread over the banks too.
-template <int DT, bool FIRST, int BATCH>
-__device__ __forceinline__ void stage_input(uint4* lds, const StageArgs& a, int c0, int cu_n, int upad) {
-    using E = Elem<DT>;
-    const int nchunks = cu_n * 16;
-#pragma unroll 1
-    for (int b = 0; b < BATCH; ++b) {
-        for (int q = threadIdx.x; q < nchunks; q += blockDim.x) {
-            const int cu = q >> 4, i = q & 15;
-            const int col = (c0 + cu) * 128 + i * 8;
-            float v[8];
-            if (a.vec_in && col + 8 <= a.K) {
-                if constexpr (FIRST) {
-                    const uint16_t* xp = (const uint16_t*)a.in + (size_t)b * a.in_stride + col;
-                    uint4 xr = *(const uint4*)xp;
-                    uint4 sr = a.s_col ? *(const uint4*)(a.s_col + col)
-                                       : make_uint4(E::kOnePair, E::kOnePair, E::kOnePair, E::kOnePair);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        uint32_t xw = comp(xr, e), sw = comp(sr, e);
-                        v[2 * e] = E::to_float(xw & 0xFFFFu) * E::to_float(sw & 0xFFFFu);
-                        v[2 * e + 1] = E::to_float(xw >> 16) * E::to_float(sw >> 16);
-                    }
-                } else {
-                    const float* hp = (const float*)a.in + (size_t)b * a.in_stride + col;
-                    float4 h0 = *(const float4*)hp, h1 = *(const float4*)(hp + 4);
-                    v[0] = h0.x; v[1] = h0.y; v[2] = h0.z; v[3] = h0.w;
-                    v[4] = h1.x; v[5] = h1.y; v[6] = h1.z; v[7] = h1.w;
-                }
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int c = col + e;
-                    float t = 0.f;
-                    if (c < a.K) {
-                        if constexpr (FIRST) {
-                            t = E::to_float(((const uint16_t*)a.in)[(size_t)b * a.in_stride + c]);
-                            if (a.s_col) t *= E::to_float(a.s_col[c]);
-                        } else {
-                            t = ((const float*)a.in)[(size_t)b * a.in_stride + c];
-                        }
-                    }
-                    v[e] = t;
-                }
-            }
-            uint4 p;
-            p.x = (uint32_t)E::from_float(v[0]) | ((uint32_t)E::from_float(v[1]) << 16);
-            p.y = (uint32_t)E::from_float(v[2]) | ((uint32_t)E::from_float(v[3]) << 16);
-            p.z = (uint32_t)E::from_float(v[4]) | ((uint32_t)E::from_float(v[5]) << 16);
-            p.w = (uint32_t)E::from_float(v[6]) | ((uint32_t)E::from_float(v[7]) << 16);
-            lds[(b * 16 + i) * upad + cu] = p;
-        }
-    }
-}
 
 template <int RPW>
 __device__ __forceinline__ void load_bits(uint4 (&w)[RPW], const StageArgs& a, int row0, int unit, bool active) {
@@ -125,8 +62,13 @@ __device__ __forceinline__ void load_bits(uint4 (&w)[RPW], const StageArgs& a, i
 template <int DT, bool FIRST, int BATCH, int RPW>
 __global__ __launch_bounds__(256) void gemv_stage_kernel(StageArgs a) {
     using E = Elem<DT>;
-    extern __shared__ uint4 lds[];
+    extern __shared__ uint4 lds_raw[];
+    float* xsum = (float*)lds_raw;                       // [BATCH][kXsumStride] per-unit input sums
+    uint4* lds = lds_raw + (BATCH * kXsumStride * sizeof(float)) / sizeof(uint4);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    StageInput sin;
+    sin.in = a.in; sin.s_col = a.s_col; sin.K = a.K; sin.in_stride = a.in_stride;
+    sin.in_f32 = FIRST ? 0 : 1; sin.in_coherent = 0; sin.vec_in = a.vec_in;
     const int G = 1 << a.group_log2;
     const int g = lane & (G - 1), slot = lane >> a.group_log2;
     const int rows_per_wave = (kWave >> a.group_log2) * RPW;
@@ -147,7 +89,7 @@ __global__ __launch_bounds__(256) void gemv_stage_kernel(StageArgs a) {
     for (int c0 = 0; c0 < a.units; c0 += a.chunk_units) {
         const int cu_n = min(a.chunk_units, a.units - c0);
         if (c0) __syncthreads();
-        stage_input<DT, FIRST, BATCH>(lds, a, c0, cu_n, upad);
+        stage_units<DT, BATCH>(lds, xsum, sin, c0, cu_n, upad, (int)blockDim.x);
         __syncthreads();
 #pragma unroll 1
         for (int cu = g; cu - g < cu_n; cu += G) {
@@ -163,26 +105,11 @@ __global__ __launch_bounds__(256) void gemv_stage_kernel(StageArgs a) {
             }
             if (active) {
 #pragma unroll
-                for (int wi = 0; wi < 4; ++wi) {
-                    uint32_t sp[RPW][16];
+                for (int rr = 0; rr < RPW; ++rr) {
+                    float part[BATCH];
+                    UnitDot<DT, BATCH>::run(w[rr], lds, xsum, upad, cu, part);
 #pragma unroll
-                    for (int rr = 0; rr < RPW; ++rr) {
-                        const uint32_t word = comp(w[rr], wi);
-#pragma unroll
-                        for (int j = 0; j < 16; ++j) sp[rr][j] = ((word << j) & kSignPair) | E::kOnePair;
-                    }
-#pragma unroll
-                    for (int b = 0; b < BATCH; ++b) {
-                        uint4 xv[4];
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) xv[q] = lds[(b * 16 + 4 * wi + q) * upad + cu];
-#pragma unroll
-                        for (int j = 0; j < 16; ++j) {
-                            const uint32_t xp = comp(xv[j >> 2], j & 3);
-#pragma unroll
-                            for (int rr = 0; rr < RPW; ++rr) acc[rr][b] = E::dot2(xp, sp[rr][j], acc[rr][b]);
-                        }
-                    }
+                    for (int b = 0; b < BATCH; ++b) acc[rr][b] += part[b];
                 }
             }
         }
@@ -219,12 +146,13 @@ static int pick_group_log2(int units) {
 }
 
 constexpr int kLdsBudget = 144 * 1024;
+constexpr int kXsumBytesPerRow = kXsumStride * (int)sizeof(float);
 
 template <int DT, bool FIRST, int BATCH, int RPW>
 static hipError_t launch_stage(StageArgs a, hipStream_t stream) {
     const int rows_per_block = 4 * (kWave >> a.group_log2) * RPW;
     const int grid = (a.rows + rows_per_block - 1) / rows_per_block;
-    const size_t lds_bytes = (size_t)BATCH * 16 * (a.chunk_units | 1) * sizeof(uint4);
+    const size_t lds_bytes = (size_t)BATCH * kXsumBytesPerRow + (size_t)BATCH * 16 * (a.chunk_units | 1) * sizeof(uint4);
     auto kern = gemv_stage_kernel<DT, FIRST, BATCH, RPW>;
     static bool attr_done = false;  // per template instance; raised once to the full budget
     if (lds_bytes > 64 * 1024 && !attr_done) {
@@ -278,8 +206,9 @@ hipError_t gemv_stage(int dtype, bool first, const uint32_t* bits, const void* i
     while (done < batch) {
         int piece = 16;
         while (piece > batch - done) piece >>= 1;
-        int cap = kLdsBudget / (piece * 16 * (int)sizeof(uint4));   // chunk_units|1 must fit
+        int cap = (kLdsBudget - piece * kXsumBytesPerRow) / (piece * 16 * (int)sizeof(uint4));   // chunk_units|1 must fit
         cap = (cap - 1) & ~1;                                       // even, so that cap|1 <= budget
+        if (cap > kXsumStride - 2) cap = kXsumStride - 2;
         a.chunk_units = a.units < cap ? a.units : cap;
         a.group_log2 = pick_group_log2(a.chunk_units);
         a.in = (const char*)in + (size_t)done * in_stride * in_elt;

@@ -38,7 +38,6 @@ constexpr int kStreamThreads = 256;
 constexpr int kRowBlock = 128;                 // rows finished per pass of a workgroup
 // Same-address device-scope atomics serialise at the memory side (tens of ns each), so completion
 // counts are spread over kSubCounters addresses per stage and kExitSubs addresses for the exit count.
-constexpr int kXsumStride = 576;                // >= largest upad (chunk_cap | 1), multiple of 4
 constexpr int kSubCounters = 8;
 constexpr int kExitSubs = 64;
 constexpr int kCounterStride = 8;              // 64-bit words between sub-counters: one 64-byte line each
@@ -270,9 +269,10 @@ static hipError_t launch_stream(const RunStage* stages, int nstages, const int* 
     return hipGetLastError();
 }
 
-// Rows per work item: about four 16-byte units per lane, at most kRowBlock rows.
+// Rows per work item: about three 16-byte units per lane (measured best for a single decoder layer per
+// launch: shorter items finish the first stages sooner), at most kRowBlock rows.
 int stream_rows_per_item(int units) {
-    int rows = (4 * kStreamThreads + units / 2) / units;
+    int rows = (3 * kStreamThreads + units / 2) / units;
     if (rows < 1) rows = 1;
     if (rows > kRowBlock) rows = kRowBlock;
     return rows;
