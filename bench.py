@@ -25,6 +25,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the headline kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
+# copy kernel of known size (profiles/gemv_stream_llama2_7b_layer_b1.md); valid for the default workload only.
+MEASURED_TRAFFIC_BYTES = 28184334
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 LLAMA2_7B_LAYER = (("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096),
@@ -77,6 +80,9 @@ def main():
     ap.add_argument("--interleave", type=int, default=7, help="first stages run ahead of second stages by this many linears")
     ap.add_argument("--no-extra", action="store_true", help="skip batch 4/16, prefill and CPU legs")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch the library's plain copy kernel on 256 MiB (5x): a known-traffic reference "
+                         "for scaling profiler memory counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the layer is a single-GPU hot path); "
@@ -199,16 +205,26 @@ def main():
         "us_per_layer": round(ms * 1e3, 3),
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_stream_kernel<fp16, batch 1> (one persistent launch per layer: 14 stages)",
+            "kernel": "gemv_stream_kernel<fp16, batch 1> (one launch per layer: 14 stages, 1559 workgroups)",
             "achieved": round(bytes1 / launches_per_step / (launch_us * 1e-6) / 1e9, 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(bytes1 / launches_per_step / (launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES if (args.copies == 26 and args.interleave == 7) else None,
             "bytes_per_launch": int(bytes1 / launches_per_step),
             "avg_launch_us": round(launch_us, 3),
         },
     }
+
+    if args.calibrate_copy:
+        nbytes = 256 << 20
+        src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            _lib.check(lib.nq_stream_copy(vp(dst.data_ptr()), vp(src.data_ptr()), nbytes,
+                                          vp(torch.cuda.current_stream().cuda_stream)))
+        torch.cuda.synchronize()
+        result["config"]["calibration_copy_bytes"] = nbytes
 
     if not args.no_extra:
         extra = {}
