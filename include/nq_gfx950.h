@@ -77,9 +77,10 @@ int nq_gemv_mixture(const void* x, const void* const* s_in, const uint32_t* cons
  *
  * nq_runlist_build writes the stage table into `workspace` (device memory of at least
  * nq_runlist_workspace_bytes(linears, nlinears) bytes, 256-byte aligned) -- it copies from host memory, so it
- * synchronises with the host and must not be captured in a graph.  `interleave` >= 1 is how many
- * first stages of independent linears are placed between a linear's two stages, which hides the
- * device-wide hand-over of h; linears inside that window need distinct h buffers.
+ * synchronises with the host and must not be captured in a graph.  Stages are grouped into phases by
+ * dependency depth and every resident workgroup gets an equal share of every phase, so all linears
+ * of a list need distinct h buffers.  `interleave` >= 1 is an ordering hint kept for interface
+ * stability; the phase schedule does not need it.
  * nq_runlist_run enqueues the single launch; it allocates nothing and can be graph-captured.  Runs of
  * the same workspace must not overlap in time.  batch must be 1, 2, 4, 8 or 16.
  * Inside the launch a stage waits for the stages it depends on through device-scope counters; the
@@ -104,7 +105,7 @@ typedef struct nq_linear {
 
 /* Launch geometry of a built run list; filled by nq_runlist_build, passed back to nq_runlist_run. */
 typedef struct nq_runlist_plan {
-    int nlinears, nstages, total_workgroups, max_units, batch, dtype;
+    int nlinears, nstages, nphases, workgroups, max_units, batch, dtype, index_words;
 } nq_runlist_plan;
 
 size_t nq_runlist_workspace_bytes(const nq_linear* linears, int nlinears);

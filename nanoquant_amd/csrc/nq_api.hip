@@ -109,26 +109,28 @@ int nq_gemv_stage(const void* in, const void* s_col, const uint32_t* bits, const
 }
 
 // ---- run list ---------------------------------------------------------------------------------
-// workspace layout: [0,256): status word; counters (one per stage + the exit counter, rounded to
-// 256 bytes); 2n RunStage records (rounded to 256 bytes); one int per workgroup naming its stage.
+// workspace layout: [0,256): status word; completion counters; 2n RunStage records; the slice index
+// (one int per workgroup and phase, +1); the slices.  Every block is rounded to 256 bytes.
 static size_t round256(size_t v) { return (v + 255) / 256 * 256; }
 static size_t runlist_counter_bytes(int n) { return round256(nq::stream_counter_bytes(2 * n)); }
 static size_t runlist_table_bytes(int n) { return round256((size_t)2 * n * sizeof(nq::RunStage)); }
+constexpr int kMaxResidentWorkgroups = 256 * 8 * 2;   // upper bound used for sizing only
 
-static int stage_workgroups(int rows, int cols) {
-    const int units = ((cols + 31) / 32 + 3) / 4;
-    const int per = nq::stream_rows_per_item(units);
-    return (rows + per - 1) / per;
+static size_t runlist_index_bytes(int nwg, int nphases) { return round256(((size_t)nwg * nphases + 1) * sizeof(int)); }
+static size_t runlist_seg_bytes(int nwg, int nphases, int nstages) {
+    return round256(((size_t)nwg * nphases + nstages) * sizeof(nq::RunSegment));
 }
 
 size_t nq_runlist_workspace_bytes(const nq_linear* linears, int nlinears) {
     if (nlinears <= 0 || !linears) return 0;
-    size_t wgs = 0;
-    for (int i = 0; i < nlinears; ++i) {
-        if (linears[i].n <= 0 || linears[i].r <= 0 || linears[i].m <= 0) return 0;
-        wgs += (size_t)stage_workgroups(linears[i].r, linears[i].n) + (size_t)stage_workgroups(linears[i].m, linears[i].r);
-    }
-    return 256 + runlist_counter_bytes(nlinears) + runlist_table_bytes(nlinears) + round256(wgs * sizeof(int));
+    // phases <= stages; a generous bound keeps the call independent of the device
+    int depth_bound = 2;
+    for (int i = 0; i < nlinears; ++i)
+        if (linears[i].x_from >= 0 || linears[i].y_from >= 0) depth_bound += 2;
+    if (depth_bound > 2 * nlinears) depth_bound = 2 * nlinears;
+    return 256 + runlist_counter_bytes(nlinears) + runlist_table_bytes(nlinears) +
+           runlist_index_bytes(kMaxResidentWorkgroups, depth_bound) +
+           runlist_seg_bytes(kMaxResidentWorkgroups, depth_bound, 2 * nlinears);
 }
 
 static inline bool al16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
@@ -147,111 +149,146 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         if (!l.x || !l.s_in || !l.vt_bits || !l.u_bits || !l.s_out || !l.h || !l.y) return NQ_ERR_NULL;
         if (l.x_from >= i || l.y_from >= i) return NQ_ERR_SHAPE;
         if (l.y_from >= 0 && !linears[l.y_from].out_f32) return NQ_ERR_SHAPE;   // addends are fp32 results
+        // two linears writing the same h would race inside a phase
+        for (int j = 0; j < i; ++j)
+            if (linears[j].h == l.h) return NQ_ERR_SHAPE;
     }
     if (workspace_bytes < nq_runlist_workspace_bytes(linears, nlinears)) return NQ_ERR_WORKSPACE;
-    // Order of stages: first stages run ahead of second stages by up to `interleave` linears, unless a
-    // dependency (or a shared h buffer) forces a second stage out earlier.
-    std::vector<nq::RunStage> table;
-    std::vector<int> first_idx(nlinears, -1), second_idx(nlinears, -1);
-    std::vector<int> pending;
-    auto emit_second = [&](int i) {
-        const nq_linear& l = linears[i];
-        nq::RunStage st{};
-        st.bits = l.u_bits; st.in = l.h; st.s_col = nullptr; st.s_row = (const uint16_t*)l.s_out;
-        st.out = l.y; st.addend = l.addend;
-        st.rows = l.m; st.K = l.r; st.words = (l.r + 31) / 32; st.units = (st.words + 3) / 4;
-        st.in_stride = l.r; st.out_stride = l.m; st.in_f32 = 1; st.out_f32 = l.out_f32 ? 1 : 0;
-        st.dep = first_idx[i];
-        st.in_coherent = 1;
-        st.dep2 = (l.addend && l.y_from >= 0) ? second_idx[l.y_from] : -1;
-        st.signal = 0;
-        st.vec_bits = (st.words % 4 == 0) && al16(l.u_bits);
-        st.vec_in = al16(l.h) && ((size_t)l.r * 4) % 16 == 0;
-        second_idx[i] = (int)table.size();
-        table.push_back(st);
-    };
-    auto flush_until = [&](int upto_linear) {   // emit pending second stages in order up to `upto_linear`
-        while (!pending.empty()) {
-            const int i = pending.front();
-            emit_second(i);
-            pending.erase(pending.begin());
-            if (i == upto_linear) break;
-        }
-    };
+    (void)interleave;   // kept for interface stability: phases make the ordering hint unnecessary
+
+    // ---- stage table: stage 2i = first stage of linear i, 2i+1 = its second stage -------------------
+    const int nstages = 2 * nlinears;
+    std::vector<nq::RunStage> table((size_t)nstages);
+    int max_units = 1, nphases = 0;
     for (int i = 0; i < nlinears; ++i) {
         const nq_linear& l = linears[i];
-        int need = -1;
-        for (int j : pending) {
-            if (j == l.x_from || j == l.y_from || linears[j].h == l.h) need = j;
+        nq::RunStage a{};
+        a.bits = l.vt_bits; a.in = l.x; a.s_col = (const uint16_t*)l.s_in; a.s_row = (const uint16_t*)l.s_mid;
+        a.out = l.h; a.addend = nullptr;
+        a.rows = l.r; a.K = l.n; a.words = (l.n + 31) / 32; a.units = (a.words + 3) / 4;
+        a.in_stride = l.n; a.out_stride = l.r; a.in_f32 = 0; a.out_f32 = 1;
+        a.dep = l.x_from >= 0 ? 2 * l.x_from + 1 : -1;
+        a.dep2 = -1;
+        a.vec_bits = (a.words % 4 == 0) && al16(l.vt_bits);
+        a.vec_in = al16(l.x) && ((size_t)l.n * 2) % 16 == 0 && al16(l.s_in);
+        a.phase = a.dep >= 0 ? table[a.dep].phase + 1 : 0;
+        if (a.dep >= 0) {                        // 16-bit y of an earlier linear is this linear's x
+            a.heavy_acquire = 1;
+            table[a.dep].heavy_release = 1;
         }
-        if (need >= 0) flush_until(need);
-        nq::RunStage st{};
-        st.bits = l.vt_bits; st.in = l.x; st.s_col = (const uint16_t*)l.s_in; st.s_row = (const uint16_t*)l.s_mid;
-        st.out = l.h; st.addend = nullptr;
-        st.rows = l.r; st.K = l.n; st.words = (l.n + 31) / 32; st.units = (st.words + 3) / 4;
-        st.in_stride = l.n; st.out_stride = l.r; st.in_f32 = 0; st.out_f32 = 1;
-        st.dep = l.x_from >= 0 ? second_idx[l.x_from] : -1;
-        if (st.dep >= 0) {                       // 16-bit y of an earlier linear is this linear's x
-            st.heavy_acquire = 1;
-            table[st.dep].heavy_release = 1;
-        }
-        st.dep2 = -1;
-        st.signal = 0;
-        st.vec_bits = (st.words % 4 == 0) && al16(l.vt_bits);
-        st.vec_in = al16(l.x) && ((size_t)l.n * 2) % 16 == 0 && al16(l.s_in);
-        first_idx[i] = (int)table.size();
-        table.push_back(st);
-        pending.push_back(i);
-        if ((int)pending.size() >= interleave) flush_until(pending.front());
+        table[2 * i] = a;
+
+        nq::RunStage b{};
+        b.bits = l.u_bits; b.in = l.h; b.s_col = nullptr; b.s_row = (const uint16_t*)l.s_out;
+        b.out = l.y; b.addend = l.addend;
+        b.rows = l.m; b.K = l.r; b.words = (l.r + 31) / 32; b.units = (b.words + 3) / 4;
+        b.in_stride = l.r; b.out_stride = l.m; b.in_f32 = 1; b.out_f32 = l.out_f32 ? 1 : 0;
+        b.dep = 2 * i;
+        b.in_coherent = 1;
+        b.dep2 = (l.addend && l.y_from >= 0) ? 2 * l.y_from + 1 : -1;
+        b.vec_bits = (b.words % 4 == 0) && al16(l.u_bits);
+        b.vec_in = al16(l.h) && ((size_t)l.r * 4) % 16 == 0;
+        b.phase = a.phase + 1;
+        if (b.dep2 >= 0 && table[b.dep2].phase + 1 > b.phase) b.phase = table[b.dep2].phase + 1;
+        table[2 * i + 1] = b;
+        if (a.units > max_units) max_units = a.units;
+        if (b.units > max_units) max_units = b.units;
+        if (b.phase + 1 > nphases) nphases = b.phase + 1;
     }
-    flush_until(-1);
-    for (auto& st : table) st.signal = 0;
-    int total_wgs = 0, max_units = 1;
     for (auto& st : table) {
-        if (st.units > max_units) max_units = st.units;
         if (st.dep >= 0) table[st.dep].signal = 1;
         if (st.dep2 >= 0) table[st.dep2].signal = 1;
-        st.rows_item = nq::stream_rows_per_item(st.units);
-        st.wg_begin = total_wgs;
-        st.wg_count = (st.rows + st.rows_item - 1) / st.rows_item;
-        total_wgs += st.wg_count;
     }
-    std::vector<int> wg_stage((size_t)total_wgs);
-    for (size_t si = 0; si < table.size(); ++si)
-        for (int w = 0; w < table[si].wg_count; ++w) wg_stage[(size_t)table[si].wg_begin + w] = (int)si;
+
+    // ---- grid = what the device keeps resident; every workgroup gets an equal share of every phase ----
+    int nwg = nq::stream_capacity(dtype, batch, max_units);
+    if (nwg <= 0) return NQ_ERR_HIP;
+    if (nwg > kMaxResidentWorkgroups) nwg = kMaxResidentWorkgroups;
+    std::vector<int> seg_index((size_t)nwg * nphases + 1, 0);
+    std::vector<nq::RunSegment> segs;
+    std::vector<std::vector<int>> by_phase((size_t)nphases);
+    for (int s = 0; s < nstages; ++s) by_phase[table[s].phase].push_back(s);
+    // slices are emitted workgroup-major so that seg_index[wg*nphases + ph] is monotonic
+    std::vector<std::vector<std::vector<nq::RunSegment>>> slice((size_t)nphases);
+    for (int ph = 0; ph < nphases; ++ph) {
+        slice[ph].resize((size_t)nwg);
+        const std::vector<int>& ids = by_phase[ph];
+        std::vector<long long> prefix(ids.size() + 1, 0);
+        for (size_t k = 0; k < ids.size(); ++k)
+            prefix[k + 1] = prefix[k] + (long long)table[ids[k]].rows * table[ids[k]].units;
+        const long long total = prefix.back();
+        // cut point -> (stage position, row): the same mapping is used for a slice's end and the next
+        // slice's begin, so the slices tile every stage exactly
+        auto locate = [&](long long c, size_t& k, int& row) {
+            k = 0;
+            while (k + 1 < ids.size() && prefix[k + 1] <= c) ++k;
+            if (c >= total) { k = ids.size() - 1; row = table[ids[k]].rows; return; }
+            row = (int)((c - prefix[k]) / table[ids[k]].units);
+        };
+        for (int w = 0; w < nwg; ++w) {
+            const long long c0 = total * w / nwg, c1 = total * (w + 1) / nwg;
+            size_t k0, k1; int r0, r1;
+            locate(c0, k0, r0);
+            locate(c1, k1, r1);
+            for (size_t k = k0; k <= k1; ++k) {
+                const int rb = (k == k0) ? r0 : 0;
+                const int re = (k == k1) ? r1 : table[ids[k]].rows;
+                if (re > rb) {
+                    slice[ph][w].push_back(nq::RunSegment{ids[k], rb, re, 0});
+                    table[ids[k]].seg_count += 1;
+                }
+            }
+        }
+    }
+    for (int w = 0; w < nwg; ++w)
+        for (int ph = 0; ph < nphases; ++ph) {
+            seg_index[(size_t)w * nphases + ph] = (int)segs.size();
+            for (const auto& sg : slice[ph][w]) segs.push_back(sg);
+        }
+    seg_index[(size_t)nwg * nphases] = (int)segs.size();
+
+    const size_t off_table = 256 + runlist_counter_bytes(nlinears);
+    const size_t off_index = off_table + runlist_table_bytes(nlinears);
+    const size_t off_segs = off_index + round256(seg_index.size() * sizeof(int));
+    if (off_segs + segs.size() * sizeof(nq::RunSegment) > workspace_bytes) return NQ_ERR_WORKSPACE;
+
     hipStream_t hs = (hipStream_t)stream;
     char* base = (char*)workspace;
-    const size_t off_table = 256 + runlist_counter_bytes(nlinears);
-    const size_t off_map = off_table + runlist_table_bytes(nlinears);
     hipError_t e = hipMemsetAsync(base, 0, off_table, hs);
     if (e != hipSuccess) return hip_status(e);
     e = hipMemcpyAsync(base + off_table, table.data(), table.size() * sizeof(nq::RunStage), hipMemcpyHostToDevice, hs);
     if (e != hipSuccess) return hip_status(e);
-    e = hipMemcpyAsync(base + off_map, wg_stage.data(), wg_stage.size() * sizeof(int), hipMemcpyHostToDevice, hs);
+    e = hipMemcpyAsync(base + off_index, seg_index.data(), seg_index.size() * sizeof(int), hipMemcpyHostToDevice, hs);
+    if (e != hipSuccess) return hip_status(e);
+    e = hipMemcpyAsync(base + off_segs, segs.data(), segs.size() * sizeof(nq::RunSegment), hipMemcpyHostToDevice, hs);
     if (e != hipSuccess) return hip_status(e);
     plan_out->nlinears = nlinears;
-    plan_out->nstages = (int)table.size();
-    plan_out->total_workgroups = total_wgs;
+    plan_out->nstages = nstages;
+    plan_out->nphases = nphases;
+    plan_out->workgroups = nwg;
     plan_out->max_units = max_units;
     plan_out->batch = batch;
     plan_out->dtype = dtype;
-    return hip_status(hipStreamSynchronize(hs));   // `table` is host memory: finish before it dies
+    plan_out->index_words = (int)seg_index.size();
+    return hip_status(hipStreamSynchronize(hs));   // the tables are host memory: finish before they die
 }
 
 int nq_runlist_run(const void* workspace, const nq_runlist_plan* plan, void* stream) {
     if (!workspace || !plan) return NQ_ERR_NULL;
     if (plan->dtype != NQ_F16 && plan->dtype != NQ_BF16) return NQ_ERR_DTYPE;
-    if (plan->nlinears <= 0 || plan->nstages != 2 * plan->nlinears || plan->total_workgroups <= 0 ||
-        plan->max_units <= 0)
+    if (plan->nlinears <= 0 || plan->nstages != 2 * plan->nlinears || plan->workgroups <= 0 || plan->max_units <= 0 ||
+        plan->nphases <= 0 || plan->index_words != plan->workgroups * plan->nphases + 1)
         return NQ_ERR_SHAPE;
     const int batch = plan->batch;
     if (batch != 1 && batch != 2 && batch != 4 && batch != 8 && batch != 16) return NQ_ERR_SHAPE;
     char* base = (char*)workspace;
     const size_t off_table = 256 + runlist_counter_bytes(plan->nlinears);
-    const size_t off_map = off_table + runlist_table_bytes(plan->nlinears);
+    const size_t off_index = off_table + runlist_table_bytes(plan->nlinears);
+    const size_t off_segs = off_index + round256((size_t)plan->index_words * sizeof(int));
     return hip_status(nq::gemv_stream(plan->dtype, batch, (const nq::RunStage*)(base + off_table), plan->nstages,
-                                      (const int*)(base + off_map), (unsigned long long*)(base + 256), (unsigned*)base,
-                                      plan->total_workgroups, plan->max_units, (hipStream_t)stream));
+                                      plan->nphases, (const int*)(base + off_index),
+                                      (const nq::RunSegment*)(base + off_segs), (unsigned long long*)(base + 256),
+                                      (unsigned*)base, plan->workgroups, plan->max_units, (hipStream_t)stream));
 }
 
 int nq_runlist_status(const void* workspace, int* status_out, void* stream) {

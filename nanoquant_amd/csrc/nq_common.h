@@ -63,6 +63,15 @@ struct Elem<1> {
     static __device__ __forceinline__ uint16_t from_float_sat(float f) { return from_float_clamped(f); }
 };
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
+// global load of the wavefront (vmcnt counts loads and stores alike), which would serialise a prefetch
+// that is deliberately kept in flight across the barrier.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // ---- cross-lane sums on a 64-wide wavefront -------------------------------------------------
 // DPP control words (gfx9 encoding): quad_perm = 4 x 2-bit selects; 0x140 row_mirror;
 // 0x141 row_half_mirror.

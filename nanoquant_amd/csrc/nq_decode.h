@@ -55,83 +55,124 @@ __device__ __forceinline__ void stage_units(uint4* xs, float* xsum, const StageI
 #pragma unroll 1
         for (int b = 0; b < BATCH; ++b) {
             const uint32_t* hp = (const uint32_t*)st.in + (size_t)b * st.in_stride;
-            for (int p = threadIdx.x; p < npairs; p += nthreads) {
-                const int col = c0 * 128 + 2 * p;
-                uint32_t lo = 0, hi = 0;
-                if (wide && col + 1 < st.K) {
-                    const uint64_t both = __hip_atomic_load((const uint64_t*)(hp + col), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    lo = (uint32_t)both; hi = (uint32_t)(both >> 32);
-                } else {
-                    if (col < st.K) lo = __hip_atomic_load(hp + col, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if (col + 1 < st.K) hi = __hip_atomic_load(hp + col + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // kBurst loads per lane are put in flight before the first one is consumed: a coherent load is
+            // a round trip to the memory side (~2 us); one round per burst instead of one per pair
+            constexpr int kBurst = 4;
+#pragma unroll 1
+            for (int p0 = threadIdx.x; p0 < npairs; p0 += nthreads * kBurst) {
+                uint32_t lo[kBurst], hi[kBurst];
+#pragma unroll
+                for (int j = 0; j < kBurst; ++j) {
+                    const int p = p0 + j * nthreads;
+                    const int col = c0 * 128 + 2 * p;
+                    lo[j] = 0; hi[j] = 0;
+                    if (p < npairs) {
+                        if (wide && col + 1 < st.K) {
+                            const uint64_t both = __hip_atomic_load((const uint64_t*)(hp + col), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            lo[j] = (uint32_t)both; hi[j] = (uint32_t)(both >> 32);
+                        } else {
+                            if (col < st.K) lo[j] = __hip_atomic_load(hp + col, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            if (col + 1 < st.K) hi[j] = __hip_atomic_load(hp + col + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        }
+                    }
                 }
-                const uint16_t r0 = E::from_float(__builtin_bit_cast(float, lo));
-                const uint16_t r1 = E::from_float(__builtin_bit_cast(float, hi));
-                const int cu = p >> 6, i = (p & 63) >> 2, slot = p & 3;
-                ((uint32_t*)xs)[((b * 16 + i) * upad + cu) * 4 + slot] = (uint32_t)r0 | ((uint32_t)r1 << 16);
-                const float tot = group_sum(E::to_float(r0) + E::to_float(r1), 64);
-                if ((p & 63) == 0) xsum[b * upad + cu] = tot;
+#pragma unroll
+                for (int j = 0; j < kBurst; ++j) {
+                    const int p = p0 + j * nthreads;
+                    if (p < npairs) {      // wave-uniform: npairs and the wave's first p are multiples of 64
+                        const uint16_t r0 = E::from_float(__builtin_bit_cast(float, lo[j]));
+                        const uint16_t r1 = E::from_float(__builtin_bit_cast(float, hi[j]));
+                        const int cu = p >> 6, i = (p & 63) >> 2, slot = p & 3;
+                        ((uint32_t*)xs)[((b * 16 + i) * upad + cu) * 4 + slot] = (uint32_t)r0 | ((uint32_t)r1 << 16);
+                        const float tot = group_sum(E::to_float(r0) + E::to_float(r1), 64);
+                        if ((p & 63) == 0) xsum[b * upad + cu] = tot;
+                    }
+                }
             }
         }
         return;
     }
     const int nchunks = cu_n * 16;
+    constexpr int kBurst = 2;   // chunks whose loads are in flight together
 #pragma unroll 1
     for (int b = 0; b < BATCH; ++b) {
-        for (int q = threadIdx.x; q < nchunks; q += nthreads) {
-            const int cu = q >> 4, i = q & 15;
-            const int col = (c0 + cu) * 128 + i * 8;
-            float v[8];
-            if (st.vec_in && col + 8 <= st.K) {
-                if (!st.in_f32) {
-                    const uint16_t* xp = (const uint16_t*)st.in + (size_t)b * st.in_stride + col;
-                    const uint4 xr = *(const uint4*)xp;
-                    const uint4 sr = st.s_col ? *(const uint4*)(st.s_col + col)
-                                              : make_uint4(E::kOnePair, E::kOnePair, E::kOnePair, E::kOnePair);
+#pragma unroll 1
+        for (int q0 = threadIdx.x; q0 < nchunks; q0 += nthreads * kBurst) {
+            uint4 raw_a[kBurst], raw_b[kBurst];
+            bool fast[kBurst];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const uint32_t xw = comp_d(xr, e), sw = comp_d(sr, e);
-                        v[2 * e] = E::to_float(xw & 0xFFFFu) * E::to_float(sw & 0xFFFFu);
-                        v[2 * e + 1] = E::to_float(xw >> 16) * E::to_float(sw >> 16);
+            for (int j = 0; j < kBurst; ++j) {
+                const int q = q0 + j * nthreads;
+                const int col = (c0 + (q >> 4)) * 128 + (q & 15) * 8;
+                fast[j] = q < nchunks && st.vec_in && col + 8 <= st.K;
+                raw_a[j] = make_uint4(0, 0, 0, 0);
+                raw_b[j] = make_uint4(E::kOnePair, E::kOnePair, E::kOnePair, E::kOnePair);
+                if (fast[j]) {
+                    if (!st.in_f32) {
+                        raw_a[j] = *(const uint4*)((const uint16_t*)st.in + (size_t)b * st.in_stride + col);
+                        if (st.s_col) raw_b[j] = *(const uint4*)(st.s_col + col);
+                    } else {
+                        const float* hp = (const float*)st.in + (size_t)b * st.in_stride + col;
+                        raw_a[j] = *(const uint4*)hp;
+                        raw_b[j] = *(const uint4*)(hp + 4);
                     }
-                } else {
-                    const float* hp = (const float*)st.in + (size_t)b * st.in_stride + col;
-                    const float4 h0 = *(const float4*)hp, h1 = *(const float4*)(hp + 4);
-                    v[0] = h0.x; v[1] = h0.y; v[2] = h0.z; v[3] = h0.w;
-                    v[4] = h1.x; v[5] = h1.y; v[6] = h1.z; v[7] = h1.w;
                 }
-            } else {
+            }
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int c = col + e;
-                    float t = 0.f;
-                    if (c < st.K) {
-                        if (!st.in_f32) {
-                            t = E::to_float(((const uint16_t*)st.in)[(size_t)b * st.in_stride + c]);
-                            if (st.s_col) t *= E::to_float(st.s_col[c]);
-                        } else {
-                            t = ((const float*)st.in)[(size_t)b * st.in_stride + c];
+            for (int j = 0; j < kBurst; ++j) {
+                const int q = q0 + j * nthreads;
+                if (q >= nchunks) continue;               // uniform over each aligned group of 16 lanes
+                const int cu = q >> 4, i = q & 15;
+                const int col = (c0 + cu) * 128 + i * 8;
+                float v[8];
+                if (fast[j]) {
+                    if (!st.in_f32) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint32_t xw = comp_d(raw_a[j], e), sw = comp_d(raw_b[j], e);
+                            v[2 * e] = E::to_float(xw & 0xFFFFu) * E::to_float(sw & 0xFFFFu);
+                            v[2 * e + 1] = E::to_float(xw >> 16) * E::to_float(sw >> 16);
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            v[e] = __builtin_bit_cast(float, comp_d(raw_a[j], e));
+                            v[4 + e] = __builtin_bit_cast(float, comp_d(raw_b[j], e));
                         }
                     }
-                    v[e] = t;
-                }
-            }
-            uint16_t r[8];
-            float tot = 0.f;
+                } else {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                r[e] = E::from_float(v[e]);
-                tot += E::to_float(r[e]);          // the sum of what the dot products will actually see
+                    for (int e = 0; e < 8; ++e) {
+                        const int c = col + e;
+                        float t = 0.f;
+                        if (c < st.K) {
+                            if (!st.in_f32) {
+                                t = E::to_float(((const uint16_t*)st.in)[(size_t)b * st.in_stride + c]);
+                                if (st.s_col) t *= E::to_float(st.s_col[c]);
+                            } else {
+                                t = ((const float*)st.in)[(size_t)b * st.in_stride + c];
+                            }
+                        }
+                        v[e] = t;
+                    }
+                }
+                uint16_t r[8];
+                float tot = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    r[e] = E::from_float(v[e]);
+                    tot += E::to_float(r[e]);          // the sum of what the dot products will actually see
+                }
+                uint4 p;
+                p.x = (uint32_t)r[0] | ((uint32_t)r[1] << 16);
+                p.y = (uint32_t)r[2] | ((uint32_t)r[3] << 16);
+                p.z = (uint32_t)r[4] | ((uint32_t)r[5] << 16);
+                p.w = (uint32_t)r[6] | ((uint32_t)r[7] << 16);
+                xs[(b * 16 + i) * upad + cu] = p;
+                // the 16 chunks of a unit are held by 16 consecutive lanes: finish the unit sum with DPP
+                tot = group_sum(tot, 16);
+                if (i == 0) xsum[b * upad + cu] = tot;
             }
-            uint4 p;
-            p.x = (uint32_t)r[0] | ((uint32_t)r[1] << 16);
-            p.y = (uint32_t)r[2] | ((uint32_t)r[3] << 16);
-            p.z = (uint32_t)r[4] | ((uint32_t)r[5] << 16);
-            p.w = (uint32_t)r[6] | ((uint32_t)r[7] << 16);
-            xs[(b * 16 + i) * upad + cu] = p;
-            // the 16 chunks of a unit are held by 16 consecutive lanes: finish the unit sum with DPP
-            tot = group_sum(tot, 16);
-            if (i == 0) xsum[b * upad + cu] = tot;
         }
     }
 }

@@ -26,16 +26,22 @@ struct RunStage {
     int dep, dep2;          // stage indices that must be complete before `in` / `addend` are read, or -1
     int signal;             // a later stage waits on this one
     int vec_bits, vec_in;
-    int wg_begin, wg_count; // this stage's work items are workgroups [wg_begin, wg_begin + wg_count)
-    int rows_item;          // rows per work item
+    int phase;              // dependency depth: a stage runs after every stage of a lower phase it depends on
+    int seg_count;          // number of workgroup slices this stage is cut into (its completion count)
     int in_coherent;        // fp32 input written by another stage of the same launch
     int heavy_release;      // 16-bit output read by a later stage: full device-scope release on completion
     int heavy_acquire;      // 16-bit input written by an earlier stage: full device-scope acquire after the wait
+    int pad_;
 };
-int stream_rows_per_item(int units);
+// One workgroup's share of one stage: rows [row_begin, row_end).
+struct RunSegment {
+    int stage, row_begin, row_end, pad_;
+};
 size_t stream_counter_bytes(int nstages);
-hipError_t gemv_stream(int dtype, int batch, const RunStage* stages, int nstages, const int* wg_stage,
-                       unsigned long long* counters, unsigned* status, int total_wgs, int max_units, hipStream_t stream);
+int stream_capacity(int dtype, int batch, int max_units);
+hipError_t gemv_stream(int dtype, int batch, const RunStage* stages, int nstages, int nphases, const int* seg_index,
+                       const RunSegment* segs, unsigned long long* counters, unsigned* status, int nwg, int max_units,
+                       hipStream_t stream);
 
 // nq_gemm.hip: C[T,R] = s_out * ((x * s_in) . sgn(W)^T) with W in the 32x256 tile layout.
 // scratch: fp32 [T,R] when gemm_scratch_bytes(T,K,R) > 0.

@@ -29,8 +29,9 @@ class NqLinear(ctypes.Structure):
 
 class NqRunlistPlan(ctypes.Structure):
     """Mirror of `nq_runlist_plan`."""
-    _fields_ = [("nlinears", ctypes.c_int), ("nstages", ctypes.c_int), ("total_workgroups", ctypes.c_int),
-                ("max_units", ctypes.c_int), ("batch", ctypes.c_int), ("dtype", ctypes.c_int)]
+    _fields_ = [("nlinears", ctypes.c_int), ("nstages", ctypes.c_int), ("nphases", ctypes.c_int),
+                ("workgroups", ctypes.c_int), ("max_units", ctypes.c_int), ("batch", ctypes.c_int),
+                ("dtype", ctypes.c_int), ("index_words", ctypes.c_int)]
 
 
 class DecodeRunList:
