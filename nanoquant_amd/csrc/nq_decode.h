@@ -270,4 +270,59 @@ struct UnitDot<1, BATCH> {   // bf16: +-1 operand pairs
     }
 };
 
+// ---- MFMA-assisted unit arithmetic (batch >= 4) -----------------------------------------------------
+// One v_mfma_f32_16x16x32 multiplies a 16-row x 32-column block of +-1 (A operand) with 32 columns x
+// 16 batch rows of staged activations (B operand).  Lane l of the wavefront owns matrix row l & 15 and
+// the column octet l >> 4: its 16 bytes of sign words (one unit of ITS row) feed 16 MFMAs, one per
+// (word, byte) of the unit, because the 8 signs a lane contributes to an MFMA are exactly one byte
+// group of the "half2" order: bits (15-s, 31-s), s = 4*q + c, for the pairs c = 0..3 of quarter q.
+// The four lanes that share a row hold four different units of that row, so a wavefront covers
+// 16 rows x 4 units per fetch and the contraction index of an MFMA is "unit-of-the-lane x octet".
+// The cost per packed bit does not depend on the batch size up to 16.
+template <int DT>
+struct Mfma16;
+template <>
+struct Mfma16<0> {
+    static __device__ __forceinline__ float4_t run(uint4 a, uint4 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+    }
+};
+template <>
+struct Mfma16<1> {
+    static __device__ __forceinline__ float4_t run(uint4 a, uint4 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf168_t, a), __builtin_bit_cast(bf168_t, b), c, 0, 0, 0);
+    }
+};
+
+// sign bits of `shifted` (bits 15 and 31) onto the pair (1.0, 1.0): one v_bfi_b32
+__device__ __forceinline__ uint32_t sign_onto_one(uint32_t shifted, uint32_t one_pair) {
+    uint32_t r;
+    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(r) : "s"(kSignPair), "v"(shifted), "v"(one_pair));
+    return r;
+}
+
+// acc += signs(w: this lane's unit) x staged activations of unit `cu` (zero contribution when !valid).
+// xs row used by this lane: batch row min(lane & 15, BATCH-1); columns beyond BATCH are never read back.
+template <int DT, int BATCH>
+__device__ __forceinline__ void unit_mfma(const uint4& w, const uint4* xs, int upad, int cu, bool valid, float4_t& acc) {
+    using E = Elem<DT>;
+    const int nb = min((int)(threadIdx.x & 15), BATCH - 1);
+    const uint32_t one = E::kOnePair;
+#pragma unroll
+    for (int wi = 0; wi < 4; ++wi) {
+        const uint32_t word = comp_d(w, wi);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            uint4 a;
+            a.x = sign_onto_one(word << (4 * q + 0), one);
+            a.y = sign_onto_one(word << (4 * q + 1), one);
+            a.z = sign_onto_one(word << (4 * q + 2), one);
+            a.w = sign_onto_one(word << (4 * q + 3), one);
+            uint4 b = make_uint4(0, 0, 0, 0);
+            if (valid) b = xs[(nb * 16 + 4 * wi + q) * upad + cu];
+            acc = Mfma16<DT>::run(a, b, acc);
+        }
+    }
+}
+
 }  // namespace nq

@@ -67,7 +67,7 @@ __device__ __forceinline__ uint4 load_unit(const RunStage& st, int row, int unit
     return w;
 }
 
-template <int DT, int BATCH>
+template <int DT, int BATCH, bool MFMA>
 __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(const RunStage* __restrict__ stages, int nstages,
                                                                      int nphases, const int* __restrict__ seg_index,
                                                                      const RunSegment* __restrict__ segs,
@@ -114,7 +114,11 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(const RunSt
 
             // First fetch of the slice, issued before any wait: the weights are always ready.
             uint4 wnext = make_uint4(0, 0, 0, 0);
-            {
+            if constexpr (MFMA) {
+                // lane (row l & 15, octet l >> 4) of wavefront w starts with unit 4*w + (l >> 4) of its row
+                const int u0 = 4 * (tid >> 6) + ((tid & 63) >> 4);
+                if (u0 < chunk_units) wnext = load_unit(st, min(seg.row_begin + (tid & 15), st.rows - 1), u0);
+            } else {
                 const int nr0 = min(seg.row_end - seg.row_begin, kRowBlock);
                 if (tid < nr0 * chunk_units) wnext = load_unit(st, seg.row_begin + tid / chunk_units, tid % chunk_units);
             }
@@ -174,27 +178,56 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(const RunSt
                             staged = true;
                         }
                         lds_barrier();                           // xs / xsum / zeroed racc visible
-                        const int total = nr * cu_n;
-                        int row_l = tid / cu_n, cu = tid % cu_n;
-                        const int srow = kStreamThreads / cu_n, scu = kStreamThreads % cu_n;
-                        uint4 w = wnext;                         // first block, chunk 0: fetched before the wait
-                        if ((rb != seg.row_begin || c0 != 0) && tid < total) w = load_unit(st, rb + row_l, c0 + cu);
+                        if constexpr (MFMA) {
+                            const int lane = tid & 63, wave = tid >> 6, r16 = lane & 15, g = lane >> 4;
+                            const int ngroups = (cu_n + 3) >> 2;          // unit groups of 4; wavefront w takes w, w+4, ...
 #pragma unroll 1
-                        for (int f = tid; f < total; f += kStreamThreads) {
-                            // next unit of this lane: put its fetch in flight before the arithmetic
-                            int nrow = row_l + srow, ncu = cu + scu;
-                            if (ncu >= cu_n) { ncu -= cu_n; ++nrow; }
-                            uint4 wpre = make_uint4(0, 0, 0, 0);
-                            if (f + kStreamThreads < total) wpre = load_unit(st, rb + nrow, c0 + ncu);
-                            float part[BATCH];
-                            UnitDot<DT, BATCH>::run(w, xs, xsum, upad, cu, part);
+                            for (int rg = 0; rg < nr; rg += 16) {
+                                const int row = min(rb + rg + r16, st.rows - 1);
+                                float4_t acc = {0.f, 0.f, 0.f, 0.f};
+                                uint4 w = wnext;                         // very first fetch of the slice
+                                if (rb != seg.row_begin || c0 != 0 || rg != 0) {
+                                    w = make_uint4(0, 0, 0, 0);
+                                    if (4 * wave + g < cu_n) w = load_unit(st, row, c0 + 4 * wave + g);
+                                }
+#pragma unroll 1
+                                for (int ub = wave; ub < ngroups; ub += 4) {
+                                    const int u = 4 * ub + g;
+                                    uint4 wpre = make_uint4(0, 0, 0, 0);
+                                    if (ub + 4 < ngroups && u + 16 < cu_n) wpre = load_unit(st, row, c0 + u + 16);
+                                    unit_mfma<DT, BATCH>(w, xs, upad, u, u < cu_n, acc);
+                                    w = wpre;
+                                }
+                                // acc[v] = partial sum of row rg + 4*g + v for batch row r16
+                                if (r16 < BATCH) {
 #pragma unroll
-                            for (int b = 0; b < BATCH; ++b) atomicAdd(&racc[row_l * BATCH + b], part[b]);
-                            w = wpre;
-                            row_l = nrow;
-                            cu = ncu;
+                                    for (int v = 0; v < 4; ++v)
+                                        if (rg + 4 * g + v < nr) atomicAdd(&racc[(rg + 4 * g + v) * BATCH + r16], acc[v]);
+                                }
+                            }
+                        } else {
+                            const int total = nr * cu_n;
+                            int row_l = tid / cu_n, cu = tid % cu_n;
+                            const int srow = kStreamThreads / cu_n, scu = kStreamThreads % cu_n;
+                            uint4 w = wnext;                         // first block, chunk 0: fetched before the wait
+                            if ((rb != seg.row_begin || c0 != 0) && tid < total) w = load_unit(st, rb + row_l, c0 + cu);
+    #pragma unroll 1
+                            for (int f = tid; f < total; f += kStreamThreads) {
+                                // next unit of this lane: put its fetch in flight before the arithmetic
+                                int nrow = row_l + srow, ncu = cu + scu;
+                                if (ncu >= cu_n) { ncu -= cu_n; ++nrow; }
+                                uint4 wpre = make_uint4(0, 0, 0, 0);
+                                if (f + kStreamThreads < total) wpre = load_unit(st, rb + nrow, c0 + ncu);
+                                float part[BATCH];
+                                UnitDot<DT, BATCH>::run(w, xs, xsum, upad, cu, part);
+    #pragma unroll
+                                for (int b = 0; b < BATCH; ++b) atomicAdd(&racc[row_l * BATCH + b], part[b]);
+                                w = wpre;
+                                row_l = nrow;
+                                cu = ncu;
+                            }
                         }
-                    }
+                        }
                     lds_barrier();                               // row sums complete
                     for (int i = tid; i < nr * BATCH; i += kStreamThreads) {
                         const int row = rb + i / BATCH, b = i % BATCH;
@@ -260,10 +293,17 @@ static void stream_lds_plan(int batch, int max_units, int* chunk_cap_out, size_t
 }
 
 template <int DT, int BATCH>
+struct StreamKernel {
+    // batches of 4 and more go through the MFMA units; 1 and 2 stay matmul-free
+    static constexpr bool kMfma = BATCH >= 4;
+    static constexpr auto fn = gemv_stream_kernel<DT, BATCH, kMfma>;
+};
+
+template <int DT, int BATCH>
 static hipError_t prepare_kernel(size_t lds) {
     static bool attr_done = false;
     if (lds > 64 * 1024 && !attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemv_stream_kernel<DT, BATCH>,
+        hipError_t e = hipFuncSetAttribute((const void*)StreamKernel<DT, BATCH>::fn,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
         if (e != hipSuccess) return e;
         attr_done = true;
@@ -278,7 +318,7 @@ static int capacity_of(int max_units) {
     stream_lds_plan(BATCH, max_units, &chunk_cap, &lds);
     if (prepare_kernel<DT, BATCH>(lds) != hipSuccess) return 0;
     int per_cu = 0, dev = 0, cus = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)gemv_stream_kernel<DT, BATCH>, kStreamThreads,
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)StreamKernel<DT, BATCH>::fn, kStreamThreads,
                                                      lds) != hipSuccess)
         return 0;
     if (hipGetDevice(&dev) != hipSuccess) return 0;
@@ -304,7 +344,7 @@ static hipError_t launch_stream(const RunStage* stages, int nstages, int nphases
         (void)hipMemcpyToSymbol(HIP_SYMBOL(g_nq_trace), &tbuf, sizeof(tbuf));
     }
 #endif
-    hipLaunchKernelGGL((gemv_stream_kernel<DT, BATCH>), dim3(nwg), dim3(kStreamThreads), lds, stream, stages, nstages,
+    hipLaunchKernelGGL((gemv_stream_kernel<DT, BATCH, StreamKernel<DT, BATCH>::kMfma>), dim3(nwg), dim3(kStreamThreads), lds, stream, stages, nstages,
                        nphases, seg_index, segs, counters, status, (unsigned)(1u << 21), chunk_cap);
 #ifdef NQ_TRACE
     if (tbuf && ++calls == 40) {
