@@ -127,7 +127,9 @@ int nq_gemv_stage(const void* in, const void* s_col, const uint32_t* bits, const
  *   layout is private to packer and kernel, as the reference's Marlin layout is).
  *   Requires k % 256 == 0 and rows % 32 == 0 (else NQ_ERR_PROB_SHAPE, the reference's error class
  *   for shapes its tiles do not cover).  scratch: nq_gemm_scratch_bytes(tokens, k, rows) bytes of
- *   device memory (may be NULL when that is 0); it holds fp32 partial sums when k is split. */
+ *   device memory (may be NULL when that is 0).  It holds fp32 partial sums and tile counters when k
+ *   is split; it MUST BE ZERO ON ENTRY and is zero again when the enqueued work has finished, so a
+ *   caller zeroes it once and reuses it (calls sharing a scratch must not overlap in time). */
 size_t nq_gemm_scratch_bytes(int tokens, int k, int rows);
 int nq_gemm_onebit(const void* x, const uint32_t* tiles, const void* s_in, const void* s_out, void* y,
                    void* scratch, size_t scratch_bytes, int tokens, int k, int rows, int dtype, void* stream);

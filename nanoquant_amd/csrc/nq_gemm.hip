@@ -16,7 +16,7 @@
 // Work split: grid.x = 128-row blocks (4 wavefronts x 32 rows), grid.y = token blocks of 32*TT,
 // grid.z = k-splits.  With one k-split the epilogue scales and stores directly; otherwise partial
 // sums are added into an fp32 scratch with hardware float atomics and a small second kernel scales
-// and converts.
+// and converts (and re-zeroes the scratch, which must be zero on entry).
 #include "nq_common.h"
 #include "nq_kernels.h"
 
@@ -146,17 +146,15 @@ __global__ __launch_bounds__(256) void gemm_onebit_kernel(GemmArgs a) {
     }
 }
 
-__global__ __launch_bounds__(256) void zero_f32_kernel(float4* p, size_t n4) {
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-}
-
+// Scales, converts and stores the accumulated sums, and puts the accumulator back to zero: the scratch
+// is zero on entry of every GEMM call and zero again when the call has finished.
 template <int DT>
-__global__ __launch_bounds__(256) void gemm_finish_kernel(const float4* acc, const uint16_t* s_out, uint16_t* y, int R, size_t n4) {
+__global__ __launch_bounds__(256) void gemm_finish_kernel(float4* acc, const uint16_t* s_out, uint16_t* y, int R, size_t n4) {
     using E = Elem<DT>;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
         const float4 v = acc[i];
+        acc[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         const int row = (int)((i * 4) % (size_t)R);   // R % 4 == 0, so the 4 values share a token
         float s0 = 1.f, s1 = 1.f, s2 = 1.f, s3 = 1.f;
         if (s_out) {
@@ -213,10 +211,9 @@ static hipError_t launch_gemm(const GemmArgs& a, const GemmPlan& p, hipStream_t 
         const size_t n4 = (size_t)a.T * a.R / 4;
         size_t zb = (n4 + 255) / 256;
         if (zb > 2048) zb = 2048;
-        hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)zb), dim3(256), 0, stream, (float4*)a.acc, n4);
         hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);
-        hipLaunchKernelGGL(gemm_finish_kernel<DT>, dim3((unsigned)zb), dim3(256), 0, stream, (const float4*)a.acc,
-                           a.s_out, (uint16_t*)a.y, a.R, n4);
+        hipLaunchKernelGGL(gemm_finish_kernel<DT>, dim3((unsigned)zb), dim3(256), 0, stream, (float4*)a.acc, a.s_out,
+                           (uint16_t*)a.y, a.R, n4);
     } else {
         auto kern = gemm_onebit_kernel<DT, TT, false>;
         static bool attr_done = false;
@@ -230,7 +227,8 @@ static hipError_t launch_gemm(const GemmArgs& a, const GemmPlan& p, hipStream_t 
     return hipGetLastError();
 }
 
-// Shapes must satisfy K % 256 == 0 and R % 32 == 0 (checked by the caller).
+// Shapes must satisfy K % 256 == 0 and R % 32 == 0 (checked by the caller).  `scratch` (when
+// gemm_scratch_bytes > 0) must be zero on entry and is zero again when the enqueued work has finished.
 hipError_t gemm_onebit(int dtype, const void* x, const uint32_t* tiles, const void* s_in, const void* s_out,
                        void* y, float* scratch, int T, int K, int R, hipStream_t stream) {
     GemmArgs a;

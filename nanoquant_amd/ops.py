@@ -195,11 +195,21 @@ def _check_gemm_tensor(t, name, dtype=None):
         raise RuntimeError(f"{name} must have dtype {dtype}")
 
 
-def _scratch(tokens, k, rows, device):
-    nbytes = int(_lib.lib().nq_gemm_scratch_bytes(tokens, k, rows))
+# Split-k scratch (fp32 partial sums + tile counters).  The kernels require it to be zero on entry and
+# leave it zero on exit, so one buffer per (device, stream) is allocated zeroed once, grown on demand and
+# reused; no per-call memset.
+_scratch_cache = {}
+
+
+def _scratch(nbytes, device):
     if nbytes == 0:
-        return None, 0
-    return torch.empty(nbytes // 4, dtype=torch.float32, device=device), nbytes
+        return None
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    buf = _scratch_cache.get(key)
+    if buf is None or buf.numel() * 4 < nbytes:
+        buf = torch.zeros((nbytes + 3) // 4, dtype=torch.float32, device=device)
+        _scratch_cache[key] = buf
+    return buf
 
 
 def marlin_onebit_forward(x, weight, scale_g, scale_h, workspace):
@@ -213,7 +223,8 @@ def marlin_onebit_forward(x, weight, scale_g, scale_h, workspace):
     C = torch.empty((m, n), dtype=x.dtype, device=x.device)
     if m == 0 or n == 0:
         return C
-    scratch, nbytes = _scratch(m, k, n, x.device)
+    nbytes = int(_lib.lib().nq_gemm_scratch_bytes(m, k, n))
+    scratch = _scratch(nbytes, x.device)
     with torch.cuda.device(x.device):
         _lib.check(_lib.lib().nq_gemm_onebit(_ptr(x), _ptr(weight), _ptr(scale_g), _ptr(scale_h), _ptr(C),
                                              _ptr(scratch), nbytes, m, k, n, dt, _stream(x.device)))
@@ -240,9 +251,8 @@ def marlin_nanoquant_forward(x, weight_u, weight_v, scale_g, scale_l, scale_h, w
     out = torch.empty((t, m), dtype=x.dtype, device=x.device)
     if t == 0 or m == 0:
         return out
-    s1, b1 = _scratch(t, n, r, x.device)
-    s2, b2 = _scratch(t, r, m, x.device)
-    scratch, nbytes = (s1, b1) if b1 >= b2 else (s2, b2)
+    nbytes = max(int(_lib.lib().nq_gemm_scratch_bytes(t, n, r)), int(_lib.lib().nq_gemm_scratch_bytes(t, r, m)))
+    scratch = _scratch(nbytes, x.device)
     with torch.cuda.device(x.device):
         _lib.check(_lib.lib().nq_gemm_nanoquant(_ptr(x), _ptr(weight_u), _ptr(weight_v), _ptr(scale_g), _ptr(scale_l),
                                                 _ptr(scale_h), _ptr(imm), _ptr(out), _ptr(scratch), nbytes,
