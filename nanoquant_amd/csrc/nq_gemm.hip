@@ -8,9 +8,10 @@
 // wavefront fetches one tile with a single 128-bit load per lane and expands it in registers: the
 // 8 k-values a lane feeds to v_mfma_f32_32x32x16 are one byte of its 16, and `(word << s) &
 // 0x80008000 | (1.0, 1.0)` turns two of those bits into a +-1 pair, so the B operand is built with
-// integer logic only.  Activations (scaled by s_in while staging) are the A operand and come from an
-// LDS slab shared by the four wavefronts of a workgroup; accumulation is fp32 in the MFMA
-// accumulators.  With A = activations the result registers of a lane run along the output row index,
+// integer logic only.  With an input scale the operand is +-s_in[k] instead of +-1 (the scale pair
+// XOR the sign bits), so x * s_in is formed exactly inside the MFMA and staging stays a plain copy.
+// Activations are the A operand and come from an LDS slab shared by the four wavefronts of a
+// workgroup; accumulation is fp32 in the MFMA accumulators.  With A = activations the result registers of a lane run along the output row index,
 // which makes the epilogue stores contiguous.
 //
 // Work split: grid.x = 128-row blocks (4 wavefronts x 32 rows), grid.y = token blocks of 32*TT,
@@ -32,10 +33,17 @@ struct GemmArgs {
     int T, K, R;
     int ktiles;             // K / 256
     int ktiles_per_split;
+    int xcd_gx;             // > 0: flat grid, token blocks dealt to the 8 XCDs; value = row blocks
 };
 
-constexpr int kSlabK = 256;
-constexpr int kPitch = kSlabK + 8;  // 16-bit elements per LDS row: 528 bytes, conflict-free b128 reads
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kTileK = 256;  // k extent of one packed weight tile (and the granularity of k-splits)
+
+// LDS row pitch in 16-bit elements for a slab of KS k-values: 16 bytes of padding make the 128-bit
+// fragment reads of 32 consecutive rows conflict-free.
+template <int KS>
+constexpr int slab_pitch() { return KS + 8; }
 
 template <int DT>
 struct Mfma;
@@ -56,91 +64,149 @@ __device__ __forceinline__ uint32_t comp4(const uint4& v, int i) {
     return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
 }
 
-template <int DT, int TT, bool SPLIT>
+// Issues the global loads of one activation slab [32*TT tokens][KS k] starting at k0 (and its KS input
+// scales) into registers; nothing waits on them here.
+template <int TT, int KS, bool SCALED>
+__device__ __forceinline__ void fetch_slab(const GemmArgs& a, int tok0, int k0, u32x4_t (&xr)[TT * KS / 64], uint32_t& sr) {
+    constexpr int kChunks = KS / 8;   // 16-byte chunks per token row
+#pragma unroll
+    for (int pass = 0; pass < TT * KS / 64; ++pass) {
+        const int q = pass * 256 + threadIdx.x;
+        // rows beyond T repeat the last token; their results are never stored
+        const int tok = min(tok0 + q / kChunks, a.T - 1), c8 = (q % kChunks) * 8;
+        xr[pass] = *(const u32x4_t*)((const uint16_t*)a.x + (size_t)tok * a.K + k0 + c8);
+    }
+    if constexpr (SCALED) {
+        if (threadIdx.x < KS / 2) sr = *(const uint32_t*)(a.s_in + k0 + 2 * threadIdx.x);
+    }
+}
+
+// TT: 32-token tiles per wavefront, RT: 32-row tiles per wavefront, KS: k-values per LDS slab (128 or
+// 256).  A workgroup of 4 wavefronts covers 32*TT tokens x 128*RT rows.
+template <int DT, int TT, int RT, int KS, bool SPLIT, bool SCALED>
 __global__ __launch_bounds__(256) void gemm_onebit_kernel(GemmArgs a) {
     using E = Elem<DT>;
-    extern __shared__ uint16_t slab[];  // [32*TT][kPitch]
+    constexpr int kPitch = slab_pitch<KS>();
+    constexpr int kSubs = kTileK / KS;       // slabs per weight tile
+    constexpr int kPasses = TT * KS / 64;    // 16-byte chunks each thread stages per slab
+    extern __shared__ uint16_t slab[];       // [32*TT][kPitch], then the KS input scales of the slab
+    uint16_t* scale_lds = slab + 32 * TT * kPitch;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int rt = blockIdx.x * 4 + wave;          // 32-row tile of this wavefront
+    // Workgroups go to the 8 XCDs round-robin by linear id.  With the flat grid every XCD owns the token
+    // blocks y = xcd (mod 8), so the workgroups that share an activation slab also share an L2.
+    int bx = blockIdx.x, by = blockIdx.y;
+    if (a.xcd_gx > 0) {
+        const int slot = blockIdx.x >> 3;
+        by = (slot / a.xcd_gx) * 8 + (blockIdx.x & 7);
+        bx = slot % a.xcd_gx;
+        if (by * (32 * TT) >= a.T) return;
+    }
+    const int rt = (bx * 4 + wave) * RT;           // first of the RT 32-row tiles of this wavefront
     const bool have_rows = rt * 32 < a.R;
-    const int tok0 = blockIdx.y * (32 * TT);
+    const int ntiles = min(RT, a.R / 32 - rt);     // R % 32 == 0
+    const int tok0 = by * (32 * TT);
     const int kt_begin = blockIdx.z * a.ktiles_per_split;
     const int kt_end = min(kt_begin + a.ktiles_per_split, a.ktiles);
 
-    float16_t acc[TT];
+    float16_t acc[RT][TT];
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt)
+    for (int r = 0; r < RT; ++r)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[tt][v] = 0.f;
+        for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[r][tt][v] = 0.f;
 
     const uint4* tile_ptr = a.tiles + ((size_t)rt * a.ktiles + kt_begin) * 64 + lane;
-    uint4 wnext = make_uint4(0, 0, 0, 0);
-    if (have_rows && kt_begin < kt_end) wnext = *tile_ptr;
+    const size_t tile_pitch = (size_t)a.ktiles * 64;   // uint4 elements between consecutive row tiles
+    uint4 wnext[RT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+        wnext[r] = make_uint4(0, 0, 0, 0);
+        if (r < ntiles && kt_begin < kt_end) wnext[r] = tile_ptr[r * tile_pitch];
+    }
+
+    // The next slab travels global -> registers while the MFMAs of the current one run, and registers
+    // -> LDS between the two barriers at the top of the next step.
+    u32x4_t xr[kPasses];
+    uint32_t sr = 0;
+    if (kt_begin < kt_end) fetch_slab<TT, KS, SCALED>(a, tok0, kt_begin * kTileK, xr, sr);
 
 #pragma unroll 1
     for (int kt = kt_begin; kt < kt_end; ++kt) {
-        // ---- stage the activation slab [32*TT tokens][256 k], scaled by s_in, zero beyond T ----
-        if (kt != kt_begin) __syncthreads();
-        const int k0 = kt * kSlabK;
+        uint4 w[RT];
 #pragma unroll
-        for (int pass = 0; pass < TT * 4; ++pass) {
-            const int q = pass * 256 + threadIdx.x;   // 16-byte chunk id: 32 chunks per token row
-            const int trow = q >> 5, c8 = (q & 31) * 8;
-            const int tok = tok0 + trow;
-            uint4 xv = make_uint4(0, 0, 0, 0);
-            if (tok < a.T) {
-                xv = *(const uint4*)((const uint16_t*)a.x + (size_t)tok * a.K + k0 + c8);
-                if (a.s_in) {
-                    const uint4 sv = *(const uint4*)(a.s_in + k0 + c8);
-                    uint32_t o[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const uint32_t xw = comp4(xv, e), sw = comp4(sv, e);
-                        const float lo = E::to_float(xw & 0xFFFFu) * E::to_float(sw & 0xFFFFu);
-                        const float hi = E::to_float(xw >> 16) * E::to_float(sw >> 16);
-                        o[e] = (uint32_t)E::from_float(lo) | ((uint32_t)E::from_float(hi) << 16);
-                    }
-                    xv = make_uint4(o[0], o[1], o[2], o[3]);
-                }
-            }
-            *(uint4*)(slab + trow * kPitch + c8) = xv;
+        for (int r = 0; r < RT; ++r) {
+            w[r] = wnext[r];
+            if (r < ntiles && kt + 1 < kt_end) wnext[r] = tile_ptr[r * tile_pitch + (size_t)(kt + 1 - kt_begin) * 64];
         }
-        const uint4 w = wnext;
-        if (have_rows && kt + 1 < kt_end) wnext = tile_ptr[(size_t)(kt + 1 - kt_begin) * 64];
-        __syncthreads();
-
-        if (have_rows) {
 #pragma unroll
-            for (int t = 0; t < 16; ++t) {
-                const uint32_t word = comp4(w, t >> 2);
-                const int s = 4 * (t & 3);
-                uint4 bfrag;
-                bfrag.x = ((word << (s + 0)) & kSignPair) | E::kOnePair;
-                bfrag.y = ((word << (s + 1)) & kSignPair) | E::kOnePair;
-                bfrag.z = ((word << (s + 2)) & kSignPair) | E::kOnePair;
-                bfrag.w = ((word << (s + 3)) & kSignPair) | E::kOnePair;
+        for (int sub = 0; sub < kSubs; ++sub) {
+            if (sub != 0 || kt != kt_begin) __syncthreads();
+#pragma unroll
+            for (int pass = 0; pass < kPasses; ++pass) {
+                const int q = pass * 256 + threadIdx.x;
+                *(u32x4_t*)(slab + (q / (KS / 8)) * kPitch + (q % (KS / 8)) * 8) = xr[pass];
+            }
+            if constexpr (SCALED) {
+                if (threadIdx.x < KS / 2) *(uint32_t*)(scale_lds + 2 * threadIdx.x) = sr;
+            }
+            __syncthreads();
+            if (sub + 1 < kSubs) fetch_slab<TT, KS, SCALED>(a, tok0, kt * kTileK + (sub + 1) * KS, xr, sr);
+            else if (kt + 1 < kt_end) fetch_slab<TT, KS, SCALED>(a, tok0, (kt + 1) * kTileK, xr, sr);
+
+            // wavefronts beyond the last row tile run on zero words; nothing of theirs is stored
+#pragma unroll
+            for (int t = 0; t < KS / 16; ++t) {
+                const int tg = sub * (KS / 16) + t;   // 16-k step within the weight tile
+                const int s = 4 * (tg & 3);
+                uint4 sp;
+                if constexpr (SCALED) sp = *(const uint4*)(scale_lds + 16 * t + 8 * (lane >> 5));   // broadcast read
+                uint4 bfrag[RT];
+#pragma unroll
+                for (int r = 0; r < RT; ++r) {
+                    const uint32_t word = comp4(w[r], tg >> 2);
+                    if constexpr (SCALED) {
+                        // +-s_in[k]: the scale pair with its sign bits flipped by the packed bits, so that
+                        // x * s_in is formed exactly inside the MFMA (the reference folds s_in into its
+                        // dequantised fragment the same way, gemm_kernel.cu:231-237)
+                        bfrag[r].x = sp.x ^ ((word << (s + 0)) & kSignPair);
+                        bfrag[r].y = sp.y ^ ((word << (s + 1)) & kSignPair);
+                        bfrag[r].z = sp.z ^ ((word << (s + 2)) & kSignPair);
+                        bfrag[r].w = sp.w ^ ((word << (s + 3)) & kSignPair);
+                    } else {
+                        bfrag[r].x = ((word << (s + 0)) & kSignPair) | E::kOnePair;
+                        bfrag[r].y = ((word << (s + 1)) & kSignPair) | E::kOnePair;
+                        bfrag[r].z = ((word << (s + 2)) & kSignPair) | E::kOnePair;
+                        bfrag[r].w = ((word << (s + 3)) & kSignPair) | E::kOnePair;
+                    }
+                }
 #pragma unroll
                 for (int tt = 0; tt < TT; ++tt) {
                     const uint4 afrag = *(const uint4*)(slab + (tt * 32 + (lane & 31)) * kPitch + 16 * t + 8 * (lane >> 5));
-                    acc[tt] = Mfma<DT>::run(afrag, bfrag, acc[tt]);
+#pragma unroll
+                    for (int r = 0; r < RT; ++r) acc[r][tt] = Mfma<DT>::run(afrag, bfrag[r], acc[r][tt]);
                 }
             }
         }
     }
 
     if (!have_rows) return;
-    const int row = rt * 32 + (lane & 31);
-    float sc = 1.f;
-    if (!SPLIT && a.s_out) sc = E::to_float(a.s_out[row]);
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt) {
+    for (int r = 0; r < RT; ++r) {
+        if (r >= ntiles) break;
+        const int row = (rt + r) * 32 + (lane & 31);
+        float sc = 1.f;
+        if (!SPLIT && a.s_out) sc = E::to_float(a.s_out[row]);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int tok = tok0 + tt * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-            if (tok < a.T) {
-                const size_t o = (size_t)tok * a.R + row;
-                if (SPLIT) atomicAdd(a.acc + o, acc[tt][v]);
-                else ((uint16_t*)a.y)[o] = E::from_float_sat(acc[tt][v] * sc);
+        for (int tt = 0; tt < TT; ++tt) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int tok = tok0 + tt * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                if (tok < a.T) {
+                    const size_t o = (size_t)tok * a.R + row;
+                    if (SPLIT) atomicAdd(a.acc + o, acc[r][tt][v]);
+                    else ((uint16_t*)a.y)[o] = E::from_float_sat(acc[r][tt][v] * sc);
+                }
             }
         }
     }
@@ -171,17 +237,21 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(float4* acc, const uin
 // ---- host side --------------------------------------------------------------------------------
 struct GemmPlan {
     int tt;       // 32-token tiles per wavefront
+    int rt;       // 32-row tiles per wavefront
     int gx, gy, ksplit, ktiles_per_split;
+    bool xcd;     // flat, XCD-aware grid
 };
 
 static GemmPlan plan_gemm(int T, int K, int R) {
     GemmPlan p;
-    // 64-token blocks measured faster than 128-token blocks at 128 and 512 tokens alike: twice the
-    // workgroups, half the slab to stage between barriers.
+    // 64-token blocks measured faster than 128-token blocks at every token count tried (128 .. 4096):
+    // more workgroups, fewer registers, three wavefronts per SIMD.  Two row tiles per wavefront halve the
+    // LDS reads per MFMA and win once that still leaves two workgroups for every CU.
     p.tt = 2;
-    p.gx = (R + 127) / 128;
     p.gy = (T + 32 * p.tt - 1) / (32 * p.tt);
-    const int ktiles = K / kSlabK;
+    p.rt = ((R + 255) / 256) * p.gy >= 512 ? 2 : 1;
+    p.gx = (R + 128 * p.rt - 1) / (128 * p.rt);
+    const int ktiles = K / kTileK;
     int want = 512 / (p.gx * p.gy);          // k-splits needed to put two workgroups on every CU
     if (want < 1) want = 1;
     int max_split = ktiles / 2;              // keep at least 512 k per split
@@ -189,42 +259,50 @@ static GemmPlan plan_gemm(int T, int K, int R) {
     int ks = want < max_split ? want : max_split;
     p.ktiles_per_split = (ktiles + ks - 1) / ks;
     p.ksplit = (ktiles + p.ktiles_per_split - 1) / p.ktiles_per_split;
+    // the XCD-aware flat grid needs token blocks in multiples of 8 (or many of them) to stay balanced
+    p.xcd = p.ksplit == 1 && (p.gy % 8 == 0 || p.gy >= 32);
     return p;
 }
 
 size_t gemm_scratch_bytes(int T, int K, int R) {
-    if (T <= 0 || K <= 0 || R <= 0 || K % kSlabK != 0) return 0;
+    if (T <= 0 || K <= 0 || R <= 0 || K % kTileK != 0) return 0;
     const GemmPlan p = plan_gemm(T, K, R);
     return p.ksplit > 1 ? (size_t)T * R * sizeof(float) : 0;
 }
 
-template <int DT, int TT>
+template <int DT, int TT, int RT, int KS, bool SPLIT, bool SCALED>
+static hipError_t launch_variant(const GemmArgs& a, dim3 grid, size_t lds, hipStream_t stream) {
+    auto kern = gemm_onebit_kernel<DT, TT, RT, KS, SPLIT, SCALED>;
+    static bool attr_done = false;
+    if (lds > 64 * 1024 && !attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);
+    return hipSuccess;
+}
+
+template <int DT, int TT, int RT, int KS>
 static hipError_t launch_gemm(const GemmArgs& a, const GemmPlan& p, hipStream_t stream) {
-    const size_t lds = (size_t)32 * TT * kPitch * sizeof(uint16_t);
+    const size_t lds = ((size_t)32 * TT * slab_pitch<KS>() + KS) * sizeof(uint16_t);
     dim3 grid(p.gx, p.gy, p.ksplit);
+    if (p.xcd) grid = dim3(p.gx * ((p.gy + 7) / 8 * 8), 1, 1);
+    const bool scaled = a.s_in != nullptr;
+    hipError_t e;
     if (p.ksplit > 1) {
-        auto kern = gemm_onebit_kernel<DT, TT, true>;
-        static bool attr_done = false;
-        if (lds > 64 * 1024 && !attr_done) {
-            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return e;
-            attr_done = true;
-        }
+        e = scaled ? launch_variant<DT, TT, RT, KS, true, true>(a, grid, lds, stream)
+                   : launch_variant<DT, TT, RT, KS, true, false>(a, grid, lds, stream);
+        if (e != hipSuccess) return e;
         const size_t n4 = (size_t)a.T * a.R / 4;
         size_t zb = (n4 + 255) / 256;
         if (zb > 2048) zb = 2048;
-        hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);
         hipLaunchKernelGGL(gemm_finish_kernel<DT>, dim3((unsigned)zb), dim3(256), 0, stream, (float4*)a.acc, a.s_out,
                            (uint16_t*)a.y, a.R, n4);
     } else {
-        auto kern = gemm_onebit_kernel<DT, TT, false>;
-        static bool attr_done = false;
-        if (lds > 64 * 1024 && !attr_done) {
-            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return e;
-            attr_done = true;
-        }
-        hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);
+        e = scaled ? launch_variant<DT, TT, RT, KS, false, true>(a, grid, lds, stream)
+                   : launch_variant<DT, TT, RT, KS, false, false>(a, grid, lds, stream);
+        if (e != hipSuccess) return e;
     }
     return hipGetLastError();
 }
@@ -238,11 +316,12 @@ hipError_t gemm_onebit(int dtype, const void* x, const uint32_t* tiles, const vo
     a.s_in = (const uint16_t*)s_in; a.s_out = (const uint16_t*)s_out;
     a.y = y; a.acc = scratch;
     a.T = T; a.K = K; a.R = R;
-    a.ktiles = K / kSlabK;
+    a.ktiles = K / kTileK;
     const GemmPlan p = plan_gemm(T, K, R);
     a.ktiles_per_split = p.ktiles_per_split;
-    if (dtype == 0) return p.tt == 2 ? launch_gemm<0, 2>(a, p, stream) : launch_gemm<0, 4>(a, p, stream);
-    return p.tt == 2 ? launch_gemm<1, 2>(a, p, stream) : launch_gemm<1, 4>(a, p, stream);
+    a.xcd_gx = p.xcd ? p.gx : 0;
+    if (dtype == 0) return p.rt == 2 ? launch_gemm<0, 2, 2, 256>(a, p, stream) : launch_gemm<0, 2, 1, 256>(a, p, stream);
+    return p.rt == 2 ? launch_gemm<1, 2, 2, 256>(a, p, stream) : launch_gemm<1, 2, 1, 256>(a, p, stream);
 }
 
 }  // namespace nq
