@@ -7,8 +7,8 @@ batch 1, fp16 activations.  One "step" is one pass over the 7 linears of the lay
 walk over distinct copies of the layer's weights (more than the 256 MB Infinity Cache in total), so
 the packed words come from HBM, not from cache.  `value` is algorithmic bytes / time.
 
-Prints ONE JSON line.  Extra keys report the same layer at batch 4 and 16 and the 128-token prefill
-GEMM; `roofline` is for the decode kernel, `cpu_baseline` is the reference's dense CPU path (two
+Prints ONE JSON line.  Extra keys report the same layer at batch 4 and 16 and the prefill GEMM at 128,
+1024 and 4096 tokens; `roofline` is for the decode kernel, `cpu_baseline` is the reference's dense CPU path (two
 F.linear on unpacked +-1 factors) timed on this host.
 """
 from __future__ import annotations
@@ -239,37 +239,39 @@ def main():
         extra["batch1_per_linear_launches"] = {"us_per_layer": round(ms_pl * 1e3, 3),
                                                "GBps": round(bytes1 / (ms_pl * 1e-3) / 1e9, 2),
                                                "note": "same layer through nq_gemv_forward: 14 launches per layer"}
-        # ---- 128-token prefill over the same layer shapes ----
-        tokens = 128
-        pre = []
+        # ---- prefill GEMM over the three distinct linear shapes of the layer ----
+        # Timed as HIP graph replays: through Python the two-GEMM op costs more host time than GPU time.
+        op = torch.ops.binary_kernels.marlin_nanoquant_forward
         g2 = torch.Generator(device=dev)
         g2.manual_seed(2)
-        for (_, m, n) in LLAMA2_7B_LAYER[3:]:  # o (4096^2), gate, up, down: the three distinct shapes + one repeat
+        packed_by_shape = {}
+        for (_, m, n) in LLAMA2_7B_LAYER[3:5] + LLAMA2_7B_LAYER[6:]:   # o (4096^2), gate, down
             r = nominal_rank(m, n)
             v = (torch.randint(0, 2, (n, r), device=dev, generator=g2, dtype=torch.int8) * 2 - 1)
             u = (torch.randint(0, 2, (r, m), device=dev, generator=g2, dtype=torch.int8) * 2 - 1)
             sc = lambda k: (torch.randn(k, device=dev, generator=g2).abs() * 0.02 + 1e-3).to(torch.float16)
-            packed = packing.marlin_nanoquant_packer(v, u, sc(n), sc(r), sc(m))
-            x = torch.randn(tokens, n, device=dev, generator=g2).to(torch.float16)
-            pre.append((m, n, r, x, packed))
-        op = torch.ops.binary_kernels.marlin_nanoquant_forward
-        gemm_lines = {}
-        for (m, n, r, x, packed) in pre:
-            for _ in range(5):
-                op(x, *packed)
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            iters = 50
-            e0.record()
-            for _ in range(iters):
-                op(x, *packed)
-            e1.record()
-            torch.cuda.synchronize()
-            us = e0.elapsed_time(e1) * 1e3 / iters
-            tf = gemm_flops(m, n, r, tokens) / (us * 1e-6) / 1e12
-            gemm_lines[f"{m}x{n}_r{r}"] = {"us": round(us, 2), "TFLOPs": round(tf, 2),
-                                           "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
-        extra["prefill_128_tokens"] = gemm_lines
+            packed_by_shape[(m, n, r)] = packing.marlin_nanoquant_packer(v, u, sc(n), sc(r), sc(m))
+            del v, u
+        for tokens in (128, 1024, 4096):
+            gemm_lines = {}
+            for (m, n, r), packed in packed_by_shape.items():
+                x = torch.randn(tokens, n, device=dev, generator=g2).to(torch.float16)
+                per_graph, replays = 10, 5
+                g = capture_rotation([lambda: op(x, *packed)] * per_graph)
+                g.replay()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(replays):
+                    g.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) * 1e3 / (per_graph * replays)
+                tf = gemm_flops(m, n, r, tokens) / (us * 1e-6) / 1e12
+                gemm_lines[f"{m}x{n}_r{r}"] = {"us": round(us, 2), "TFLOPs": round(tf, 2),
+                                               "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+                del g, x
+            extra[f"prefill_{tokens}_tokens"] = gemm_lines
         result["extra"] = extra
 
         # ---- CPU baseline: the reference's dense path on this host (bounded sample) ----

@@ -225,6 +225,73 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
             if (c >= total) { k = ids.size() - 1; row = table[ids[k]].rows; return; }
             row = (int)((c - prefix[k]) / table[ids[k]].units);
         };
+        if (ids.size() * 2 <= (size_t)nwg) {
+            // Few stages, many workgroups: give every stage whole workgroups, so that no workgroup stages
+            // two input vectors in one phase.  A slice costs units * (rows + kSliceOverheadRows): staging the
+            // input vector takes about as long as the arithmetic of a dozen rows of the same width.  The
+            // workgroup counts n_s minimise the slowest slice, max_s units_s * (rows_s / n_s + overhead).
+            const double kSliceOverheadRows = 12.0;
+            std::vector<int> share(ids.size(), 1);
+            auto needed = [&](double t) {       // workgroups needed for every slice to cost at most t
+                long long sum = 0;
+                for (size_t k = 0; k < ids.size(); ++k) {
+                    const double u = table[ids[k]].units, r = table[ids[k]].rows;
+                    const double room = t - u * kSliceOverheadRows;
+                    if (room <= 0) return (long long)nwg + 1;
+                    long long n = (long long)((u * r + room - 1e-9) / room);
+                    if (n < 1) n = 1;
+                    if (n > table[ids[k]].rows) n = table[ids[k]].rows;
+                    sum += n;
+                }
+                return sum;
+            };
+            double lo = 0, hi = 0;
+            for (size_t k = 0; k < ids.size(); ++k) {
+                const double t1 = (double)table[ids[k]].units * (table[ids[k]].rows + kSliceOverheadRows);
+                if (t1 > hi) hi = t1;
+            }
+            for (int iter = 0; iter < 60; ++iter) {
+                const double mid = 0.5 * (lo + hi);
+                if (needed(mid) <= nwg) hi = mid; else lo = mid;
+            }
+            int used = 0;
+            for (size_t k = 0; k < ids.size(); ++k) {
+                const double u = table[ids[k]].units, r = table[ids[k]].rows;
+                const double room = hi - u * kSliceOverheadRows;
+                long long n = room > 0 ? (long long)((u * r + room - 1e-9) / room) : 1;
+                if (n < 1) n = 1;
+                if (n > table[ids[k]].rows) n = table[ids[k]].rows;
+                share[k] = (int)n;
+                used += share[k];
+            }
+            // left-over workgroups go where a slice is slowest
+            while (used < nwg) {
+                size_t best = ids.size();
+                double worst = -1;
+                for (size_t k = 0; k < ids.size(); ++k) {
+                    if (share[k] >= table[ids[k]].rows) continue;
+                    const double t = table[ids[k]].units * ((double)table[ids[k]].rows / share[k] + kSliceOverheadRows);
+                    if (t > worst) { worst = t; best = k; }
+                }
+                if (best == ids.size()) break;
+                ++share[best];
+                ++used;
+            }
+            int w = 0;
+            for (size_t k = 0; k < ids.size(); ++k) {
+                const int rows = table[ids[k]].rows;
+                for (int j = 0; j < share[k]; ++j, ++w) {
+                    const int rb = (int)((long long)rows * j / share[k]);
+                    const int re = (int)((long long)rows * (j + 1) / share[k]);
+                    if (re > rb) {
+                        slice[ph][(size_t)w].push_back(nq::RunSegment{ids[k], rb, re, 0});
+                        table[ids[k]].seg_count += 1;
+                    }
+                }
+            }
+            continue;
+        }
+        // Many stages: equal shares of the total arithmetic, cut wherever they fall.
         for (int w = 0; w < nwg; ++w) {
             const long long c0 = total * w / nwg, c1 = total * (w + 1) / nwg;
             size_t k0, k1; int r0, r1;

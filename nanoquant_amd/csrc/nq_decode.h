@@ -41,140 +41,192 @@ struct StageInput {
     int vec_in;             // 16-byte loads allowed
 };
 
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+// By value on purpose: __builtin_bit_cast applied directly to a vector element (v.y, v[e]) reads
+// element 0 with this compiler.
+__device__ __forceinline__ float as_float(uint32_t bits) { return __builtin_bit_cast(float, bits); }
+
+// Raw buffer view (gfx9 resource words) of `bytes` bytes at p: loads past the end return zeros, so a
+// lane whose columns lie beyond K is pointed past the end instead of being branched around.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t raw_buffer(const void* p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
+}
+constexpr uint32_t kPastEnd = 0x7FFFFFF0u;
+constexpr int kCacheDefault = 0;
+constexpr int kCacheAgentCoherent = 16;   // sc1: served coherently at device scope, not from this XCD's L2
+
+// Coherent fp32 input (the intermediate h written by other workgroups of this launch): 16-byte
+// device-coherent loads, kBurst per lane in flight before the first is consumed (a round trip to the
+// memory side costs about a microsecond; 256 lanes x 4 loads cover 4096 values in one round trip).
+// One lane holds 4 consecutive values = 2 pairs; the 128 values of a unit sit in 32 consecutive lanes.
+// Requires K % 4 == 0 and 16-byte aligned rows.
+template <int DT, int BATCH>
+__device__ __forceinline__ void stage_units_coherent(uint4* xs, float* xsum, const StageInput& st, int c0, int cu_n,
+                                                     int upad, int nthreads) {
+    using E = Elem<DT>;
+    constexpr int kBurst = 4;
+    const int nquads = cu_n * 32;
+    const int total = BATCH * nquads;
+    const __amdgpu_buffer_rsrc_t rsrc =
+        raw_buffer(st.in, (uint32_t)(((size_t)(BATCH - 1) * st.in_stride + st.K) * sizeof(float)));
+#pragma unroll 1
+    for (int it0 = threadIdx.x; it0 < total; it0 += nthreads * kBurst) {   // wave-uniform trip count: it0 - lane
+        u32x4_t raw[kBurst];
+#pragma unroll
+        for (int j = 0; j < kBurst; ++j) {
+            const int it = it0 + j * nthreads;
+            const int b = it / nquads, q = it - b * nquads;
+            const int col = c0 * 128 + 4 * q;
+            const uint32_t off = (it < total && col < st.K) ? (uint32_t)(((size_t)b * st.in_stride + col) * sizeof(float)) : kPastEnd;
+            raw[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, kCacheAgentCoherent);
+        }
+#pragma unroll
+        for (int j = 0; j < kBurst; ++j) {
+            const int it = it0 + j * nthreads;
+            const int b = it / nquads, q = it - b * nquads;
+            const uint16_t r0 = E::from_float(as_float(raw[j].x));
+            const uint16_t r1 = E::from_float(as_float(raw[j].y));
+            const uint16_t r2 = E::from_float(as_float(raw[j].z));
+            const uint16_t r3 = E::from_float(as_float(raw[j].w));
+            // the sum of what the dot products will actually see; lanes past the end hold zeros
+            const float tot = group_sum((E::to_float(r0) + E::to_float(r1)) + (E::to_float(r2) + E::to_float(r3)), 32);
+            if (it < total) {
+                const int cu = q >> 5, i = (q & 31) >> 1;
+                uint2 pr;
+                pr.x = (uint32_t)r0 | ((uint32_t)r1 << 16);
+                pr.y = (uint32_t)r2 | ((uint32_t)r3 << 16);
+                *(uint2*)((uint32_t*)xs + ((size_t)(b * 16 + i) * upad + cu) * 4 + 2 * (q & 1)) = pr;
+                if ((q & 31) == 0) xsum[b * upad + cu] = tot;
+            }
+        }
+    }
+}
+
+// 16-bit input (times its per-column scale) or non-coherent fp32 input, 8 columns per lane and load.
+// Requires 16-byte aligned rows and K % 8 == 0 (st.vec_in).
+template <int DT, int BATCH>
+__device__ __forceinline__ void stage_units_vector(uint4* xs, float* xsum, const StageInput& st, int c0, int cu_n,
+                                                   int upad, int nthreads) {
+    using E = Elem<DT>;
+    constexpr int kBurst = 6;   // 256 lanes x 6 chunks = 12288 columns in one round trip
+    const int nchunks = cu_n * 16;
+    const int total = BATCH * nchunks;
+    const uint32_t esize = st.in_f32 ? 4u : 2u;
+    const __amdgpu_buffer_rsrc_t rin = raw_buffer(st.in, (uint32_t)(((size_t)(BATCH - 1) * st.in_stride + st.K) * esize));
+    const bool scaled = !st.in_f32 && st.s_col != nullptr;
+    const __amdgpu_buffer_rsrc_t rsc = raw_buffer(scaled ? (const void*)st.s_col : st.in, scaled ? (uint32_t)st.K * 2u : 0u);
+#pragma unroll 1
+    for (int it0 = threadIdx.x; it0 < total; it0 += nthreads * kBurst) {
+        u32x4_t raw_a[kBurst], raw_b[kBurst];
+#pragma unroll
+        for (int j = 0; j < kBurst; ++j) {
+            const int it = it0 + j * nthreads;
+            const int b = it / nchunks, q = it - b * nchunks;
+            const int col = c0 * 128 + 8 * q;
+            const bool live = it < total && col < st.K;
+            const uint32_t off = live ? (uint32_t)(((size_t)b * st.in_stride + col) * esize) : kPastEnd;
+            raw_a[j] = __builtin_amdgcn_raw_buffer_load_b128(rin, off, 0, kCacheDefault);
+            if (st.in_f32) raw_b[j] = __builtin_amdgcn_raw_buffer_load_b128(rin, live ? off + 16u : kPastEnd, 0, kCacheDefault);
+            else raw_b[j] = __builtin_amdgcn_raw_buffer_load_b128(rsc, live ? (uint32_t)col * 2u : kPastEnd, 0, kCacheDefault);
+        }
+#pragma unroll
+        for (int j = 0; j < kBurst; ++j) {
+            const int it = it0 + j * nthreads;
+            const int b = it / nchunks, q = it - b * nchunks;
+            float v[8];
+            if (!st.in_f32) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t xw = raw_a[j][e], sw = scaled ? raw_b[j][e] : E::kOnePair;
+                    v[2 * e] = E::to_float(xw & 0xFFFFu) * E::to_float(sw & 0xFFFFu);
+                    v[2 * e + 1] = E::to_float(xw >> 16) * E::to_float(sw >> 16);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = as_float(raw_a[j][e]);
+                    v[4 + e] = as_float(raw_b[j][e]);
+                }
+            }
+            uint16_t r[8];
+            float tot = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                r[e] = E::from_float(v[e]);
+                tot += E::to_float(r[e]);          // the sum of what the dot products will actually see
+            }
+            // the 16 chunks of a unit are held by 16 consecutive lanes: finish the unit sum with DPP
+            tot = group_sum(tot, 16);
+            if (it < total) {
+                const int cu = q >> 4, i = q & 15;
+                uint4 pk;
+                pk.x = (uint32_t)r[0] | ((uint32_t)r[1] << 16);
+                pk.y = (uint32_t)r[2] | ((uint32_t)r[3] << 16);
+                pk.z = (uint32_t)r[4] | ((uint32_t)r[5] << 16);
+                pk.w = (uint32_t)r[6] | ((uint32_t)r[7] << 16);
+                xs[(b * 16 + i) * upad + cu] = pk;
+                if (i == 0) xsum[b * upad + cu] = tot;
+            }
+        }
+    }
+}
+
+// Element-wise fallback for inputs that allow no 16-byte loads (odd K, unaligned rows).
+template <int DT, int BATCH>
+__device__ __forceinline__ void stage_units_scalar(uint4* xs, float* xsum, const StageInput& st, int c0, int cu_n,
+                                                   int upad, int nthreads) {
+    using E = Elem<DT>;
+    const int nchunks = cu_n * 16;
+#pragma unroll 1
+    for (int b = 0; b < BATCH; ++b) {
+#pragma unroll 1
+        for (int q0 = 0; q0 < nchunks; q0 += nthreads) {    // all lanes take every trip: group_sum needs them
+            const int q = q0 + threadIdx.x;
+            const int cu = q >> 4, i = q & 15;
+            const int col = (c0 + cu) * 128 + i * 8;
+            uint16_t r[8];
+            float tot = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int c = col + e;
+                float t = 0.f;
+                if (q < nchunks && c < st.K) {
+                    if (!st.in_f32) {
+                        t = E::to_float(((const uint16_t*)st.in)[(size_t)b * st.in_stride + c]);
+                        if (st.s_col) t *= E::to_float(st.s_col[c]);
+                    } else if (st.in_coherent) {
+                        t = __builtin_bit_cast(float, __hip_atomic_load((const uint32_t*)st.in + (size_t)b * st.in_stride + c,
+                                                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+                    } else {
+                        t = ((const float*)st.in)[(size_t)b * st.in_stride + c];
+                    }
+                }
+                r[e] = E::from_float(t);
+                tot += E::to_float(r[e]);
+            }
+            tot = group_sum(tot, 16);
+            if (q < nchunks) {
+                uint4 pk;
+                pk.x = (uint32_t)r[0] | ((uint32_t)r[1] << 16);
+                pk.y = (uint32_t)r[2] | ((uint32_t)r[3] << 16);
+                pk.z = (uint32_t)r[4] | ((uint32_t)r[5] << 16);
+                pk.w = (uint32_t)r[6] | ((uint32_t)r[7] << 16);
+                xs[(b * 16 + i) * upad + cu] = pk;
+                if (i == 0) xsum[b * upad + cu] = tot;
+            }
+        }
+    }
+}
+
 // Stage units [c0, c0+cu_n) for BATCH rows.  All threads of the workgroup call this; nthreads is the
 // workgroup size (a multiple of 64).  Must be followed by a barrier before xs/xsum are read.
 template <int DT, int BATCH>
 __device__ __forceinline__ void stage_units(uint4* xs, float* xsum, const StageInput& st, int c0, int cu_n, int upad,
                                             int nthreads) {
-    using E = Elem<DT>;
-    if (st.in_f32 && st.in_coherent) {
-        // Device-coherent loads are not served from this XCD's L2: keep them dense -- consecutive
-        // lanes read consecutive pairs, one wavefront covers exactly one unit (64 pairs).
-        const int npairs = cu_n * 64;
-        const bool wide = (((uintptr_t)st.in | ((uintptr_t)st.in_stride * 4)) & 7u) == 0;
-#pragma unroll 1
-        for (int b = 0; b < BATCH; ++b) {
-            const uint32_t* hp = (const uint32_t*)st.in + (size_t)b * st.in_stride;
-            // kBurst loads per lane are put in flight before the first one is consumed: a coherent load is
-            // a round trip to the memory side (~2 us); one round per burst instead of one per pair
-            constexpr int kBurst = 4;
-#pragma unroll 1
-            for (int p0 = threadIdx.x; p0 < npairs; p0 += nthreads * kBurst) {
-                uint32_t lo[kBurst], hi[kBurst];
-#pragma unroll
-                for (int j = 0; j < kBurst; ++j) {
-                    const int p = p0 + j * nthreads;
-                    const int col = c0 * 128 + 2 * p;
-                    lo[j] = 0; hi[j] = 0;
-                    if (p < npairs) {
-                        if (wide && col + 1 < st.K) {
-                            const uint64_t both = __hip_atomic_load((const uint64_t*)(hp + col), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                            lo[j] = (uint32_t)both; hi[j] = (uint32_t)(both >> 32);
-                        } else {
-                            if (col < st.K) lo[j] = __hip_atomic_load(hp + col, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                            if (col + 1 < st.K) hi[j] = __hip_atomic_load(hp + col + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        }
-                    }
-                }
-#pragma unroll
-                for (int j = 0; j < kBurst; ++j) {
-                    const int p = p0 + j * nthreads;
-                    if (p < npairs) {      // wave-uniform: npairs and the wave's first p are multiples of 64
-                        const uint16_t r0 = E::from_float(__builtin_bit_cast(float, lo[j]));
-                        const uint16_t r1 = E::from_float(__builtin_bit_cast(float, hi[j]));
-                        const int cu = p >> 6, i = (p & 63) >> 2, slot = p & 3;
-                        ((uint32_t*)xs)[((b * 16 + i) * upad + cu) * 4 + slot] = (uint32_t)r0 | ((uint32_t)r1 << 16);
-                        const float tot = group_sum(E::to_float(r0) + E::to_float(r1), 64);
-                        if ((p & 63) == 0) xsum[b * upad + cu] = tot;
-                    }
-                }
-            }
-        }
-        return;
-    }
-    const int nchunks = cu_n * 16;
-    constexpr int kBurst = 2;   // chunks whose loads are in flight together
-#pragma unroll 1
-    for (int b = 0; b < BATCH; ++b) {
-#pragma unroll 1
-        for (int q0 = threadIdx.x; q0 < nchunks; q0 += nthreads * kBurst) {
-            uint4 raw_a[kBurst], raw_b[kBurst];
-            bool fast[kBurst];
-#pragma unroll
-            for (int j = 0; j < kBurst; ++j) {
-                const int q = q0 + j * nthreads;
-                const int col = (c0 + (q >> 4)) * 128 + (q & 15) * 8;
-                fast[j] = q < nchunks && st.vec_in && col + 8 <= st.K;
-                raw_a[j] = make_uint4(0, 0, 0, 0);
-                raw_b[j] = make_uint4(E::kOnePair, E::kOnePair, E::kOnePair, E::kOnePair);
-                if (fast[j]) {
-                    if (!st.in_f32) {
-                        raw_a[j] = *(const uint4*)((const uint16_t*)st.in + (size_t)b * st.in_stride + col);
-                        if (st.s_col) raw_b[j] = *(const uint4*)(st.s_col + col);
-                    } else {
-                        const float* hp = (const float*)st.in + (size_t)b * st.in_stride + col;
-                        raw_a[j] = *(const uint4*)hp;
-                        raw_b[j] = *(const uint4*)(hp + 4);
-                    }
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < kBurst; ++j) {
-                const int q = q0 + j * nthreads;
-                if (q >= nchunks) continue;               // uniform over each aligned group of 16 lanes
-                const int cu = q >> 4, i = q & 15;
-                const int col = (c0 + cu) * 128 + i * 8;
-                float v[8];
-                if (fast[j]) {
-                    if (!st.in_f32) {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const uint32_t xw = comp_d(raw_a[j], e), sw = comp_d(raw_b[j], e);
-                            v[2 * e] = E::to_float(xw & 0xFFFFu) * E::to_float(sw & 0xFFFFu);
-                            v[2 * e + 1] = E::to_float(xw >> 16) * E::to_float(sw >> 16);
-                        }
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            v[e] = __builtin_bit_cast(float, comp_d(raw_a[j], e));
-                            v[4 + e] = __builtin_bit_cast(float, comp_d(raw_b[j], e));
-                        }
-                    }
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const int c = col + e;
-                        float t = 0.f;
-                        if (c < st.K) {
-                            if (!st.in_f32) {
-                                t = E::to_float(((const uint16_t*)st.in)[(size_t)b * st.in_stride + c]);
-                                if (st.s_col) t *= E::to_float(st.s_col[c]);
-                            } else {
-                                t = ((const float*)st.in)[(size_t)b * st.in_stride + c];
-                            }
-                        }
-                        v[e] = t;
-                    }
-                }
-                uint16_t r[8];
-                float tot = 0.f;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    r[e] = E::from_float(v[e]);
-                    tot += E::to_float(r[e]);          // the sum of what the dot products will actually see
-                }
-                uint4 p;
-                p.x = (uint32_t)r[0] | ((uint32_t)r[1] << 16);
-                p.y = (uint32_t)r[2] | ((uint32_t)r[3] << 16);
-                p.z = (uint32_t)r[4] | ((uint32_t)r[5] << 16);
-                p.w = (uint32_t)r[6] | ((uint32_t)r[7] << 16);
-                xs[(b * 16 + i) * upad + cu] = p;
-                // the 16 chunks of a unit are held by 16 consecutive lanes: finish the unit sum with DPP
-                tot = group_sum(tot, 16);
-                if (i == 0) xsum[b * upad + cu] = tot;
-            }
-        }
-    }
+    if (!st.vec_in || (st.K & 7)) stage_units_scalar<DT, BATCH>(xs, xsum, st, c0, cu_n, upad, nthreads);
+    else if (st.in_f32 && st.in_coherent) stage_units_coherent<DT, BATCH>(xs, xsum, st, c0, cu_n, upad, nthreads);
+    else stage_units_vector<DT, BATCH>(xs, xsum, st, c0, cu_n, upad, nthreads);
 }
 
 // Signed sum over one unit for BATCH rows: out[b] = sum_{c in unit} sgn(bit c) * x[b][c].

@@ -37,7 +37,6 @@ __device__ unsigned long long* g_nq_trace = nullptr;
 
 namespace nq {
 
-constexpr int kStreamThreads = 256;
 constexpr int kRowBlock = 128;                 // rows finished per pass of a workgroup
 // Same-address device-scope atomics serialise at the memory side (tens of ns each), so completion
 // counts are spread over kSubCounters addresses per stage and kExitSubs addresses for the exit count,
@@ -67,13 +66,18 @@ __device__ __forceinline__ uint4 load_unit(const RunStage& st, int row, int unit
     return w;
 }
 
-template <int DT, int BATCH, bool MFMA>
-__global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(const RunStage* __restrict__ stages, int nstages,
+// Items of the MFMA path that each wavefront of a workgroup takes (contiguous runs).
+__host__ __device__ __forceinline__ int mfma_items_per_wave(int nitems, int waves) { return (nitems + waves - 1) / waves; }
+
+template <int DT, int BATCH, bool MFMA, int THREADS>
+__global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __restrict__ stages, int nstages,
                                                                      int nphases, const int* __restrict__ seg_index,
                                                                      const RunSegment* __restrict__ segs,
                                                                      unsigned long long* counters, unsigned* status,
                                                                      unsigned spin_limit, int chunk_cap) {
     using E = Elem<DT>;
+    constexpr int kStreamThreads = THREADS;
+    constexpr int kWaves = THREADS / kWave;
     extern __shared__ uint4 lds_raw[];
     float* racc = (float*)lds_raw;                              // [kRowBlock][BATCH] row sums
     float* xsum = racc + kRowBlock * BATCH;                     // [BATCH][kXsumStride] per-unit input sums
@@ -115,9 +119,14 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(const RunSt
             // First fetch of the slice, issued before any wait: the weights are always ready.
             uint4 wnext = make_uint4(0, 0, 0, 0);
             if constexpr (MFMA) {
-                // lane (row l & 15, octet l >> 4) of wavefront w starts with unit 4*w + (l >> 4) of its row
-                const int u0 = 4 * (tid >> 6) + ((tid & 63) >> 4);
-                if (u0 < chunk_units) wnext = load_unit(st, min(seg.row_begin + (tid & 15), st.rows - 1), u0);
+                // wavefront w starts with item w of the first row block: 16 rows x 4 units, lane (row l & 15,
+                // unit l >> 4)
+                const int ng0 = (chunk_units + 3) >> 2;
+                const int nr0 = min(seg.row_end - seg.row_begin, kRowBlock);
+                const int item0 = (tid >> 6) * mfma_items_per_wave(((nr0 + 15) >> 4) * ng0, kWaves);
+                const int u0 = 4 * (item0 % ng0) + ((tid & 63) >> 4);
+                if (item0 < ((nr0 + 15) >> 4) * ng0 && u0 < chunk_units)
+                    wnext = load_unit(st, min(seg.row_begin + 16 * (item0 / ng0) + (tid & 15), st.rows - 1), u0);
             } else {
                 const int nr0 = min(seg.row_end - seg.row_begin, kRowBlock);
                 if (tid < nr0 * chunk_units) wnext = load_unit(st, seg.row_begin + tid / chunk_units, tid % chunk_units);
@@ -162,6 +171,7 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(const RunSt
             }
             lds_barrier();                                       // s_flag; previous slice is done with xs / racc
             aborted = aborted || (s_flag != 0);
+            if (sg == seg_begin && ph < 3) NQ_MARK(1 + 4 * ph);
 
             if (!aborted) {
                 bool staged = false;
@@ -178,31 +188,41 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(const RunSt
                             staged = true;
                         }
                         lds_barrier();                           // xs / xsum / zeroed racc visible
+                        if (sg == seg_begin && ph < 3 && rb == seg.row_begin && c0 == 0) NQ_MARK(2 + 4 * ph);
                         if constexpr (MFMA) {
+                            // Items = (16-row group, 4-unit group), unit group fastest; every wavefront takes a
+                            // contiguous run of items, so it mostly stays on one row group and adds its
+                            // accumulator to the row sums only when the row group changes.
                             const int lane = tid & 63, wave = tid >> 6, r16 = lane & 15, g = lane >> 4;
-                            const int ngroups = (cu_n + 3) >> 2;          // unit groups of 4; wavefront w takes w, w+4, ...
+                            const int ngroups = (cu_n + 3) >> 2;
+                            const int nitems = ((nr + 15) >> 4) * ngroups;
+                            const int per = mfma_items_per_wave(nitems, kWaves);
+                            const int it_begin = wave * per, it_end = min(it_begin + per, nitems);
+                            float4_t acc = {0.f, 0.f, 0.f, 0.f};
+                            uint4 w = wnext;                             // very first fetch of the slice
+                            if ((rb != seg.row_begin || c0 != 0) && it_begin < it_end) {
+                                w = make_uint4(0, 0, 0, 0);
+                                const int u = 4 * (it_begin % ngroups) + g;
+                                if (u < cu_n) w = load_unit(st, min(rb + 16 * (it_begin / ngroups) + r16, st.rows - 1), c0 + u);
+                            }
 #pragma unroll 1
-                            for (int rg = 0; rg < nr; rg += 16) {
-                                const int row = min(rb + rg + r16, st.rows - 1);
-                                float4_t acc = {0.f, 0.f, 0.f, 0.f};
-                                uint4 w = wnext;                         // very first fetch of the slice
-                                if (rb != seg.row_begin || c0 != 0 || rg != 0) {
-                                    w = make_uint4(0, 0, 0, 0);
-                                    if (4 * wave + g < cu_n) w = load_unit(st, row, c0 + 4 * wave + g);
+                            for (int it = it_begin; it < it_end; ++it) {
+                                const int rg = 16 * (it / ngroups), u = 4 * (it % ngroups) + g;
+                                uint4 wpre = make_uint4(0, 0, 0, 0);
+                                if (it + 1 < it_end) {
+                                    const int un = 4 * ((it + 1) % ngroups) + g;
+                                    if (un < cu_n) wpre = load_unit(st, min(rb + 16 * ((it + 1) / ngroups) + r16, st.rows - 1), c0 + un);
                                 }
-#pragma unroll 1
-                                for (int ub = wave; ub < ngroups; ub += 4) {
-                                    const int u = 4 * ub + g;
-                                    uint4 wpre = make_uint4(0, 0, 0, 0);
-                                    if (ub + 4 < ngroups && u + 16 < cu_n) wpre = load_unit(st, row, c0 + u + 16);
-                                    unit_mfma<DT, BATCH>(w, xs, upad, u, u < cu_n, acc);
-                                    w = wpre;
-                                }
-                                // acc[v] = partial sum of row rg + 4*g + v for batch row r16
-                                if (r16 < BATCH) {
+                                unit_mfma<DT, BATCH>(w, xs, upad, u, u < cu_n, acc);
+                                w = wpre;
+                                if (it + 1 == it_end || (it + 1) % ngroups == 0) {
+                                    // acc[v] = partial sum of row rg + 4*g + v for batch row r16
+                                    if (r16 < BATCH) {
 #pragma unroll
-                                    for (int v = 0; v < 4; ++v)
-                                        if (rg + 4 * g + v < nr) atomicAdd(&racc[(rg + 4 * g + v) * BATCH + r16], acc[v]);
+                                        for (int v = 0; v < 4; ++v)
+                                            if (rg + 4 * g + v < nr) atomicAdd(&racc[(rg + 4 * g + v) * BATCH + r16], acc[v]);
+                                    }
+                                    acc = (float4_t){0.f, 0.f, 0.f, 0.f};
                                 }
                             }
                         } else {
@@ -229,6 +249,7 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(const RunSt
                         }
                         }
                     lds_barrier();                               // row sums complete
+                    if (ph < 3) NQ_MARK(3 + 4 * ph);
                     for (int i = tid; i < nr * BATCH; i += kStreamThreads) {
                         const int row = rb + i / BATCH, b = i % BATCH;
                         float v = racc[i];
@@ -267,7 +288,7 @@ __global__ __launch_bounds__(kStreamThreads) void gemv_stream_kernel(const RunSt
                 }
             }
         }
-        NQ_MARK(1 + (ph < 14 ? ph : 14));
+        if (ph < 3) NQ_MARK(4 + 4 * ph);
     }
 
     if (tid == 0) {
@@ -292,11 +313,21 @@ static void stream_lds_plan(int batch, int max_units, int* chunk_cap_out, size_t
     *lds_out = (size_t)racc_bytes + (size_t)batch * 16 * (chunk_units | 1) * sizeof(uint4);
 }
 
+// Workgroup size by batch.  Every workgroup stages the whole input vector of its stage, so larger
+// workgroups mean less staging traffic per row: decisive from batch 4 up (batch 16: 211 -> 93 us per
+// Llama-2-7B layer going from 256 to 1024 lanes).  At batch 1 four independent 256-lane workgroups per
+// CU overlap each other's staging and arithmetic better than one large one (32.7 vs 35.0 us); the
+// matmul-free batch-2 kernel needs more than the 128 registers a 1024-lane workgroup leaves per lane.
+#ifndef NQ_STREAM_THREADS
+#define NQ_STREAM_THREADS(BATCH) ((BATCH) == 1 ? 256 : (BATCH) == 2 ? 512 : 1024)
+#endif
+
 template <int DT, int BATCH>
 struct StreamKernel {
     // batches of 4 and more go through the MFMA units; 1 and 2 stay matmul-free
     static constexpr bool kMfma = BATCH >= 4;
-    static constexpr auto fn = gemv_stream_kernel<DT, BATCH, kMfma>;
+    static constexpr int kThreads = NQ_STREAM_THREADS(BATCH);
+    static constexpr auto fn = gemv_stream_kernel<DT, BATCH, kMfma, kThreads>;
 };
 
 template <int DT, int BATCH>
@@ -318,7 +349,7 @@ static int capacity_of(int max_units) {
     stream_lds_plan(BATCH, max_units, &chunk_cap, &lds);
     if (prepare_kernel<DT, BATCH>(lds) != hipSuccess) return 0;
     int per_cu = 0, dev = 0, cus = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)StreamKernel<DT, BATCH>::fn, kStreamThreads,
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)StreamKernel<DT, BATCH>::fn, StreamKernel<DT, BATCH>::kThreads,
                                                      lds) != hipSuccess)
         return 0;
     if (hipGetDevice(&dev) != hipSuccess) return 0;
@@ -344,7 +375,8 @@ static hipError_t launch_stream(const RunStage* stages, int nstages, int nphases
         (void)hipMemcpyToSymbol(HIP_SYMBOL(g_nq_trace), &tbuf, sizeof(tbuf));
     }
 #endif
-    hipLaunchKernelGGL((gemv_stream_kernel<DT, BATCH, StreamKernel<DT, BATCH>::kMfma>), dim3(nwg), dim3(kStreamThreads), lds, stream, stages, nstages,
+    using SK = StreamKernel<DT, BATCH>;
+    hipLaunchKernelGGL((SK::fn), dim3(nwg), dim3(SK::kThreads), lds, stream, stages, nstages,
                        nphases, seg_index, segs, counters, status, (unsigned)(1u << 21), chunk_cap);
 #ifdef NQ_TRACE
     if (tbuf && ++calls == 40) {
