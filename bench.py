@@ -27,7 +27,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the headline kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
 # copy kernel of known size (profiles/gemv_stream_llama2_7b_layer_b1.md); valid for the default workload only.
-MEASURED_TRAFFIC_BYTES = 28184334
+MEASURED_TRAFFIC_BYTES = 28549760
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 LLAMA2_7B_LAYER = (("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096),
@@ -77,7 +77,6 @@ def main():
     ap.add_argument("--steps", type=int, default=520)
     ap.add_argument("--warmup", type=int, default=52)
     ap.add_argument("--copies", type=int, default=26, help="distinct weight copies of the layer (26 x 25.3 MB > 256 MB)")
-    ap.add_argument("--interleave", type=int, default=7, help="first stages run ahead of second stages by this many linears")
     ap.add_argument("--no-extra", action="store_true", help="skip batch 4/16, prefill and CPU legs")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -120,13 +119,13 @@ def main():
             if st != 0:
                 raise RuntimeError(_lib.status_message(st))
 
-    def make_runlists(io, batch, interleave):
+    def make_runlists(io, batch):
         """One run list (= one persistent launch) per weight copy."""
         from nanoquant_amd import DecodeRunList
         xs, _, ys = io
         lists = []
         for layer in layers:
-            rl = DecodeRunList(batch, torch.float16, dev, interleave=interleave)
+            rl = DecodeRunList(batch, torch.float16, dev)
             for lin, x, y in zip(layer, xs, ys):
                 rl.add(x, lin.s_in, lin.vt_bits, lin.s_mid, lin.u_bits, lin.s_out, y=y)
             rl.build()
@@ -171,7 +170,7 @@ def main():
 
     # ---- headline: batch 1 -------------------------------------------------------------------
     io1 = make_io(1)
-    lists1 = make_runlists(io1, 1, args.interleave)
+    lists1 = make_runlists(io1, 1)
     ms = timed([rl.run for rl in lists1], args.steps, args.warmup)
     for rl in lists1:
         if rl.status() != 0:
@@ -205,12 +204,13 @@ def main():
         "us_per_layer": round(ms * 1e3, 3),
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_stream_kernel<fp16, batch 1> (one launch per layer: 14 stages, 1559 workgroups)",
+            "kernel": "gemv_stream_kernel<fp16, batch 1, 256 lanes> (one launch per layer: 14 stages in 2 phases, "
+                      "1024 resident workgroups)",
             "achieved": round(bytes1 / launches_per_step / (launch_us * 1e-6) / 1e9, 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(bytes1 / launches_per_step / (launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES if (args.copies == 26 and args.interleave == 7) else None,
+            "traffic": MEASURED_TRAFFIC_BYTES if args.copies == 26 else None,
             "bytes_per_launch": int(bytes1 / launches_per_step),
             "avg_launch_us": round(launch_us, 3),
         },
@@ -230,11 +230,26 @@ def main():
         extra = {}
         for b in (4, 16):
             io = make_io(b)
-            lists = make_runlists(io, b, args.interleave)
+            lists = make_runlists(io, b)
             msb = timed([rl.run for rl in lists], max(args.steps // 4, args.copies), args.copies)
             extra[f"batch{b}"] = {"us_per_layer": round(msb * 1e3, 3),
                                   "GBps": round(layer_bytes(b) / (msb * 1e-3) / 1e9, 2)}
             del lists
+        # all weight copies in ONE run list (= one launch over copies x 7 linears): the per-launch latencies
+        # (descriptor fetch, two dependency phases, drain) are paid once for the whole stack
+        from nanoquant_amd import DecodeRunList
+        stack = DecodeRunList(1, torch.float16, dev)
+        for layer in layers:
+            for lin, x, y in zip(layer, io1[0], io1[2]):
+                stack.add(x, lin.s_in, lin.vt_bits, lin.s_mid, lin.u_bits, lin.s_out, y=y)
+        stack.build()
+        ms_stack = timed([stack.run], 10, 2) / len(layers)
+        if stack.status() != 0:
+            raise RuntimeError("run list reported an expired dependency wait")
+        extra["batch1_stack_one_launch"] = {"us_per_layer": round(ms_stack * 1e3, 3),
+                                            "GBps": round(bytes1 / (ms_stack * 1e-3) / 1e9, 2),
+                                            "note": "%d layers (%d linears) in one run-list launch" % (len(layers), 7 * len(layers))}
+        del stack
         ms_pl = timed(per_linear_steps(io1, 1), max(args.steps // 4, args.copies), args.copies)
         extra["batch1_per_linear_launches"] = {"us_per_layer": round(ms_pl * 1e3, 3),
                                                "GBps": round(bytes1 / (ms_pl * 1e-3) / 1e9, 2),
