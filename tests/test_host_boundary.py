@@ -223,3 +223,23 @@ def test_mixture_dense_path_is_the_sum():
     x = oracle.synth_x(2, 96, 5).astype(np.float32)
     y = mix(torch.from_numpy(x)).numpy()
     assert np.allclose(y, oracle.mixture_forward(x, [ta, tb]), rtol=1e-5, atol=1e-7)
+
+
+def test_ops_trace_under_fake_tensors_and_make_fx():
+    # What torch.compile needs from a custom op: it runs on fake tensors of the device the real kernel serves,
+    # and a traced graph holds the op itself (no decomposition, no host fallback).  No GPU is touched.
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.fx.experimental.proxy_tensor import make_fx
+
+    def layer(x, s_in, vt_bits, s_mid, u_bits, s_out):
+        return torch.ops.binary_kernels.nanoquant_dyn_forward(x, s_in, vt_bits, s_mid, u_bits, s_out, 128, 128, 2, 2,
+                                                              1, 1, 8, 8)
+
+    with FakeTensorMode(allow_non_fake_inputs=False) as mode:
+        ft = lambda *shape, dtype=torch.float16: torch.empty(*shape, dtype=dtype, device="cuda")
+        args = (ft(4, 256), ft(256), ft(128, 8, dtype=torch.int32), ft(128), ft(512, 4, dtype=torch.int32), ft(512))
+        y = layer(*args)
+        assert y.shape == (4, 512) and y.dtype == torch.float16 and y.device.type == "cuda"
+        g = make_fx(layer, tracing_mode="real")(*args)
+    targets = [n.target for n in g.graph.nodes if n.op == "call_function"]
+    assert targets == [torch.ops.binary_kernels.nanoquant_dyn_forward.default]
