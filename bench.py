@@ -7,8 +7,8 @@ batch 1, fp16 activations.  One "step" is one pass over the 7 linears of the lay
 walk over distinct copies of the layer's weights (more than the 256 MB Infinity Cache in total), so
 the packed words come from HBM, not from cache.  `value` is algorithmic bytes / time.
 
-Prints ONE JSON line.  Extra keys report the same layer at batch 4 and 16 and the prefill GEMM at 128,
-1024 and 4096 tokens; `roofline` is for the decode kernel, `cpu_baseline` is the reference's dense CPU path (two
+Prints ONE JSON line.  Extra keys report the same layer at batch 4 and 16, the prefill GEMM at 128, 512
+and 4096 tokens, the two-term Qwen3-8B-like layer (cfg3) and the Llama-3-70B weight stream (cfg4); `roofline` is for the decode kernel, `cpu_baseline` is the reference's dense CPU path (two
 F.linear on unpacked +-1 factors) timed on this host.
 """
 from __future__ import annotations
@@ -267,7 +267,7 @@ def main():
             sc = lambda k: (torch.randn(k, device=dev, generator=g2).abs() * 0.02 + 1e-3).to(torch.float16)
             packed_by_shape[(m, n, r)] = packing.marlin_nanoquant_packer(v, u, sc(n), sc(r), sc(m))
             del v, u
-        for tokens in (128, 1024, 4096):
+        for tokens in (128, 512, 4096):
             gemm_lines = {}
             for (m, n, r), packed in packed_by_shape.items():
                 x = torch.randn(tokens, n, device=dev, generator=g2).to(torch.float16)
@@ -287,6 +287,62 @@ def main():
                                                "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
                 del g, x
             extra[f"prefill_{tokens}_tokens"] = gemm_lines
+        # ---- cfg3: Qwen3-8B-like layer, every weight a sum of two terms (ranks 3:1, ~0.55 bpw), batch 1 ----
+        qwen = (("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
+                ("gate", 12288, 4096), ("up", 12288, 4096), ("down", 4096, 12288))
+
+        def mixture_ranks(m, n):
+            total = 0.55 * m * n / (m + n)
+            return (max(32, int(round(0.75 * total / 32)) * 32), max(32, int(round(0.25 * total / 32)) * 32))
+
+        gq = torch.Generator(device=dev)
+        gq.manual_seed(4)
+        q_copies = 26
+        q_lists, q_bytes = [], 0.0
+        xq = {n: torch.randn(1, n, device=dev, generator=gq).to(torch.float16) for n in (4096, 12288)}
+        for c in range(q_copies):
+            rl = DecodeRunList(1, torch.float16, dev)
+            for (_, m, n) in qwen:
+                r0, r1 = mixture_ranks(m, n)
+                t0, t1 = SynthLinear(torch, dev, m, n, r0, gq), SynthLinear(torch, dev, m, n, r1, gq)
+                i0 = rl.add(xq[n], t0.s_in, t0.vt_bits, t0.s_mid, t0.u_bits, t0.s_out, out_f32=True)
+                rl.add(xq[n], t1.s_in, t1.vt_bits, t1.s_mid, t1.u_bits, t1.s_out, addend=rl.outputs[i0], y_from=i0)
+                if c == 0:
+                    q_bytes += gemv_bytes(m, n, r0, 1) + gemv_bytes(m, n, r1, 1)
+            rl.build()
+            q_lists.append(rl)
+        ms_q = timed([rl.run for rl in q_lists], 4 * q_copies, q_copies)
+        for rl in q_lists:
+            if rl.status() != 0:
+                raise RuntimeError("run list reported an expired dependency wait")
+        extra["cfg3_qwen3_8b_two_term_layer_batch1"] = {
+            "us_per_layer": round(ms_q * 1e3, 3), "GBps": round(q_bytes / (ms_q * 1e-3) / 1e9, 2),
+            "note": "14 terms in one launch, second terms add onto the fp32 output of the first inside the kernel"}
+        del q_lists
+
+        # ---- cfg4: Llama-3-70B-shaped weight stream, 80 layers x 7 linears in one launch ----
+        llama70 = (("q", 8192, 8192), ("k", 1024, 8192), ("v", 1024, 8192), ("o", 8192, 8192),
+                   ("gate", 28672, 8192), ("up", 28672, 8192), ("down", 8192, 28672))
+        g70 = torch.Generator(device=dev)
+        g70.manual_seed(5)
+        stack70 = [[SynthLinear(torch, dev, m, n, nominal_rank(m, n), g70) for (_, m, n) in llama70] for _ in range(80)]
+        for b in (1, 8):
+            x70 = {n: torch.randn(b, n, device=dev, generator=g70).to(torch.float16) for n in (8192, 28672)}
+            rl = DecodeRunList(b, torch.float16, dev)
+            for layer in stack70:
+                for lin in layer:
+                    rl.add(x70[lin.n], lin.s_in, lin.vt_bits, lin.s_mid, lin.u_bits, lin.s_out)
+            rl.build()
+            ms70 = timed([rl.run], 5, 1)
+            if rl.status() != 0:
+                raise RuntimeError("run list reported an expired dependency wait")
+            bytes70 = 80 * sum(gemv_bytes(lin.m, lin.n, lin.r, b) for lin in stack70[0])
+            extra[f"cfg4_llama3_70b_stream_batch{b}"] = {
+                "us_per_token_step": round(ms70 * 1e3, 1), "GBps": round(bytes70 / (ms70 * 1e-3) / 1e9, 2),
+                "resident_weight_GB": round(80 * sum(lin.r * (lin.m + lin.n) / 8 for lin in stack70[0]) / 1e9, 2),
+                "note": "560 linears in one run-list launch"}
+            del rl
+        del stack70
         result["extra"] = extra
 
         # ---- CPU baseline: the reference's dense path on this host (bounded sample) ----

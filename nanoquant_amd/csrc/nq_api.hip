@@ -190,6 +190,8 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         b.vec_in = al16(l.h) && ((size_t)l.r * 4) % 16 == 0;
         b.phase = a.phase + 1;
         if (b.dep2 >= 0 && table[b.dep2].phase + 1 > b.phase) b.phase = table[b.dep2].phase + 1;
+        // the kernel addresses the packed words of a stage with 32-bit byte offsets
+        if ((size_t)a.rows * a.words * 4 >= 0x7FFFFFF0ull || (size_t)b.rows * b.words * 4 >= 0x7FFFFFF0ull) return NQ_ERR_SHAPE;
         table[2 * i + 1] = b;
         if (a.units > max_units) max_units = a.units;
         if (b.units > max_units) max_units = b.units;

@@ -94,4 +94,23 @@ __device__ __forceinline__ float group_sum(float v, int group) {
     return v;
 }
 
+// Sum over aligned groups of 16, 32 or 64 lanes with DPP moves only (no LDS crossbar).  The total is
+// valid in the LAST 16 lanes of every group; the other lanes hold partial sums.  0x142 = row_bcast15
+// (lane 15 of a row to the next row), 0x143 = row_bcast31 (lane 31 to rows 2 and 3).
+__device__ __forceinline__ float group_sum_tail(float v, int group) {
+    v = dpp_add<0xB1>(v);
+    v = dpp_add<0x4E>(v);
+    v = dpp_add<0x141>(v);
+    v = dpp_add<0x140>(v);       // every lane: the total of its 16-lane row
+    if (group >= 32) {
+        const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false);
+        v += __builtin_bit_cast(float, moved);
+    }
+    if (group >= 64) {
+        const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false);
+        v += __builtin_bit_cast(float, moved);
+    }
+    return v;
+}
+
 }  // namespace nq

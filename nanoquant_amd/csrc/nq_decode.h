@@ -2,7 +2,7 @@
 // and the arithmetic of one 16-byte unit of packed signs (4 words = 128 columns of one row).
 //
 // LDS layout of the staged input (per batch row b): 16-byte chunk (b, i, cu) at
-// xs[(b*16 + i)*upad + cu] holds the 8 consecutive columns 128*(c0+cu) + 8*i .. +7 as 16-bit values;
+// xs[xs_chunk(b, i, upad, cu)] = xs[b*(16*upad+1) + i*upad + cu] holds the 8 consecutive columns 128*(c0+cu) + 8*i .. +7 as 16-bit values;
 // upad is odd.  For a fixed i the lanes of a row read consecutive chunks (conflict-free) and lanes of
 // different rows read the same chunk (broadcast).  xsum[b*upad + cu] is the fp32 sum of the 128
 // staged values of unit cu.
@@ -56,14 +56,53 @@ constexpr uint32_t kPastEnd = 0x7FFFFFF0u;
 constexpr int kCacheDefault = 0;
 constexpr int kCacheAgentCoherent = 16;   // sc1: served coherently at device scope, not from this XCD's L2
 
+// Two LDS layouts of a staged unit (128 columns = 64 pairs P = 0..63, pair P = columns 2P, 2P+1):
+//   chunk-major (PM = false): 16-byte chunk i = P >> 2 holds pairs 4i..4i+3 = 8 consecutive columns;
+//   pair-major  (PM = true):  16-byte chunk j = P & 15 holds pair j of each of the four 32-column words
+//                             (dword wi = P >> 4), the order in which one sign-bit position of the
+//                             four words of a unit addresses the columns.
+// Returns the dword index into xs.
+// 16-byte chunk index of (batch row b, chunk i, unit cu).  The batch-row pitch 16*upad + 1 chunks is
+// 4 dwords off a multiple of 64: the 16 lanes of an MFMA operand read that differ only in the batch row
+// fall into 16 different bank groups (a pitch of 16*upad chunks puts all of them into the same one).
+__device__ __forceinline__ int xs_chunk(int b, int i, int upad, int cu) { return b * (16 * upad + 1) + i * upad + cu; }
+// chunks of staged input for `batch` rows
+__host__ __device__ constexpr int xs_chunks(int batch, int upad) { return batch * (16 * upad + 1); }
+
+template <bool PM>
+__device__ __forceinline__ int xs_dword(int b, int P, int upad, int cu) {
+    if constexpr (PM) return xs_chunk(b, P & 15, upad, cu) * 4 + (P >> 4);
+    else return xs_chunk(b, P >> 2, upad, cu) * 4 + (P & 3);
+}
+
+// Stores the 8 consecutive 16-bit values r[0..7] of chunk i (columns 8i..8i+7) of unit cu.
+template <bool PM>
+__device__ __forceinline__ void store_chunk(uint4* xs, int b, int i, int upad, int cu, const uint16_t (&r)[8]) {
+    if constexpr (PM) {
+        uint32_t* xd = (uint32_t*)xs;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) xd[xs_dword<true>(b, 4 * i + k, upad, cu)] = (uint32_t)r[2 * k] | ((uint32_t)r[2 * k + 1] << 16);
+    } else {
+        uint4 pk;
+        pk.x = (uint32_t)r[0] | ((uint32_t)r[1] << 16);
+        pk.y = (uint32_t)r[2] | ((uint32_t)r[3] << 16);
+        pk.z = (uint32_t)r[4] | ((uint32_t)r[5] << 16);
+        pk.w = (uint32_t)r[6] | ((uint32_t)r[7] << 16);
+        xs[xs_chunk(b, i, upad, cu)] = pk;
+    }
+}
+
+// Staging variants below: `xtot` (may be null) receives the sum over all staged units per batch row
+// (LDS float atomics; the caller zeroes it and puts a barrier before and after).
+
 // Coherent fp32 input (the intermediate h written by other workgroups of this launch): 16-byte
 // device-coherent loads, kBurst per lane in flight before the first is consumed (a round trip to the
 // memory side costs about a microsecond; 256 lanes x 4 loads cover 4096 values in one round trip).
 // One lane holds 4 consecutive values = 2 pairs; the 128 values of a unit sit in 32 consecutive lanes.
 // Requires K % 4 == 0 and 16-byte aligned rows.
-template <int DT, int BATCH>
-__device__ __forceinline__ void stage_units_coherent(uint4* xs, float* xsum, const StageInput& st, int c0, int cu_n,
-                                                     int upad, int nthreads) {
+template <int DT, int BATCH, bool PM>
+__device__ __forceinline__ void stage_units_coherent(uint4* xs, float* xsum, float* xtot, const StageInput& st, int c0,
+                                                     int cu_n, int upad, int nthreads) {
     using E = Elem<DT>;
     constexpr int kBurst = 4;
     const int nquads = cu_n * 32;
@@ -92,12 +131,14 @@ __device__ __forceinline__ void stage_units_coherent(uint4* xs, float* xsum, con
             // the sum of what the dot products will actually see; lanes past the end hold zeros
             const float tot = group_sum((E::to_float(r0) + E::to_float(r1)) + (E::to_float(r2) + E::to_float(r3)), 32);
             if (it < total) {
-                const int cu = q >> 5, i = (q & 31) >> 1;
-                uint2 pr;
-                pr.x = (uint32_t)r0 | ((uint32_t)r1 << 16);
-                pr.y = (uint32_t)r2 | ((uint32_t)r3 << 16);
-                *(uint2*)((uint32_t*)xs + ((size_t)(b * 16 + i) * upad + cu) * 4 + 2 * (q & 1)) = pr;
-                if ((q & 31) == 0) xsum[b * upad + cu] = tot;
+                const int cu = q >> 5, P = 2 * (q & 31);
+                uint32_t* xd = (uint32_t*)xs;
+                xd[xs_dword<PM>(b, P, upad, cu)] = (uint32_t)r0 | ((uint32_t)r1 << 16);
+                xd[xs_dword<PM>(b, P + 1, upad, cu)] = (uint32_t)r2 | ((uint32_t)r3 << 16);
+                if ((q & 31) == 0) {
+                    xsum[b * upad + cu] = tot;
+                    if (xtot) atomicAdd(&xtot[b], tot);
+                }
             }
         }
     }
@@ -105,9 +146,9 @@ __device__ __forceinline__ void stage_units_coherent(uint4* xs, float* xsum, con
 
 // 16-bit input (times its per-column scale) or non-coherent fp32 input, 8 columns per lane and load.
 // Requires 16-byte aligned rows and K % 8 == 0 (st.vec_in).
-template <int DT, int BATCH>
-__device__ __forceinline__ void stage_units_vector(uint4* xs, float* xsum, const StageInput& st, int c0, int cu_n,
-                                                   int upad, int nthreads) {
+template <int DT, int BATCH, bool PM>
+__device__ __forceinline__ void stage_units_vector(uint4* xs, float* xsum, float* xtot, const StageInput& st, int c0,
+                                                   int cu_n, int upad, int nthreads) {
     using E = Elem<DT>;
     constexpr int kBurst = 6;   // 256 lanes x 6 chunks = 12288 columns in one round trip
     const int nchunks = cu_n * 16;
@@ -160,22 +201,20 @@ __device__ __forceinline__ void stage_units_vector(uint4* xs, float* xsum, const
             tot = group_sum(tot, 16);
             if (it < total) {
                 const int cu = q >> 4, i = q & 15;
-                uint4 pk;
-                pk.x = (uint32_t)r[0] | ((uint32_t)r[1] << 16);
-                pk.y = (uint32_t)r[2] | ((uint32_t)r[3] << 16);
-                pk.z = (uint32_t)r[4] | ((uint32_t)r[5] << 16);
-                pk.w = (uint32_t)r[6] | ((uint32_t)r[7] << 16);
-                xs[(b * 16 + i) * upad + cu] = pk;
-                if (i == 0) xsum[b * upad + cu] = tot;
+                store_chunk<PM>(xs, b, i, upad, cu, r);
+                if (i == 0) {
+                    xsum[b * upad + cu] = tot;
+                    if (xtot) atomicAdd(&xtot[b], tot);
+                }
             }
         }
     }
 }
 
 // Element-wise fallback for inputs that allow no 16-byte loads (odd K, unaligned rows).
-template <int DT, int BATCH>
-__device__ __forceinline__ void stage_units_scalar(uint4* xs, float* xsum, const StageInput& st, int c0, int cu_n,
-                                                   int upad, int nthreads) {
+template <int DT, int BATCH, bool PM>
+__device__ __forceinline__ void stage_units_scalar(uint4* xs, float* xsum, float* xtot, const StageInput& st, int c0,
+                                                   int cu_n, int upad, int nthreads) {
     using E = Elem<DT>;
     const int nchunks = cu_n * 16;
 #pragma unroll 1
@@ -207,26 +246,24 @@ __device__ __forceinline__ void stage_units_scalar(uint4* xs, float* xsum, const
             }
             tot = group_sum(tot, 16);
             if (q < nchunks) {
-                uint4 pk;
-                pk.x = (uint32_t)r[0] | ((uint32_t)r[1] << 16);
-                pk.y = (uint32_t)r[2] | ((uint32_t)r[3] << 16);
-                pk.z = (uint32_t)r[4] | ((uint32_t)r[5] << 16);
-                pk.w = (uint32_t)r[6] | ((uint32_t)r[7] << 16);
-                xs[(b * 16 + i) * upad + cu] = pk;
-                if (i == 0) xsum[b * upad + cu] = tot;
+                store_chunk<PM>(xs, b, i, upad, cu, r);
+                if (i == 0) {
+                    xsum[b * upad + cu] = tot;
+                    if (xtot) atomicAdd(&xtot[b], tot);
+                }
             }
         }
     }
 }
 
 // Stage units [c0, c0+cu_n) for BATCH rows.  All threads of the workgroup call this; nthreads is the
-// workgroup size (a multiple of 64).  Must be followed by a barrier before xs/xsum are read.
-template <int DT, int BATCH>
+// workgroup size (a multiple of 64).  Must be followed by a barrier before xs/xsum/xtot are read.
+template <int DT, int BATCH, bool PM = false>
 __device__ __forceinline__ void stage_units(uint4* xs, float* xsum, const StageInput& st, int c0, int cu_n, int upad,
-                                            int nthreads) {
-    if (!st.vec_in || (st.K & 7)) stage_units_scalar<DT, BATCH>(xs, xsum, st, c0, cu_n, upad, nthreads);
-    else if (st.in_f32 && st.in_coherent) stage_units_coherent<DT, BATCH>(xs, xsum, st, c0, cu_n, upad, nthreads);
-    else stage_units_vector<DT, BATCH>(xs, xsum, st, c0, cu_n, upad, nthreads);
+                                            int nthreads, float* xtot = nullptr) {
+    if (!st.vec_in || (st.K & 7)) stage_units_scalar<DT, BATCH, PM>(xs, xsum, xtot, st, c0, cu_n, upad, nthreads);
+    else if (st.in_f32 && st.in_coherent) stage_units_coherent<DT, BATCH, PM>(xs, xsum, xtot, st, c0, cu_n, upad, nthreads);
+    else stage_units_vector<DT, BATCH, PM>(xs, xsum, xtot, st, c0, cu_n, upad, nthreads);
 }
 
 // Signed sum over one unit for BATCH rows: out[b] = sum_{c in unit} sgn(bit c) * x[b][c].
@@ -253,10 +290,10 @@ struct UnitDot<0, BATCH> {   // fp16: single-exponent-bit operands, 5 accumulato
             const uint32_t m11 = wc & M14, m12 = wc & M13, m13 = wc & M12, m14 = wc & M11, m15 = wc & M10;
 #pragma unroll
             for (int b = 0; b < BATCH; ++b) {
-                const uint4 x0 = xs[(b * 16 + 4 * wi + 0) * upad + cu];
-                const uint4 x1 = xs[(b * 16 + 4 * wi + 1) * upad + cu];
-                const uint4 x2 = xs[(b * 16 + 4 * wi + 2) * upad + cu];
-                const uint4 x3 = xs[(b * 16 + 4 * wi + 3) * upad + cu];
+                const uint4 x0 = xs[xs_chunk(b, 4 * wi + 0, upad, cu)];
+                const uint4 x1 = xs[xs_chunk(b, 4 * wi + 1, upad, cu)];
+                const uint4 x2 = xs[xs_chunk(b, 4 * wi + 2, upad, cu)];
+                const uint4 x3 = xs[xs_chunk(b, 4 * wi + 3, upad, cu)];
                 a14[b] = E::dot2(x0.x, m0, a14[b]);
                 a14[b] = E::dot2(x0.y, m1, a14[b]);
                 a13[b] = E::dot2(x0.z, m2, a13[b]);
@@ -306,7 +343,7 @@ struct UnitDot<1, BATCH> {   // bf16: +-1 operand pairs
             for (int b = 0; b < BATCH; ++b) {
                 uint4 xv[4];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) xv[q] = xs[(b * 16 + 4 * wi + q) * upad + cu];
+                for (int q = 0; q < 4; ++q) xv[q] = xs[xs_chunk(b, 4 * wi + q, upad, cu)];
 #pragma unroll
                 for (int j = 0; j < 16; ++j)
                     acc[b][j % NACC] = E::dot2(comp_d(xv[j >> 2], j & 3), sp[j], acc[b][j % NACC]);
@@ -355,8 +392,12 @@ __device__ __forceinline__ uint32_t sign_onto_one(uint32_t shifted, uint32_t one
 
 // acc += signs(w: this lane's unit) x staged activations of unit `cu` (zero contribution when !valid).
 // xs row used by this lane: batch row min(lane & 15, BATCH-1); columns beyond BATCH are never read back.
+// Four accumulators in rotation: consecutive MFMAs do not depend on each other.
+constexpr int kMfmaAccs = 4;
+
 template <int DT, int BATCH>
-__device__ __forceinline__ void unit_mfma(const uint4& w, const uint4* xs, int upad, int cu, bool valid, float4_t& acc) {
+__device__ __forceinline__ void unit_mfma(const uint4& w, const uint4* xs, int upad, int cu, bool valid,
+                                          float4_t (&acc)[kMfmaAccs]) {
     using E = Elem<DT>;
     const int nb = min((int)(threadIdx.x & 15), BATCH - 1);
     const uint32_t one = E::kOnePair;
@@ -371,10 +412,51 @@ __device__ __forceinline__ void unit_mfma(const uint4& w, const uint4* xs, int u
             a.z = sign_onto_one(word << (4 * q + 2), one);
             a.w = sign_onto_one(word << (4 * q + 3), one);
             uint4 b = make_uint4(0, 0, 0, 0);
-            if (valid) b = xs[(nb * 16 + 4 * wi + q) * upad + cu];
-            acc = Mfma16<DT>::run(a, b, acc);
+            if (valid) b = xs[xs_chunk(nb, 4 * wi + q, upad, cu)];
+            acc[q] = Mfma16<DT>::run(a, b, acc[q]);
         }
     }
+}
+
+// fp16 only: the single-exponent-bit operand of the matmul-free loop as the MFMA weight operand.  For a
+// pair position j the four dwords `word_wi & mask` (wi = 0..3) ARE the fp16 pairs c*(b_lo, b_hi) of pair
+// j of the unit's four words, with c = 2^1, 2^-7, 2^-11, 2^-13, 2^-14 for the mask bit 14..10: one AND
+// per dword instead of a shift and a bit-field insert.  Three shifted copies of every word (>>1, <<5,
+// <<10) bring all 16 pair positions onto an exponent bit.  The activation operand comes from the
+// pair-major staging layout, whose chunk j holds exactly those 8 columns.  Each class of c has its own
+// accumulator: acc[0..4] for bit 14..10; sum b*x = acc0/2 + 128 acc1 + 2048 acc2 + 8192 acc3 + 16384 acc4,
+// and the signed sum is (sum of x) - 2 (sum b*x).  Zero words contribute nothing, so "no unit" is w = 0.
+constexpr int kPow2Classes = 5;
+
+template <int BATCH>
+__device__ __forceinline__ void unit_mfma_pow2(const uint4& w, const uint4* xs, int upad, int cu,
+                                               float4_t (&acc)[kPow2Classes]) {
+    constexpr uint32_t M14 = 0x40004000u;
+    const int nb = min((int)(threadIdx.x & 15), BATCH - 1);
+    const uint4* xrow = xs + xs_chunk(nb, 0, upad, cu);
+    uint32_t src[4][4];   // [copy][word]: copy 0 = >>1, 1 = as is, 2 = <<5, 3 = <<10
+#pragma unroll
+    for (int wi = 0; wi < 4; ++wi) {
+        const uint32_t w0 = comp_d(w, wi);
+        src[0][wi] = w0 >> 1; src[1][wi] = w0; src[2][wi] = w0 << 5; src[3][wi] = w0 << 10;
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        // pair j sits at bits (15-j, 31-j): j = 0 -> copy 0 bit 14; j = 1..5 -> copy 1 bits 14..10;
+        // j = 6..10 -> copy 2 bits 14..10; j = 11..15 -> copy 3 bits 14..10
+        const int copy = j == 0 ? 0 : (j + 4) / 5;
+        const int cls = j == 0 ? 0 : (j - 1) % 5;
+        const uint32_t mask = M14 >> cls;
+        uint4 a;
+        a.x = src[copy][0] & mask; a.y = src[copy][1] & mask; a.z = src[copy][2] & mask; a.w = src[copy][3] & mask;
+        const uint4 b = xrow[(size_t)j * upad];
+        acc[cls] = Mfma16<0>::run(a, b, acc[cls]);
+    }
+}
+
+// sum b*x per accumulator element from the five class accumulators (exact power-of-two rescaling)
+__device__ __forceinline__ float4_t pow2_combine(const float4_t (&acc)[kPow2Classes]) {
+    return acc[0] * 0.5f + acc[1] * 128.f + acc[2] * 2048.f + acc[3] * 8192.f + acc[4] * 16384.f;
 }
 
 }  // namespace nq

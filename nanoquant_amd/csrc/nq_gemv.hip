@@ -152,7 +152,7 @@ template <int DT, bool FIRST, int BATCH, int RPW>
 static hipError_t launch_stage(StageArgs a, hipStream_t stream) {
     const int rows_per_block = 4 * (kWave >> a.group_log2) * RPW;
     const int grid = (a.rows + rows_per_block - 1) / rows_per_block;
-    const size_t lds_bytes = (size_t)BATCH * kXsumBytesPerRow + (size_t)BATCH * 16 * (a.chunk_units | 1) * sizeof(uint4);
+    const size_t lds_bytes = (size_t)BATCH * kXsumBytesPerRow + (size_t)xs_chunks(BATCH, a.chunk_units | 1) * sizeof(uint4);
     auto kern = gemv_stage_kernel<DT, FIRST, BATCH, RPW>;
     static bool attr_done = false;  // per template instance; raised once to the full budget
     if (lds_bytes > 64 * 1024 && !attr_done) {
@@ -206,7 +206,7 @@ hipError_t gemv_stage(int dtype, bool first, const uint32_t* bits, const void* i
     while (done < batch) {
         int piece = 16;
         while (piece > batch - done) piece >>= 1;
-        int cap = (kLdsBudget - piece * kXsumBytesPerRow) / (piece * 16 * (int)sizeof(uint4));   // chunk_units|1 must fit
+        int cap = (kLdsBudget - piece * kXsumBytesPerRow - piece * (int)sizeof(uint4)) / (piece * 16 * (int)sizeof(uint4));   // chunk_units|1 must fit
         cap = (cap - 1) & ~1;                                       // even, so that cap|1 <= budget
         if (cap > kXsumStride - 2) cap = kXsumStride - 2;
         a.chunk_units = a.units < cap ? a.units : cap;

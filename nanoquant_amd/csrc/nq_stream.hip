@@ -37,7 +37,9 @@ __device__ unsigned long long* g_nq_trace = nullptr;
 
 namespace nq {
 
-constexpr int kRowBlock = 128;                 // rows finished per pass of a workgroup
+// Rows whose sums a workgroup keeps in LDS at a time (then: barrier, scale, store, barrier).  Few large
+// blocks at small batch; 16 KiB of row sums at most.
+__host__ __device__ constexpr int row_block(int batch) { return batch == 1 ? 1024 : batch == 2 ? 512 : batch == 4 ? 256 : 128; }
 // Same-address device-scope atomics serialise at the memory side (tens of ns each), so completion
 // counts are spread over kSubCounters addresses per stage and kExitSubs addresses for the exit count,
 // one 64-byte line each.
@@ -50,20 +52,39 @@ constexpr int kCounterStride = 8;              // 64-bit words between sub-count
 // is complete in launch g when its sub-counters add up to (g+1) * seg_count(s).
 constexpr int kStreamLdsMax = 144 * 1024;      // staged activations + row accumulators, upper bound
 
-__device__ __forceinline__ uint4 load_unit(const RunStage& st, int row, int unit) {
-    const uint32_t* p = st.bits + (size_t)row * st.words + 4 * unit;
-    if (st.vec_bits) {
-        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-        const u32x4 v = __builtin_nontemporal_load((const u32x4*)p);
-        return make_uint4(v.x, v.y, v.z, v.w);
+// The packed words of one stage as a raw buffer: one 16-byte load per unit whatever the row alignment
+// (buffer loads need dword alignment only), zeros past the end of the matrix, and "no load" expressed
+// as an offset past the end instead of a branch -- with exactly one load instruction per loop trip the
+// compiler can leave younger fetches in flight (vmcnt counting) instead of waiting for all of them.
+struct BitsView {
+    __amdgpu_buffer_rsrc_t rsrc;
+    int words;      // 32-bit words per row
+    int ragged;     // words % 4 != 0: the last unit of a row holds fewer than 4 words
+};
+
+__device__ __forceinline__ BitsView bits_view(const RunStage& st) {
+    BitsView v;
+    v.rsrc = raw_buffer(st.bits, (uint32_t)((size_t)st.rows * st.words * sizeof(uint32_t)));
+    v.words = st.words;
+    v.ragged = (st.words & 3) != 0;
+    return v;
+}
+
+__device__ __forceinline__ uint4 load_unit(const BitsView& v, int row, int unit, bool live) {
+    const uint32_t off = live ? ((uint32_t)row * (uint32_t)v.words + 4u * (uint32_t)unit) * 4u : kPastEnd;
+    const u32x4_t w = __builtin_amdgcn_raw_buffer_load_b128(v.rsrc, off, 0, 2 /* nt: streamed once */);
+    return make_uint4(w.x, w.y, w.z, w.w);
+}
+
+// To be applied where a fetched unit is consumed (not where it is fetched: that would wait for the load):
+// the last unit of a ragged row holds fewer than 4 words of it, the rest belong to the next row.
+__device__ __forceinline__ void trim_unit(const BitsView& v, uint4& w, int unit) {
+    if (v.ragged) {
+        const int left = v.words - 4 * unit;
+        if (left < 4) w.w = 0;
+        if (left < 3) w.z = 0;
+        if (left < 2) w.y = 0;
     }
-    uint4 w = make_uint4(0, 0, 0, 0);
-    const int left = st.words - 4 * unit;
-    w.x = p[0];
-    if (left > 1) w.y = p[1];
-    if (left > 2) w.z = p[2];
-    if (left > 3) w.w = p[3];
-    return w;
 }
 
 // Items of the MFMA path that each wavefront of a workgroup takes (contiguous runs).
@@ -78,10 +99,13 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
     using E = Elem<DT>;
     constexpr int kStreamThreads = THREADS;
     constexpr int kWaves = THREADS / kWave;
+    constexpr int kRowBlock = row_block(BATCH);
     extern __shared__ uint4 lds_raw[];
+    constexpr bool kPow2Mfma = MFMA && DT == 0;                 // fp16 MFMA path: single-bit operands, pair-major x
     float* racc = (float*)lds_raw;                              // [kRowBlock][BATCH] row sums
-    float* xsum = racc + kRowBlock * BATCH;                     // [BATCH][kXsumStride] per-unit input sums
-    uint4* xs = lds_raw + ((kRowBlock + kXsumStride) * BATCH * sizeof(float)) / sizeof(uint4);
+    float* xtot = racc + kRowBlock * BATCH;                     // [16] sum of the staged input per batch row
+    float* xsum = xtot + 16;                                    // [BATCH][kXsumStride] per-unit input sums
+    uint4* xs = lds_raw + ((kRowBlock + kXsumStride) * BATCH * sizeof(float) + 64) / sizeof(uint4);
     __shared__ int s_flag;
     const int tid = threadIdx.x;
     const int wg = blockIdx.x;
@@ -109,6 +133,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
         for (int sg = seg_begin; sg < seg_end; ++sg) {
             const RunSegment seg = segs[sg];
             const RunStage st = stages[seg.stage];
+            const BitsView bv = bits_view(st);
             const int chunk_units = min(st.units, chunk_cap);
             const int upad = chunk_units | 1;
             const bool one_chunk = chunk_units == st.units;
@@ -125,11 +150,11 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                 const int nr0 = min(seg.row_end - seg.row_begin, kRowBlock);
                 const int item0 = (tid >> 6) * mfma_items_per_wave(((nr0 + 15) >> 4) * ng0, kWaves);
                 const int u0 = 4 * (item0 % ng0) + ((tid & 63) >> 4);
-                if (item0 < ((nr0 + 15) >> 4) * ng0 && u0 < chunk_units)
-                    wnext = load_unit(st, min(seg.row_begin + 16 * (item0 / ng0) + (tid & 15), st.rows - 1), u0);
+                wnext = load_unit(bv, min(seg.row_begin + 16 * (item0 / ng0) + (tid & 15), st.rows - 1), u0,
+                                  item0 < ((nr0 + 15) >> 4) * ng0 && u0 < chunk_units);
             } else {
                 const int nr0 = min(seg.row_end - seg.row_begin, kRowBlock);
-                if (tid < nr0 * chunk_units) wnext = load_unit(st, seg.row_begin + tid / chunk_units, tid % chunk_units);
+                wnext = load_unit(bv, seg.row_begin + tid / chunk_units, tid % chunk_units, tid < nr0 * chunk_units);
             }
 
             if ((st.dep >= 0 || st.dep2 >= 0) && !aborted) {
@@ -184,7 +209,13 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                         const int cu_n = min(chunk_units, st.units - c0);
                         if (!(one_chunk && staged)) {
                             if (c0) lds_barrier();
-                            stage_units<DT, BATCH>(xs, xsum, sin, c0, cu_n, upad, kStreamThreads);
+                            if (kPow2Mfma && c0 == 0) {
+                                // every reader of the previous total has passed a barrier by now
+                                if (tid < 16) xtot[tid] = 0.f;
+                                lds_barrier();
+                            }
+                            stage_units<DT, BATCH, kPow2Mfma>(xs, xsum, sin, c0, cu_n, upad, kStreamThreads,
+                                                              kPow2Mfma ? xtot : nullptr);
                             staged = true;
                         }
                         lds_barrier();                           // xs / xsum / zeroed racc visible
@@ -198,53 +229,105 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                             const int nitems = ((nr + 15) >> 4) * ngroups;
                             const int per = mfma_items_per_wave(nitems, kWaves);
                             const int it_begin = wave * per, it_end = min(it_begin + per, nitems);
-                            float4_t acc = {0.f, 0.f, 0.f, 0.f};
+                            constexpr int kAccs = kPow2Mfma ? kPow2Classes : kMfmaAccs;
+                            float4_t acc[kAccs];
+#pragma unroll
+                            for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
                             uint4 w = wnext;                             // very first fetch of the slice
                             if ((rb != seg.row_begin || c0 != 0) && it_begin < it_end) {
-                                w = make_uint4(0, 0, 0, 0);
                                 const int u = 4 * (it_begin % ngroups) + g;
-                                if (u < cu_n) w = load_unit(st, min(rb + 16 * (it_begin / ngroups) + r16, st.rows - 1), c0 + u);
+                                w = load_unit(bv, min(rb + 16 * (it_begin / ngroups) + r16, st.rows - 1), c0 + u, u < cu_n);
                             }
 #pragma unroll 1
                             for (int it = it_begin; it < it_end; ++it) {
                                 const int rg = 16 * (it / ngroups), u = 4 * (it % ngroups) + g;
-                                uint4 wpre = make_uint4(0, 0, 0, 0);
-                                if (it + 1 < it_end) {
-                                    const int un = 4 * ((it + 1) % ngroups) + g;
-                                    if (un < cu_n) wpre = load_unit(st, min(rb + 16 * ((it + 1) / ngroups) + r16, st.rows - 1), c0 + un);
-                                }
-                                unit_mfma<DT, BATCH>(w, xs, upad, u, u < cu_n, acc);
+                                const int un = 4 * ((it + 1) % ngroups) + g;
+                                const uint4 wpre = load_unit(bv, min(rb + 16 * ((it + 1) / ngroups) + r16, st.rows - 1), c0 + un,
+                                                             it + 1 < it_end && un < cu_n);
+                                trim_unit(bv, w, c0 + u);
+                                if constexpr (kPow2Mfma) unit_mfma_pow2<BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
+                                else unit_mfma<DT, BATCH>(w, xs, upad, u, u < cu_n, acc);
                                 w = wpre;
                                 if (it + 1 == it_end || (it + 1) % ngroups == 0) {
-                                    // acc[v] = partial sum of row rg + 4*g + v for batch row r16
+                                    // sum[v] = partial sum of row rg + 4*g + v for batch row r16
+                                    float4_t sum;
+                                    if constexpr (kPow2Mfma) sum = pow2_combine(acc) * -2.f;   // + sum of x at the end
+                                    else sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
                                     if (r16 < BATCH) {
 #pragma unroll
                                         for (int v = 0; v < 4; ++v)
-                                            if (rg + 4 * g + v < nr) atomicAdd(&racc[(rg + 4 * g + v) * BATCH + r16], acc[v]);
+                                            if (rg + 4 * g + v < nr) atomicAdd(&racc[(rg + 4 * g + v) * BATCH + r16], sum[v]);
                                     }
-                                    acc = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                                    for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
                                 }
                             }
                         } else {
                             const int total = nr * cu_n;
-                            int row_l = tid / cu_n, cu = tid % cu_n;
+                            // Lane t takes the (row, unit) pairs t, t + T, t + 2T, ... of the block (row-major), so
+                            // the lanes of a wavefront hold consecutive units of one to a few rows.  Two fetches
+                            // are kept in flight ahead of the arithmetic.  Row sums: lanes of the same row are
+                            // summed across the wavefront first and one lane adds the total to the row
+                            // accumulator -- 64 lanes adding to one LDS address serialise and cost a third of the
+                            // loop otherwise.  Every lane of a wavefront takes every trip (cross-lane sums).
+                            const int lane = tid & 63;
+                            // 0: per-lane adds (a wavefront spans many rows); 1: cu_n is 16, 32 or a multiple of 64,
+                            // rows coincide with aligned lane groups; 2: rows start anywhere in the wavefront
+                            const int sum_group = (cu_n & 63) == 0 ? 64 : cu_n;
+                            const int sum_mode = cu_n < 16 ? 0 : (sum_group == 16 || sum_group == 32 || sum_group == 64) ? 1 : 2;
+                            // Three fetch registers in rotation (trip k uses A, k+1 uses B, k+2 uses C, each
+                            // refilled for three trips later right after its use): nothing in flight is ever
+                            // copied, so the wait before a unit's arithmetic leaves the two younger fetches out.
                             const int srow = kStreamThreads / cu_n, scu = kStreamThreads % cu_n;
-                            uint4 w = wnext;                         // first block, chunk 0: fetched before the wait
-                            if ((rb != seg.row_begin || c0 != 0) && tid < total) w = load_unit(st, rb + row_l, c0 + cu);
-    #pragma unroll 1
-                            for (int f = tid; f < total; f += kStreamThreads) {
-                                // next unit of this lane: put its fetch in flight before the arithmetic
-                                int nrow = row_l + srow, ncu = cu + scu;
-                                if (ncu >= cu_n) { ncu -= cu_n; ++nrow; }
-                                uint4 wpre = make_uint4(0, 0, 0, 0);
-                                if (f + kStreamThreads < total) wpre = load_unit(st, rb + nrow, c0 + ncu);
+                            const int srow3 = 3 * kStreamThreads / cu_n, scu3 = 3 * kStreamThreads % cu_n;
+                            int row_a = tid / cu_n, cu_a = tid % cu_n;
+                            int row_b = row_a + srow, cu_b = cu_a + scu;
+                            if (cu_b >= cu_n) { cu_b -= cu_n; ++row_b; }
+                            int row_c = row_b + srow, cu_c = cu_b + scu;
+                            if (cu_c >= cu_n) { cu_c -= cu_n; ++row_c; }
+                            uint4 wa = wnext;                        // first block, chunk 0: fetched before the wait
+                            if (rb != seg.row_begin || c0 != 0) wa = load_unit(bv, rb + row_a, c0 + cu_a, tid < total);
+                            uint4 wb = load_unit(bv, rb + row_b, c0 + cu_b, tid + kStreamThreads < total);
+                            uint4 wc = load_unit(bv, rb + row_c, c0 + cu_c, tid + 2 * kStreamThreads < total);
+                            auto step = [&](uint4& w, int& row_l, int& cu, int f) {
+                                const bool valid = f < total;
                                 float part[BATCH];
-                                UnitDot<DT, BATCH>::run(w, xs, xsum, upad, cu, part);
-    #pragma unroll
-                                for (int b = 0; b < BATCH; ++b) atomicAdd(&racc[row_l * BATCH + b], part[b]);
-                                w = wpre;
-                                row_l = nrow;
-                                cu = ncu;
+                                trim_unit(bv, w, c0 + cu);
+                                UnitDot<DT, BATCH>::run(w, xs, xsum, upad, valid ? cu : 0, part);
+                                const int row_now = row_l;
+                                // refill this register for three trips later
+                                row_l += srow3; cu += scu3;
+                                if (cu >= cu_n) { cu -= cu_n; ++row_l; }
+                                w = load_unit(bv, rb + row_l, c0 + cu, f + 3 * kStreamThreads < total);
+                                if (sum_mode == 1) {
+                                    // the group's total arrives in its last 16 lanes; the first of them adds it
+#pragma unroll
+                                    for (int b = 0; b < BATCH; ++b) {
+                                        const float tot = group_sum_tail(valid ? part[b] : 0.f, sum_group);
+                                        if (valid && (lane & (sum_group - 1)) == sum_group - 16) atomicAdd(&racc[row_now * BATCH + b], tot);
+                                    }
+                                } else if (sum_mode == 2) {
+                                    const int r_lo = __builtin_amdgcn_readfirstlane(row_now);
+                                    const int r_hi = (f - lane + 63 < total) ? __builtin_amdgcn_readlane(row_now, 63) : nr - 1;
+                                    for (int r = r_lo; r <= r_hi; ++r) {
+#pragma unroll
+                                        for (int b = 0; b < BATCH; ++b) {
+                                            const float tot = group_sum_tail((valid && row_now == r) ? part[b] : 0.f, 64);
+                                            if (lane == 63) atomicAdd(&racc[r * BATCH + b], tot);
+                                        }
+                                    }
+                                } else if (valid) {
+#pragma unroll
+                                    for (int b = 0; b < BATCH; ++b) atomicAdd(&racc[row_now * BATCH + b], part[b]);
+                                }
+                            };
+#pragma unroll 1
+                            for (int f = tid; f - lane < total; f += 3 * kStreamThreads) {   // wave-uniform trip counts
+                                step(wa, row_a, cu_a, f);
+                                if (f + kStreamThreads - lane >= total) break;
+                                step(wb, row_b, cu_b, f + kStreamThreads);
+                                if (f + 2 * kStreamThreads - lane >= total) break;
+                                step(wc, row_c, cu_c, f + 2 * kStreamThreads);
                             }
                         }
                         }
@@ -253,6 +336,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                     for (int i = tid; i < nr * BATCH; i += kStreamThreads) {
                         const int row = rb + i / BATCH, b = i % BATCH;
                         float v = racc[i];
+                        if constexpr (kPow2Mfma) v += xtot[b];
                         if (st.s_row) v *= E::to_float(st.s_row[row]);
                         const size_t o = (size_t)b * st.out_stride + row;
                         if (st.addend) {
@@ -304,29 +388,35 @@ size_t stream_counter_bytes(int nstages) {
 
 // ---- host side --------------------------------------------------------------------------------
 static void stream_lds_plan(int batch, int max_units, int* chunk_cap_out, size_t* lds_out) {
-    const int racc_bytes = (kRowBlock + kXsumStride) * batch * (int)sizeof(float);
-    int chunk_cap = (kStreamLdsMax - racc_bytes) / (batch * 16 * (int)sizeof(uint4));
+    const int racc_bytes = (row_block(batch) + kXsumStride) * batch * (int)sizeof(float) + 64;
+    int chunk_cap = (kStreamLdsMax - racc_bytes - batch * (int)sizeof(uint4)) / (batch * 16 * (int)sizeof(uint4));
     chunk_cap = (chunk_cap - 1) & ~1;
     if (chunk_cap > kXsumStride - 2) chunk_cap = kXsumStride - 2;
     const int chunk_units = max_units < chunk_cap ? max_units : chunk_cap;
     *chunk_cap_out = chunk_cap;
-    *lds_out = (size_t)racc_bytes + (size_t)batch * 16 * (chunk_units | 1) * sizeof(uint4);
+    *lds_out = (size_t)racc_bytes + (size_t)xs_chunks(batch, chunk_units | 1) * sizeof(uint4);
 }
 
-// Workgroup size by batch.  Every workgroup stages the whole input vector of its stage, so larger
-// workgroups mean less staging traffic per row: decisive from batch 4 up (batch 16: 211 -> 93 us per
-// Llama-2-7B layer going from 256 to 1024 lanes).  At batch 1 four independent 256-lane workgroups per
-// CU overlap each other's staging and arithmetic better than one large one (32.7 vs 35.0 us); the
-// matmul-free batch-2 kernel needs more than the 128 registers a 1024-lane workgroup leaves per lane.
+// Which arithmetic and which workgroup size, by element type and batch (measured on Llama-2-7B layers):
+//  * fp16, every batch: MFMA with single-exponent-bit weight operands (one AND per operand dword).  At batch 1
+//    it beats the matmul-free loop when a launch covers one layer (27.5 vs 31.3 us) and loses a little in
+//    long run lists (15.2 vs 14.1 us per layer), where the launch latencies it saves do not matter.
+//  * bf16: batch 1 matmul-free (+-1 operands, dot2), batch >= 2 MFMA with +-1 operands decoded in registers.
+// Every workgroup stages the whole input vector of its stage, so larger workgroups mean less staging
+// traffic per row: decisive for the MFMA path (batch 16: 211 -> 80 us per layer going from 256 to 1024
+// lanes).  The matmul-free batch-1 kernel prefers four independent 256-lane workgroups per CU, which overlap
+// each other's staging and arithmetic (32.7 vs 35.0 us with one 1024-lane workgroup).
+#ifndef NQ_STREAM_MFMA
+#define NQ_STREAM_MFMA(DT, BATCH) ((BATCH) >= 2 || (DT) == 0)
+#endif
 #ifndef NQ_STREAM_THREADS
-#define NQ_STREAM_THREADS(BATCH) ((BATCH) == 1 ? 256 : (BATCH) == 2 ? 512 : 1024)
+#define NQ_STREAM_THREADS(DT, BATCH) ((BATCH) >= 2 ? 1024 : (DT) == 0 ? 512 : 256)
 #endif
 
 template <int DT, int BATCH>
 struct StreamKernel {
-    // batches of 4 and more go through the MFMA units; 1 and 2 stay matmul-free
-    static constexpr bool kMfma = BATCH >= 4;
-    static constexpr int kThreads = NQ_STREAM_THREADS(BATCH);
+    static constexpr bool kMfma = NQ_STREAM_MFMA(DT, BATCH);
+    static constexpr int kThreads = NQ_STREAM_THREADS(DT, BATCH);
     static constexpr auto fn = gemv_stream_kernel<DT, BATCH, kMfma, kThreads>;
 };
 
