@@ -60,7 +60,7 @@ constexpr int kCacheAgentCoherent = 16;   // sc1: served coherently at device sc
 //   chunk-major (PM = false): 16-byte chunk i = P >> 2 holds pairs 4i..4i+3 = 8 consecutive columns;
 //   pair-major  (PM = true):  16-byte chunk j = P & 15 holds pair j of each of the four 32-column words
 //                             (dword wi = P >> 4), the order in which one sign-bit position of the
-//                             four words of a unit addresses the columns.
+//                             four words of a unit addresses the columns; chunks are stored unit by unit.
 // Returns the dword index into xs.
 // 16-byte chunk index of (batch row b, chunk i, unit cu).  The batch-row pitch 16*upad + 1 chunks is
 // 4 dwords off a multiple of 64: the 16 lanes of an MFMA operand read that differ only in the batch row
@@ -69,9 +69,13 @@ __device__ __forceinline__ int xs_chunk(int b, int i, int upad, int cu) { return
 // chunks of staged input for `batch` rows
 __host__ __device__ constexpr int xs_chunks(int batch, int upad) { return batch * (16 * upad + 1); }
 
+// Pair-major chunks are stored unit by unit (chunk j of unit cu at b*pitch + 16*cu + j): the 16 reads of
+// one unit differ by compile-time offsets.
+__device__ __forceinline__ int xs_chunk_pm(int b, int j, int upad, int cu) { return b * (16 * upad + 1) + 16 * cu + j; }
+
 template <bool PM>
 __device__ __forceinline__ int xs_dword(int b, int P, int upad, int cu) {
-    if constexpr (PM) return xs_chunk(b, P & 15, upad, cu) * 4 + (P >> 4);
+    if constexpr (PM) return xs_chunk_pm(b, P & 15, upad, cu) * 4 + (P >> 4);
     else return xs_chunk(b, P >> 2, upad, cu) * 4 + (P & 3);
 }
 
@@ -433,7 +437,7 @@ __device__ __forceinline__ void unit_mfma_pow2(const uint4& w, const uint4* xs, 
                                                float4_t (&acc)[kPow2Classes]) {
     constexpr uint32_t M14 = 0x40004000u;
     const int nb = min((int)(threadIdx.x & 15), BATCH - 1);
-    const uint4* xrow = xs + xs_chunk(nb, 0, upad, cu);
+    const uint4* xrow = xs + xs_chunk_pm(nb, 0, upad, cu);
     uint32_t src[4][4];   // [copy][word]: copy 0 = >>1, 1 = as is, 2 = <<5, 3 = <<10
 #pragma unroll
     for (int wi = 0; wi < 4; ++wi) {
@@ -449,7 +453,7 @@ __device__ __forceinline__ void unit_mfma_pow2(const uint4& w, const uint4* xs, 
         const uint32_t mask = M14 >> cls;
         uint4 a;
         a.x = src[copy][0] & mask; a.y = src[copy][1] & mask; a.z = src[copy][2] & mask; a.w = src[copy][3] & mask;
-        const uint4 b = xrow[(size_t)j * upad];
+        const uint4 b = xrow[j];
         acc[cls] = Mfma16<0>::run(a, b, acc[cls]);
     }
 }

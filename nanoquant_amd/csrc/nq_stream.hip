@@ -148,7 +148,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                 // unit l >> 4)
                 const int ng0 = (chunk_units + 3) >> 2;
                 const int nr0 = min(seg.row_end - seg.row_begin, kRowBlock);
-                const int item0 = (tid >> 6) * mfma_items_per_wave(((nr0 + 15) >> 4) * ng0, kWaves);
+                const int item0 = __builtin_amdgcn_readfirstlane(tid >> 6) * mfma_items_per_wave(((nr0 + 15) >> 4) * ng0, kWaves);
                 const int u0 = 4 * (item0 % ng0) + ((tid & 63) >> 4);
                 wnext = load_unit(bv, min(seg.row_begin + 16 * (item0 / ng0) + (tid & 15), st.rows - 1), u0,
                                   item0 < ((nr0 + 15) >> 4) * ng0 && u0 < chunk_units);
@@ -224,42 +224,48 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                             // Items = (16-row group, 4-unit group), unit group fastest; every wavefront takes a
                             // contiguous run of items, so it mostly stays on one row group and adds its
                             // accumulator to the row sums only when the row group changes.
-                            const int lane = tid & 63, wave = tid >> 6, r16 = lane & 15, g = lane >> 4;
+                            const int lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+                            const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar item arithmetic
                             const int ngroups = (cu_n + 3) >> 2;
                             const int nitems = ((nr + 15) >> 4) * ngroups;
                             const int per = mfma_items_per_wave(nitems, kWaves);
                             const int it_begin = wave * per, it_end = min(it_begin + per, nitems);
                             constexpr int kAccs = kPow2Mfma ? kPow2Classes : kMfmaAccs;
-                            float4_t acc[kAccs];
-#pragma unroll
-                            for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
+                            // (row group, unit group) of the current and of the next item, advanced without divisions
+                            int rg = 16 * (it_begin / ngroups), ub = it_begin % ngroups;
+                            int rg_n = rg, ub_n = ub + 1;
+                            if (ub_n == ngroups) { ub_n = 0; rg_n += 16; }
                             uint4 w = wnext;                             // very first fetch of the slice
-                            if ((rb != seg.row_begin || c0 != 0) && it_begin < it_end) {
-                                const int u = 4 * (it_begin % ngroups) + g;
-                                w = load_unit(bv, min(rb + 16 * (it_begin / ngroups) + r16, st.rows - 1), c0 + u, u < cu_n);
-                            }
+                            if ((rb != seg.row_begin || c0 != 0) && it_begin < it_end)
+                                w = load_unit(bv, min(rb + rg + r16, st.rows - 1), c0 + 4 * ub + g, 4 * ub + g < cu_n);
 #pragma unroll 1
-                            for (int it = it_begin; it < it_end; ++it) {
-                                const int rg = 16 * (it / ngroups), u = 4 * (it % ngroups) + g;
-                                const int un = 4 * ((it + 1) % ngroups) + g;
-                                const uint4 wpre = load_unit(bv, min(rb + 16 * ((it + 1) / ngroups) + r16, st.rows - 1), c0 + un,
-                                                             it + 1 < it_end && un < cu_n);
-                                trim_unit(bv, w, c0 + u);
-                                if constexpr (kPow2Mfma) unit_mfma_pow2<BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
-                                else unit_mfma<DT, BATCH>(w, xs, upad, u, u < cu_n, acc);
-                                w = wpre;
-                                if (it + 1 == it_end || (it + 1) % ngroups == 0) {
-                                    // sum[v] = partial sum of row rg + 4*g + v for batch row r16
-                                    float4_t sum;
-                                    if constexpr (kPow2Mfma) sum = pow2_combine(acc) * -2.f;   // + sum of x at the end
-                                    else sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
-                                    if (r16 < BATCH) {
+                            for (int it = it_begin; it < it_end;) {
+                                // one run = the items of this wavefront that share a row group
+                                const int run = min(ngroups - ub, it_end - it);
+                                const int rg_run = rg;
+                                float4_t acc[kAccs];
 #pragma unroll
-                                        for (int v = 0; v < 4; ++v)
-                                            if (rg + 4 * g + v < nr) atomicAdd(&racc[(rg + 4 * g + v) * BATCH + r16], sum[v]);
-                                    }
+                                for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+                                for (int k = 0; k < run; ++k, ++it) {
+                                    const int u = 4 * ub + g, un = 4 * ub_n + g;
+                                    const uint4 wpre = load_unit(bv, min(rb + rg_n + r16, st.rows - 1), c0 + un,
+                                                                 it + 1 < it_end && un < cu_n);
+                                    trim_unit(bv, w, c0 + u);
+                                    if constexpr (kPow2Mfma) unit_mfma_pow2<BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
+                                    else unit_mfma<DT, BATCH>(w, xs, upad, u, u < cu_n, acc);
+                                    w = wpre;
+                                    rg = rg_n; ub = ub_n;
+                                    if (++ub_n == ngroups) { ub_n = 0; rg_n += 16; }
+                                }
+                                // sum[v] = partial sum of row rg_run + 4*g + v for batch row r16
+                                float4_t sum;
+                                if constexpr (kPow2Mfma) sum = pow2_combine(acc) * -2.f;   // + sum of x at the end
+                                else sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+                                if (r16 < BATCH) {
 #pragma unroll
-                                    for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
+                                    for (int v = 0; v < 4; ++v)
+                                        if (rg_run + 4 * g + v < nr) atomicAdd(&racc[(rg_run + 4 * g + v) * BATCH + r16], sum[v]);
                                 }
                             }
                         } else {
