@@ -27,7 +27,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the headline kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
 # copy kernel of known size (profiles/gemv_stream_llama2_7b_layer_b1.md); valid for the default workload only.
-MEASURED_TRAFFIC_BYTES = 28549760
+MEASURED_TRAFFIC_BYTES = 33866687
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 LLAMA2_7B_LAYER = (("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096),
@@ -204,8 +204,8 @@ def main():
         "us_per_layer": round(ms * 1e3, 3),
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_stream_kernel<fp16, batch 1, 256 lanes> (one launch per layer: 14 stages in 2 phases, "
-                      "1024 resident workgroups)",
+            "kernel": "gemv_stream_kernel<fp16, batch 1, MFMA, 512 lanes> (one launch per layer: 14 stages in 2 phases, "
+                      "512 resident workgroups)",
             "achieved": round(bytes1 / launches_per_step / (launch_us * 1e-6) / 1e9, 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
