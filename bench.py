@@ -228,6 +228,17 @@ def main():
 
     if not args.no_extra:
         extra = {}
+        # measured streaming ceiling of this box: the library's plain copy kernel, 256 MiB read + 256 MiB written
+        nbytes = 256 << 20
+        csrc_ = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_()
+        cdst_ = torch.empty_like(csrc_)
+        copy_fn = lambda: _lib.check(lib.nq_stream_copy(vp(cdst_.data_ptr()), vp(csrc_.data_ptr()), nbytes,
+                                                        vp(torch.cuda.current_stream().cuda_stream)))
+        ms_copy = timed([copy_fn], 20, 3)
+        extra["hbm_copy_kernel"] = {"GBps_read_plus_write": round(2 * nbytes / (ms_copy * 1e-3) / 1e9, 1),
+                                    "note": "plain 16-byte copy kernel, 256 MiB each way: a measured ceiling for streaming "
+                                            "kernels on this box (vendor peak 8000 GB/s)"}
+        del csrc_, cdst_
         for b in (4, 16):
             io = make_io(b)
             lists = make_runlists(io, b)
@@ -374,10 +385,26 @@ def main():
                 break
         times.sort()
         med = times[len(times) // 2]
+        # the reference module's default dtype is bf16 (modules/linear.py:27): same pass in bf16, fewer repeats
+        bf_terms = [tuple(t.to(torch.bfloat16) for t in term) for term in cpu_terms]
+        bf_times = []
+        for _ in range(2):
+            for (x, vt, u, s_in, s_mid, s_out) in bf_terms:
+                oracle.torch_dense_forward(x, vt, u, s_in, s_mid, s_out)
+        t_bf_end = time.perf_counter() + max(2.0, args.cpu_seconds / 4)
+        while len(bf_times) < 5 or (time.perf_counter() < t_bf_end and len(bf_times) < 50):
+            t0 = time.perf_counter()
+            for (x, vt, u, s_in, s_mid, s_out) in bf_terms:
+                oracle.torch_dense_forward(x, vt, u, s_in, s_mid, s_out)
+            bf_times.append(time.perf_counter() - t0)
+            if time.perf_counter() > t_bf_end + 20:
+                break
+        bf_times.sort()
         result["cpu_baseline"] = {
             "value": round(bytes1 / med / 1e9, 3),
             "unit": "GB/s",
             "us_per_layer": round(med * 1e6, 1),
+            "us_per_layer_bf16": round(bf_times[len(bf_times) // 2] * 1e6, 1),
             "cores": torch.get_num_threads(),
             "kind": "port",
             "sample": "same 7-linear layer, batch 1, fp32 dense +-1 factors through two F.linear per linear "

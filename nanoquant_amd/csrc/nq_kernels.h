@@ -43,6 +43,9 @@ hipError_t gemv_stream(int dtype, int batch, const RunStage* stages, int nstages
                        const RunSegment* segs, unsigned long long* counters, unsigned* status, int nwg, int max_units,
                        hipStream_t stream);
 
+// One stage on its own through the run-list kernel (no tables, no counters); batch 16 only.
+hipError_t gemv_stream_single(int dtype, int batch, const RunStage& st, hipStream_t stream);
+
 // nq_gemm.hip: C[T,R] = s_out * ((x * s_in) . sgn(W)^T) with W in the 32x256 tile layout.
 // scratch: fp32 [T,R] when gemm_scratch_bytes(T,K,R) > 0.
 size_t gemm_scratch_bytes(int T, int K, int R);

@@ -90,12 +90,13 @@ __device__ __forceinline__ void trim_unit(const BitsView& v, uint4& w, int unit)
 // Items of the MFMA path that each wavefront of a workgroup takes (contiguous runs).
 __host__ __device__ __forceinline__ int mfma_items_per_wave(int nitems, int waves) { return (nitems + waves - 1) / waves; }
 
-template <int DT, int BATCH, bool MFMA, int THREADS>
+template <int DT, int BATCH, bool MFMA, int THREADS, bool SINGLE>
 __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __restrict__ stages, int nstages,
                                                                      int nphases, const int* __restrict__ seg_index,
                                                                      const RunSegment* __restrict__ segs,
                                                                      unsigned long long* counters, unsigned* status,
-                                                                     unsigned spin_limit, int chunk_cap) {
+                                                                     unsigned spin_limit, int chunk_cap,
+                                                                     RunStage single, int single_rows) {
     using E = Elem<DT>;
     constexpr int kStreamThreads = THREADS;
     constexpr int kWaves = THREADS / kWave;
@@ -116,7 +117,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
     // its latency is hidden behind phase 0.
     unsigned long long gen_raw = 0;
     unsigned members = 1;
-    if (tid < kWave) {
+    if (tid < kWave && !SINGLE) {
         const unsigned long long* exit_sub = counters + (size_t)nstages * kSubCounters * kCounterStride;
         const unsigned total = gridDim.x;
         const unsigned sub = (unsigned)wg & (kExitSubs - 1);
@@ -127,12 +128,25 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
 
 #pragma unroll 1
     for (int ph = 0; ph < nphases; ++ph) {
-        const int seg_begin = seg_index[wg * nphases + ph];
-        const int seg_end = seg_index[wg * nphases + ph + 1];
+        // SINGLE: one stage given by value, no tables and no counters; workgroup w takes rows
+        // [w * single_rows, (w + 1) * single_rows)
+        int seg_begin = 0, seg_end = 1;
+        if constexpr (!SINGLE) {
+            seg_begin = seg_index[wg * nphases + ph];
+            seg_end = seg_index[wg * nphases + ph + 1];
+        }
 #pragma unroll 1
         for (int sg = seg_begin; sg < seg_end; ++sg) {
-            const RunSegment seg = segs[sg];
-            const RunStage st = stages[seg.stage];
+            RunSegment seg;
+            RunStage st;
+            if constexpr (SINGLE) {
+                seg = RunSegment{0, wg * single_rows, min(single.rows, (wg + 1) * single_rows), 0};
+                st = single;
+                if (seg.row_end <= seg.row_begin) break;
+            } else {
+                seg = segs[sg];
+                st = stages[seg.stage];
+            }
             const BitsView bv = bits_view(st);
             const int chunk_units = min(st.units, chunk_cap);
             const int upad = chunk_units | 1;
@@ -381,7 +395,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
         if (ph < 3) NQ_MARK(4 + 4 * ph);
     }
 
-    if (tid == 0) {
+    if (tid == 0 && !SINGLE) {
         unsigned long long* exit_sub = counters + (size_t)nstages * kSubCounters * kCounterStride;
         __hip_atomic_fetch_add(exit_sub + (size_t)(wg & (kExitSubs - 1)) * kCounterStride, 1ull, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
@@ -423,7 +437,8 @@ template <int DT, int BATCH>
 struct StreamKernel {
     static constexpr bool kMfma = NQ_STREAM_MFMA(DT, BATCH);
     static constexpr int kThreads = NQ_STREAM_THREADS(DT, BATCH);
-    static constexpr auto fn = gemv_stream_kernel<DT, BATCH, kMfma, kThreads>;
+    static constexpr auto fn = gemv_stream_kernel<DT, BATCH, kMfma, kThreads, false>;
+    static constexpr auto fn_single = gemv_stream_kernel<DT, BATCH, kMfma, kThreads, true>;
 };
 
 template <int DT, int BATCH>
@@ -473,7 +488,7 @@ static hipError_t launch_stream(const RunStage* stages, int nstages, int nphases
 #endif
     using SK = StreamKernel<DT, BATCH>;
     hipLaunchKernelGGL((SK::fn), dim3(nwg), dim3(SK::kThreads), lds, stream, stages, nstages,
-                       nphases, seg_index, segs, counters, status, (unsigned)(1u << 21), chunk_cap);
+                       nphases, seg_index, segs, counters, status, (unsigned)(1u << 21), chunk_cap, RunStage{}, 0);
 #ifdef NQ_TRACE
     if (tbuf && ++calls == 40) {
         (void)hipStreamSynchronize(stream);
@@ -489,6 +504,47 @@ static hipError_t launch_stream(const RunStage* stages, int nstages, int nphases
     }
 #endif
     return hipGetLastError();
+}
+
+// One stage on its own: the same kernel without tables, dependencies or counters.
+template <int DT, int BATCH>
+static hipError_t launch_single(const RunStage& st, hipStream_t stream) {
+    using SK = StreamKernel<DT, BATCH>;
+    int chunk_cap;
+    size_t lds;
+    stream_lds_plan(BATCH, st.units, &chunk_cap, &lds);
+    static bool attr_done = false;
+    if (lds > 64 * 1024 && !attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void*)SK::fn_single, hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    static size_t cached_lds = 0;                // per template instance: the occupancy query is host time
+    static int cached_cap = 0;
+    if (cached_cap <= 0 || cached_lds != lds) {
+        int per_cu = 0, dev = 0, cus = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)SK::fn_single, SK::kThreads, lds) != hipSuccess ||
+            hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+            return hipErrorInvalidValue;
+        cached_cap = per_cu * cus;
+        cached_lds = lds;
+    }
+    const int cap = cached_cap;
+    if (cap <= 0) return hipErrorInvalidValue;
+    // whole 16-row groups per workgroup, as few rows as the resident grid allows
+    const int rows_per_wg = ((st.rows + cap - 1) / cap + 15) & ~15;
+    const int nwg = (st.rows + rows_per_wg - 1) / rows_per_wg;
+    hipLaunchKernelGGL((SK::fn_single), dim3(nwg), dim3(SK::kThreads), lds, stream, (const RunStage*)nullptr, 0, 1,
+                       (const int*)nullptr, (const RunSegment*)nullptr, (unsigned long long*)nullptr, (unsigned*)nullptr,
+                       0u, chunk_cap, st, rows_per_wg);
+    return hipGetLastError();
+}
+
+// Only the batch sizes that the per-linear path sends here are instantiated.
+hipError_t gemv_stream_single(int dtype, int batch, const RunStage& st, hipStream_t stream) {
+    if (batch != 16) return hipErrorInvalidValue;
+    return dtype == 0 ? launch_single<0, 16>(st, stream) : launch_single<1, 16>(st, stream);
 }
 
 #define NQ_STREAM_DISPATCH(CALL)                                          \
