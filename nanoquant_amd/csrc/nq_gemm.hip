@@ -248,6 +248,17 @@ static GemmPlan plan_gemm(int T, int K, int R) {
     // more workgroups, fewer registers, three wavefronts per SIMD.  Two row tiles per wavefront halve the
     // LDS reads per MFMA and win once that still leaves two workgroups for every CU.
     p.tt = 2;
+    {
+        // Few tokens: 32-token blocks give twice the workgroups, which can spare the k-split and with it
+        // the atomics and the finish launch (4096x4096 at 256 tokens: 44 -> 27 us per linear).  Only when
+        // k is short enough for one workgroup to walk it (<= 16 tiles).
+        const int gx1 = (R + 127) / 128, gy1 = (T + 31) / 32;
+        if (gx1 * ((T + 63) / 64) < 256 && gx1 * gy1 >= 128 && K / kTileK <= 16) {
+            p.tt = 1; p.rt = 1; p.gx = gx1; p.gy = gy1;
+            p.ktiles_per_split = K / kTileK; p.ksplit = 1; p.xcd = false;
+            return p;
+        }
+    }
     p.gy = (T + 32 * p.tt - 1) / (32 * p.tt);
     p.rt = ((R + 255) / 256) * p.gy >= 512 ? 2 : 1;
     p.gx = (R + 128 * p.rt - 1) / (128 * p.rt);
@@ -320,6 +331,7 @@ hipError_t gemm_onebit(int dtype, const void* x, const uint32_t* tiles, const vo
     const GemmPlan p = plan_gemm(T, K, R);
     a.ktiles_per_split = p.ktiles_per_split;
     a.xcd_gx = p.xcd ? p.gx : 0;
+    if (p.tt == 1) return dtype == 0 ? launch_gemm<0, 1, 1, 256>(a, p, stream) : launch_gemm<1, 1, 1, 256>(a, p, stream);
     if (dtype == 0) return p.rt == 2 ? launch_gemm<0, 2, 2, 256>(a, p, stream) : launch_gemm<0, 2, 1, 256>(a, p, stream);
     return p.rt == 2 ? launch_gemm<1, 2, 2, 256>(a, p, stream) : launch_gemm<1, 2, 1, 256>(a, p, stream);
 }
