@@ -144,3 +144,25 @@ def test_graph_replay_of_a_run_list(dev):
         assert rl.status() == 0
         for y, e in zip(rl.outputs, eager):
             assert torch.equal(y, e), rep
+
+
+@pytest.mark.parametrize("batch", [2, 16])
+def test_bf16_batches_on_the_mfma_path(dev, batch):
+    # bf16 keeps +-1 weight operands on the MFMA units (no single-bit trick): cover it with ragged ranks too
+    rl = DecodeRunList(batch, torch.bfloat16, dev)
+    refs = []
+    for i, (m, n, r) in enumerate([(512, 1024, 256), (200, 4096, 736), (1376, 512, 96)]):
+        vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, 400 + i)
+        x = oracle.synth_x(batch, n, 400 + i)
+        bf = lambda a: torch.from_numpy(a.astype(np.float32)).to(torch.bfloat16)
+        xt, si, sm, so = bf(x), bf(s_in), bf(s_mid), bf(s_out)
+        rl.add(xt.to(dev), si.to(dev), packing.binary_packer(torch.from_numpy(vt), "half2").to(dev), sm.to(dev),
+               packing.binary_packer(torch.from_numpy(u), "half2").to(dev), so.to(dev))
+        refs.append(oracle.layer_forward(xt.float().numpy(), vt, u, si.float().numpy(), sm.float().numpy(),
+                                         so.float().numpy(), dtype=np.float64))
+    print(f"bf16 run list batch={batch}", flush=True)
+    ys = rl.run()
+    torch.cuda.synchronize()
+    assert rl.status() == 0
+    for y, ref in zip(ys, refs):
+        assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < 1e-2
