@@ -216,7 +216,7 @@ __global__ __launch_bounds__(256) void gemm_onebit_kernel(GemmArgs a) {
 // (wavefront w takes the weight tiles w, w+4, ...) and add their accumulators through LDS at the end.
 // No global atomics, no scratch, no second launch; R/32 x T/32 workgroups, and the wavefronts of a workgroup
 // never wait for each other inside the k loop (each stages its own activation slab).
-template <int DT, bool SCALED>
+template <int DT, bool SCALED, int RT>
 __global__ __launch_bounds__(256) void gemm_kwave_kernel(GemmArgs a) {
     using E = Elem<DT>;
     constexpr int kPitch = slab_pitch<kTileK>();
@@ -225,12 +225,15 @@ __global__ __launch_bounds__(256) void gemm_kwave_kernel(GemmArgs a) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint16_t* slab = slabs + wave * kSlabHalves;
     uint16_t* scale_lds = slab + 32 * kPitch;
-    const int rt = blockIdx.x;                                   // 32-row tile
+    const int rt = blockIdx.x * RT;                              // first of the RT 32-row tiles of this workgroup
+    const int ntiles = min(RT, a.R / 32 - rt);
     const int tok0 = blockIdx.y * 32;
 
-    float16_t acc;
+    float16_t acc[RT];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[r][v] = 0.f;
 
     // the wavefront's slab: 32 tokens x 256 k = 1024 16-byte chunks, 16 per lane
     u32x4_t xr[16];
@@ -246,9 +249,14 @@ __global__ __launch_bounds__(256) void gemm_kwave_kernel(GemmArgs a) {
         if constexpr (SCALED) sr = *(const u32x4_t*)(a.s_in + k0 + 8 * (lane & 31));
     };
     const uint4* tile_ptr = a.tiles + (size_t)rt * a.ktiles * 64 + lane;
-    uint4 wnext = make_uint4(0, 0, 0, 0);
+    const size_t tile_pitch = (size_t)a.ktiles * 64;             // uint4 elements between consecutive row tiles
+    uint4 wnext[RT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) wnext[r] = make_uint4(0, 0, 0, 0);
     if (wave < a.ktiles) {
-        wnext = tile_ptr[(size_t)wave * 64];
+#pragma unroll
+        for (int r = 0; r < RT; ++r)
+            if (r < ntiles) wnext[r] = tile_ptr[r * tile_pitch + (size_t)wave * 64];
         fetch(wave);
     }
 #pragma unroll 1
@@ -262,38 +270,48 @@ __global__ __launch_bounds__(256) void gemm_kwave_kernel(GemmArgs a) {
         if constexpr (SCALED) {
             if (lane < 32) *(u32x4_t*)(scale_lds + 8 * lane) = sr;
         }
-        const uint4 w = wnext;
+        uint4 w[RT];
+#pragma unroll
+        for (int r = 0; r < RT; ++r) w[r] = wnext[r];
         if (kt + 4 < a.ktiles) {
-            wnext = tile_ptr[(size_t)(kt + 4) * 64];
+#pragma unroll
+            for (int r = 0; r < RT; ++r)
+                if (r < ntiles) wnext[r] = tile_ptr[r * tile_pitch + (size_t)(kt + 4) * 64];
             fetch(kt + 4);
         }
 #pragma unroll
         for (int t = 0; t < 16; ++t) {
             const int s = 4 * (t & 3);
-            const uint32_t word = comp4(w, t >> 2);
-            uint4 bfrag;
-            if constexpr (SCALED) {
-                const uint4 sp = *(const uint4*)(scale_lds + 16 * t + 8 * (lane >> 5));
-                bfrag.x = sp.x ^ ((word << (s + 0)) & kSignPair);
-                bfrag.y = sp.y ^ ((word << (s + 1)) & kSignPair);
-                bfrag.z = sp.z ^ ((word << (s + 2)) & kSignPair);
-                bfrag.w = sp.w ^ ((word << (s + 3)) & kSignPair);
-            } else {
-                bfrag.x = ((word << (s + 0)) & kSignPair) | E::kOnePair;
-                bfrag.y = ((word << (s + 1)) & kSignPair) | E::kOnePair;
-                bfrag.z = ((word << (s + 2)) & kSignPair) | E::kOnePair;
-                bfrag.w = ((word << (s + 3)) & kSignPair) | E::kOnePair;
-            }
+            uint4 sp;
+            if constexpr (SCALED) sp = *(const uint4*)(scale_lds + 16 * t + 8 * (lane >> 5));
             const uint4 afrag = *(const uint4*)(slab + (lane & 31) * kPitch + 16 * t + 8 * (lane >> 5));
-            acc = Mfma<DT>::run(afrag, bfrag, acc);
+#pragma unroll
+            for (int r = 0; r < RT; ++r) {
+                const uint32_t word = comp4(w[r], t >> 2);
+                uint4 bfrag;
+                if constexpr (SCALED) {
+                    bfrag.x = sp.x ^ ((word << (s + 0)) & kSignPair);
+                    bfrag.y = sp.y ^ ((word << (s + 1)) & kSignPair);
+                    bfrag.z = sp.z ^ ((word << (s + 2)) & kSignPair);
+                    bfrag.w = sp.w ^ ((word << (s + 3)) & kSignPair);
+                } else {
+                    bfrag.x = ((word << (s + 0)) & kSignPair) | E::kOnePair;
+                    bfrag.y = ((word << (s + 1)) & kSignPair) | E::kOnePair;
+                    bfrag.z = ((word << (s + 2)) & kSignPair) | E::kOnePair;
+                    bfrag.w = ((word << (s + 3)) & kSignPair) | E::kOnePair;
+                }
+                acc[r] = Mfma<DT>::run(afrag, bfrag, acc[r]);
+            }
         }
     }
 
     // ---- add the four partial tiles through LDS (the slabs are free now) ----
     __syncthreads();
-    float* part = (float*)slabs;                                 // [4][16][64] floats = 16 KiB
+    float* part = (float*)slabs;                                 // [RT][4][16][64] floats = RT x 16 KiB
 #pragma unroll
-    for (int v = 0; v < 16; ++v) part[(wave * 16 + v) * 64 + lane] = acc[v];
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) part[((r * 4 + wave) * 16 + v) * 64 + lane] = acc[r][v];
     __syncthreads();
     // Thread (token t, row octet o) of the first 128 threads sums the four partial values of 8 consecutive
     // rows and stores them as one 16-byte chunk.  Accumulator element v of lane l is token
@@ -301,23 +319,29 @@ __global__ __launch_bounds__(256) void gemm_kwave_kernel(GemmArgs a) {
     if (threadIdx.x < 128) {
         const int t = threadIdx.x >> 2, o = threadIdx.x & 3;
         const int v = 4 * (t >> 3) + (t & 3), l0 = 32 * ((t >> 2) & 1) + 8 * o;
-        const int tok = tok0 + t, row0 = rt * 32 + 8 * o;
-        float sums[8];
+        const int tok = tok0 + t;
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-            sums[j] = (part[(0 * 16 + v) * 64 + l0 + j] + part[(1 * 16 + v) * 64 + l0 + j]) +
-                      (part[(2 * 16 + v) * 64 + l0 + j] + part[(3 * 16 + v) * 64 + l0 + j]);
-        u32x4_t sc = {E::kOnePair, E::kOnePair, E::kOnePair, E::kOnePair};
-        if (a.s_out) sc = *(const u32x4_t*)(a.s_out + row0);
-        u32x4_t outv;
+        for (int r = 0; r < RT; ++r) {
+            if (r >= ntiles) break;
+            const int row0 = (rt + r) * 32 + 8 * o;
+            const float* pr = part + (size_t)r * 4 * 16 * 64;
+            float sums[8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t sw = sc[j];
-            const uint16_t lo = E::from_float_sat(sums[2 * j] * E::to_float((uint16_t)(sw & 0xFFFFu)));
-            const uint16_t hi = E::from_float_sat(sums[2 * j + 1] * E::to_float((uint16_t)(sw >> 16)));
-            outv[j] = (uint32_t)lo | ((uint32_t)hi << 16);
+            for (int j = 0; j < 8; ++j)
+                sums[j] = (pr[(0 * 16 + v) * 64 + l0 + j] + pr[(1 * 16 + v) * 64 + l0 + j]) +
+                          (pr[(2 * 16 + v) * 64 + l0 + j] + pr[(3 * 16 + v) * 64 + l0 + j]);
+            u32x4_t sc = {E::kOnePair, E::kOnePair, E::kOnePair, E::kOnePair};
+            if (a.s_out) sc = *(const u32x4_t*)(a.s_out + row0);
+            u32x4_t outv;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t sw = sc[j];
+                const uint16_t lo = E::from_float_sat(sums[2 * j] * E::to_float((uint16_t)(sw & 0xFFFFu)));
+                const uint16_t hi = E::from_float_sat(sums[2 * j + 1] * E::to_float((uint16_t)(sw >> 16)));
+                outv[j] = (uint32_t)lo | ((uint32_t)hi << 16);
+            }
+            if (tok < a.T) *(u32x4_t*)((uint16_t*)a.y + (size_t)tok * a.R + row0) = outv;
         }
-        if (tok < a.T) *(u32x4_t*)((uint16_t*)a.y + (size_t)tok * a.R + row0) = outv;
     }
 }
 
@@ -361,7 +385,12 @@ static GemmPlan plan_gemm(int T, int K, int R) {
         // 32x32 output tiles, wavefronts split k: no k-split scratch, one launch (4096x4096 at 128 tokens:
         // 16.8 vs 22.7 us per linear with the block kernel; no gain above 128 tokens)
         p.kwave = true;
-        p.tt = 1; p.rt = 1; p.gx = R / 32; p.gy = (T + 31) / 32;
+        p.tt = 1; p.gy = (T + 31) / 32;
+        // every 32-row tile re-reads the 32-token activation slab: wider workgroups once there are enough of them
+        // (two per CU; 11008 rows at 128 tokens: 36.4 -> 31.5 us per linear with two row tiles per workgroup)
+        p.rt = 1;
+        while (p.rt < 4 && (R / 32 / (2 * p.rt)) * p.gy >= 512) p.rt *= 2;
+        p.gx = (R / 32 + p.rt - 1) / p.rt;
         p.ktiles_per_split = K / kTileK; p.ksplit = 1; p.xcd = false;
         return p;
     }
@@ -461,8 +490,10 @@ hipError_t gemm_onebit(int dtype, const void* x, const uint32_t* tiles, const vo
             hipLaunchKernelGGL(kern, dim3(p.gx, p.gy), dim3(256), lds, stream, a);
             return hipGetLastError();
         };
-        if (dtype == 0) return scaled ? launch(gemm_kwave_kernel<0, true>) : launch(gemm_kwave_kernel<0, false>);
-        return scaled ? launch(gemm_kwave_kernel<1, true>) : launch(gemm_kwave_kernel<1, false>);
+#define NQ_KW(D, S) (p.rt == 1 ? launch(gemm_kwave_kernel<D, S, 1>) : p.rt == 2 ? launch(gemm_kwave_kernel<D, S, 2>) : launch(gemm_kwave_kernel<D, S, 4>))
+        if (dtype == 0) return scaled ? NQ_KW(0, true) : NQ_KW(0, false);
+        return scaled ? NQ_KW(1, true) : NQ_KW(1, false);
+#undef NQ_KW
     }
     if (p.tt == 1) return dtype == 0 ? launch_gemm<0, 1, 1, 256>(a, p, stream) : launch_gemm<1, 1, 1, 256>(a, p, stream);
     if (dtype == 0) return p.rt == 2 ? launch_gemm<0, 2, 2, 256>(a, p, stream) : launch_gemm<0, 2, 1, 256>(a, p, stream);
