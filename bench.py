@@ -27,7 +27,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the headline kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
 # copy kernel of known size (profiles/gemv_stream_llama2_7b_layer_b1.md); valid for the default workload only.
-MEASURED_TRAFFIC_BYTES = 33866687
+MEASURED_TRAFFIC_BYTES = 33966528
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 LLAMA2_7B_LAYER = (("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096),
