@@ -103,3 +103,33 @@ def test_k_split_matches_single_pass(dev):
     for (m, n, r) in [(128, 4096, 256), (4096, 512, 256)]:
         err = _run_fused(dev, m, n, r, 128, torch.float16, seed=m)
         assert err < TOL[torch.float16], (m, n, r, err)
+
+
+def test_graph_replay_of_the_split_k_path(dev):
+    # k-split partial sums live in a scratch that the finish kernel re-zeroes: replays of a captured call
+    # must equal the eager result every time (no memset nodes involved, the scratch is never cleared by the host)
+    m, n, r, tokens = 512, 4096, 512, 300
+    vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, 77)
+    x = torch.from_numpy(oracle.synth_x(tokens, n, 78)).to(dev)
+    f = lambda a: torch.from_numpy(a).to(dev)
+    packed = packing.marlin_nanoquant_packer(torch.from_numpy(vt.T.copy()).to(dev), torch.from_numpy(u.T.copy()).to(dev),
+                                             f(s_in), f(s_mid), f(s_out))
+    op = torch.ops.binary_kernels.marlin_nanoquant_forward
+    print("graph replay of marlin_nanoquant_forward", flush=True)
+    eager = op(x, *packed).clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        op(x, *packed)                       # the side stream's scratch exists before the capture
+    side.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        y = op(x, *packed)
+    for rep in range(4):
+        y.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager) or oracle.max_rel_err(y.float().cpu().numpy(), eager.float().cpu().numpy()) < 1e-3, rep
+        op(x, *packed)                       # eager work between the replays
+        torch.cuda.synchronize()
