@@ -463,4 +463,235 @@ __device__ __forceinline__ float4_t pow2_combine(const float4_t (&acc)[kPow2Clas
     return acc[0] * 0.5f + acc[1] * 128.f + acc[2] * 2048.f + acc[3] * 8192.f + acc[4] * 16384.f;
 }
 
+// ---- one-bit fp4 weights x fp8 pieces of the input (batch 1..4, fp16 and bf16 alike) ---------------
+// v_mfma_f32_16x16x128_f8f6f4 takes an fp4 (e2m1) A operand and an fp8 (e4m3) B operand.  A 4-bit pattern
+// with a single bit set is a valid e2m1 number (0.5, 1, 2 for bit 0, 1, 2; bit 3 is the sign of zero), so
+// `word & 0x11111111 << p` IS the weight operand "c_p * b" of the eight sign bits at position p of the
+// eight nibbles of a packed word: one AND per 32 bits and class (bit 3 goes through a one-bit shift), and
+// one MFMA multiplies 16 rows x 512 columns of signs.  The input is staged as kQ8Pieces fp8 numbers per
+// element, u = x * s * S ~ q0 + q1 + q2 with q_k = fp8(u - q_0 - .. - q_{k-1}) and S a power of two that brings
+// the largest |u| of the staged slice into [128, 256): every piece carries 4 significant bits, three of them
+// reproduce u to 2^-12 relative or 2^-17 of the slice maximum, whichever is larger (fp16 staging keeps 2^-11
+// relative); all products are exact and accumulate in fp32.  Pieces and batch rows
+// are columns of the B operand: column j = b * kQ8Pieces + piece, at most 16.
+//
+// Operand geometry (measured on gfx950 with one-hot operands): lane (i = l & 15, g = l >> 4) supplies
+//   A (fp4, 4 dwords): row i, k = 32 g + idx, idx = 8 t + e for nibble e of dword t;
+//   B (fp8, 8 dwords): column i, k = 64 (idx >> 4) + 16 g + (idx & 15) for byte idx of the 32.
+// With A dword t = word t of the lane's 16-byte unit (unit 4 ub + g of the row), nibble e at class p is bit
+// 4 e + p of that word, i.e. column 32 t + elem(4 e + p) of the unit, elem(b) = b < 16 ? 2 (15 - b) :
+// 2 (31 - b) + 1 (the "half2" order).  So B lane g needs, for class p, the 16 bytes (words 2 (g & 1),
+// 2 (g & 1) + 1; e = 0..7) of unit 4 ub + (g >> 1) and the same of unit 4 ub + 2 + (g >> 1).
+// LDS layout in 16-byte chunks: chunk(j, u, p, hf) = j * pitch + 8 u + 2 p + hf holds, for column j, unit u,
+// class p, the bytes of words 2 hf, 2 hf + 1 (8 bytes each, e = 0..7).  pitch = 8 * units4 + 1 with units4 the
+// number of staged units rounded up to a multiple of 4 (the padding is staged as zeros).
+constexpr int kQ8Pieces = 3;
+typedef int v8i_t __attribute__((ext_vector_type(8)));
+
+__host__ __device__ constexpr int q8_units4(int units) { return (units + 3) & ~3; }
+__host__ __device__ constexpr int q8_pitch(int units4) { return 8 * units4 + 1; }
+__host__ __device__ constexpr int q8_chunks(int batch, int units4) { return batch * kQ8Pieces * q8_pitch(units4); }
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_mov_u32(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, false);
+}
+
+// Lane q of a quad holds M_q (bytes c = 0..3); returns T with T byte e = byte q of M_{3-e}: a 4x4 byte
+// transpose across the quad with the lane order reversed, two exchange-and-permute steps.
+__device__ __forceinline__ uint32_t quad_transpose_rev(uint32_t m, bool odd, bool upper) {
+    const uint32_t p1 = dpp_mov_u32<0xB1>(m);                       // lane ^ 1
+    const uint32_t y = __builtin_amdgcn_perm(p1, m, odd ? 0x03070105u : 0x06020400u);
+    const uint32_t p2 = dpp_mov_u32<0x4E>(y);                       // lane ^ 2
+    return __builtin_amdgcn_perm(p2, y, upper ? 0x06070203u : 0x00010405u);
+}
+
+// power of two S = 2^(7 - E) for a slice maximum with biased exponent eb = E + 127 (clamped below so that an
+// all-zero slice gives a finite S), and the factor -2 / S that takes an accumulator back
+__device__ __forceinline__ uint32_t q8_exponent(uint32_t max_bits) { return max(max_bits >> 23, 32u); }
+__device__ __forceinline__ float q8_scale(uint32_t eb) { return as_float((261u - eb) << 23); }
+__device__ __forceinline__ float q8_unscale_neg2(uint32_t eb) { return as_float(0x80000000u | ((eb - 6u) << 23)); }
+
+// Stage units [c0, c0 + cu_n) (plus zero padding up to q8_units4(cu_n)) of BATCH rows.  smax[b] (uint32,
+// zeroed by the caller, barrier before) receives the bit pattern of max |u| per batch row, xtot[b] the sum of
+// the staged values.  The wavefronts of the workgroup are divided among the batch rows (nthreads / 64 must be a
+// multiple of BATCH), so a lane reduces maximum and sum over all its chunks before anything crosses lanes.
+// Contains one workgroup barrier; a barrier must follow before the staged data is read.
+template <int DT, int BATCH>
+__device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* smax, float* xtot, const StageInput& st, int c0,
+                                               int cu_n, int pitch, int nthreads) {
+    using E = Elem<DT>;
+    constexpr int kBurst = BATCH >= 4 ? 6 : 3;
+    const int nchunks = q8_units4(cu_n) * 16;            // 8-column chunks per batch row, a multiple of 64
+    const int tpr = nthreads / BATCH;                    // lanes per batch row
+    const int b = threadIdx.x / tpr, tl = threadIdx.x - b * tpr;
+    const int lane = threadIdx.x & 63;
+    const uint32_t esize = st.in_f32 ? 4u : 2u;
+    const bool fast = st.vec_in && (st.K & 7) == 0;
+    const __amdgpu_buffer_rsrc_t rin = raw_buffer(st.in, (uint32_t)(((size_t)(BATCH - 1) * st.in_stride + st.K) * esize));
+    const bool scaled = !st.in_f32 && st.s_col != nullptr;
+    const __amdgpu_buffer_rsrc_t rsc = raw_buffer(scaled ? (const void*)st.s_col : st.in, scaled ? (uint32_t)st.K * 2u : 0u);
+    const bool coherent = st.in_f32 && st.in_coherent;
+
+    auto issue = [&](int q, u32x4_t& ra, u32x4_t& rb) {
+        const int col = c0 * 128 + 8 * q;
+        const bool live = fast && q < nchunks && col < st.K;
+        const uint32_t off = live ? (uint32_t)(((size_t)b * st.in_stride + col) * esize) : kPastEnd;
+        if (coherent) {
+            ra = __builtin_amdgcn_raw_buffer_load_b128(rin, off, 0, kCacheAgentCoherent);
+            rb = __builtin_amdgcn_raw_buffer_load_b128(rin, live ? off + 16u : kPastEnd, 0, kCacheAgentCoherent);
+        } else {
+            ra = __builtin_amdgcn_raw_buffer_load_b128(rin, off, 0, kCacheDefault);
+            if (st.in_f32) rb = __builtin_amdgcn_raw_buffer_load_b128(rin, live ? off + 16u : kPastEnd, 0, kCacheDefault);
+            else rb = __builtin_amdgcn_raw_buffer_load_b128(rsc, live ? (uint32_t)col * 2u : kPastEnd, 0, kCacheDefault);
+        }
+    };
+    // the 8 values of chunk q as fp32, input scale applied; running maximum of |v| and sum
+    auto values = [&](int q, const u32x4_t& ra, const u32x4_t& rb, float (&v)[8], float& m, float& tot) {
+        if (fast) {
+            if (!st.in_f32) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t xw = ra[e], sw = scaled ? rb[e] : E::kOnePair;
+                    v[2 * e] = E::to_float(xw & 0xFFFFu) * E::to_float(sw & 0xFFFFu);
+                    v[2 * e + 1] = E::to_float(xw >> 16) * E::to_float(sw >> 16);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = as_float(ra[e]);
+                    v[4 + e] = as_float(rb[e]);
+                }
+            }
+        } else {
+            // element-wise fallback: odd K or rows that allow no 16-byte loads
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int c = c0 * 128 + 8 * q + e;
+                float t = 0.f;
+                if (q < nchunks && c < st.K) {
+                    if (!st.in_f32) {
+                        t = E::to_float(((const uint16_t*)st.in)[(size_t)b * st.in_stride + c]);
+                        if (st.s_col) t *= E::to_float(st.s_col[c]);
+                    } else if (st.in_coherent) {
+                        t = __builtin_bit_cast(float, __hip_atomic_load((const uint32_t*)st.in + (size_t)b * st.in_stride + c,
+                                                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+                    } else {
+                        t = ((const float*)st.in)[(size_t)b * st.in_stride + c];
+                    }
+                }
+                v[e] = t;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            m = fmaxf(m, fabsf(v[e]));
+            tot += v[e];
+        }
+    };
+    // wavefront maximum and sum into smax / xtot: one LDS atomic each per wavefront
+    auto publish = [&](float m, float tot) {
+        uint32_t mb = __builtin_bit_cast(uint32_t, m);
+        mb = max(mb, dpp_mov_u32<0xB1>(mb));
+        mb = max(mb, dpp_mov_u32<0x4E>(mb));
+        mb = max(mb, dpp_mov_u32<0x141>(mb));
+        mb = max(mb, dpp_mov_u32<0x140>(mb));
+        mb = max(mb, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mb, 0x142, 0xA, 0xF, false));
+        mb = max(mb, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mb, 0x143, 0xC, 0xF, false));
+        tot = group_sum_tail(tot, 64);
+        if (lane == 63) {
+            atomicMax(&smax[b], mb);
+            atomicAdd(&xtot[b], tot);
+        }
+    };
+    // pieces of chunk q into LDS: q_k = fp8(u - q_0 - .. - q_{k-1}), all on the scale of u
+    auto quantize = [&](int q, float (&v)[8], float S) {
+        const int cu = q >> 4, t = (q >> 2) & 3, qq = q & 3;
+        float u[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) u[e] = v[e] * S;
+        uint2* dst = (uint2*)xq + 2 * ((size_t)(b * kQ8Pieces) * pitch + 8 * cu + 2 * qq + (t >> 1)) + (t & 1);
+#pragma unroll
+        for (int k = 0; k < kQ8Pieces; ++k) {
+            // class p = 0..3 <-> elements 6, 4, 2, 0 (even) and 7, 5, 3, 1 (odd) of the chunk
+            int lo = __builtin_amdgcn_cvt_pk_fp8_f32(u[6], u[4], 0, false);
+            lo = __builtin_amdgcn_cvt_pk_fp8_f32(u[2], u[0], lo, true);
+            int hi = __builtin_amdgcn_cvt_pk_fp8_f32(u[7], u[5], 0, false);
+            hi = __builtin_amdgcn_cvt_pk_fp8_f32(u[3], u[1], hi, true);
+            if (k + 1 < kQ8Pieces) {
+                const auto l0 = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false), l1 = __builtin_amdgcn_cvt_pk_f32_fp8(lo, true);
+                const auto h0 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false), h1 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
+                u[6] -= l0[0]; u[4] -= l0[1]; u[2] -= l1[0]; u[0] -= l1[1];
+                u[7] -= h0[0]; u[5] -= h0[1]; u[3] -= h1[0]; u[1] -= h1[1];
+            }
+            uint2 out;
+            out.x = quad_transpose_rev((uint32_t)lo, lane & 1, lane & 2);
+            out.y = quad_transpose_rev((uint32_t)hi, lane & 1, lane & 2);
+            if (q < nchunks) dst[(size_t)k * pitch * 2] = out;
+        }
+    };
+
+    if (nchunks <= tpr * kBurst) {
+        // everything in one round trip; the values stay in registers across the barrier
+        u32x4_t ra[kBurst], rb[kBurst];
+        float v[kBurst][8];
+        float m = 0.f, tot = 0.f;
+#pragma unroll
+        for (int j = 0; j < kBurst; ++j) issue(tl + j * tpr, ra[j], rb[j]);
+#pragma unroll
+        for (int j = 0; j < kBurst; ++j) values(tl + j * tpr, ra[j], rb[j], v[j], m, tot);
+        publish(m, tot);
+        lds_barrier();
+        const float S = q8_scale(q8_exponent(smax[b]));
+#pragma unroll
+        for (int j = 0; j < kBurst; ++j) {
+            const int q = tl + j * tpr;
+            if (q - lane < nchunks) quantize(q, v[j], S);
+        }
+    } else {
+        // long inputs: one pass for the maximum, a second one (re-reading the input) for the pieces
+        float m = 0.f, tot = 0.f;
+#pragma unroll 1
+        for (int q = tl; q - lane < nchunks; q += tpr) {
+            u32x4_t ra, rb;
+            float v[8];
+            issue(q, ra, rb);
+            values(q, ra, rb, v, m, tot);
+        }
+        publish(m, tot);
+        lds_barrier();
+        const float S = q8_scale(q8_exponent(smax[b]));
+#pragma unroll 1
+        for (int q = tl; q - lane < nchunks; q += tpr) {
+            u32x4_t ra, rb;
+            float v[8], m2 = 0.f, t2 = 0.f;
+            issue(q, ra, rb);
+            values(q, ra, rb, v, m2, t2);
+            quantize(q, v, S);
+        }
+    }
+}
+
+// acc[p] += (single-bit fp4 operand of class p of this lane's unit) x (fp8 pieces); bp = this lane's first
+// chunk of the item: xq + column * pitch + 8 * (4 ub + (g >> 1)) + (g & 1).  Class values 0.5, 1, 2, 2.
+constexpr int kQ8Accs = 4;
+__device__ __forceinline__ void unit_mfma_q8(const uint4& w, const uint4* bp, float4_t (&acc)[kQ8Accs]) {
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const uint32_t mask = p == 3 ? 0x44444444u : (0x11111111u << p);
+        const int sh = p == 3 ? 1 : 0;
+        v8i_t a = {0, 0, 0, 0, 0, 0, 0, 0};
+        a[0] = (int)((w.x >> sh) & mask);
+        a[1] = (int)((w.y >> sh) & mask);
+        a[2] = (int)((w.z >> sh) & mask);
+        a[3] = (int)((w.w >> sh) & mask);
+        const uint4 b0 = bp[2 * p], b1 = bp[2 * p + 16];
+        const v8i_t b = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+        acc[p] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[p], 4 /* A: fp4 */, 0 /* B: fp8 */, 0, 0, 0, 0);
+    }
+}
+__device__ __forceinline__ float4_t q8_combine(const float4_t (&acc)[kQ8Accs]) {
+    return acc[0] * 2.f + acc[1] + (acc[2] + acc[3]) * 0.5f;   // undo the class values 0.5, 1, 2, 2
+}
+
 }  // namespace nq

@@ -87,10 +87,19 @@ __device__ __forceinline__ void trim_unit(const BitsView& v, uint4& w, int unit)
     }
 }
 
+// Bytes of LDS in front of the staged input: row sums, the input totals, and the per-unit input sums (the fp4 x
+// fp8 path keeps the per-row maxima there instead).
+__host__ __device__ constexpr size_t stream_head_bytes(int batch, int arith) {
+    return arith == 2 ? (size_t)row_block(batch) * batch * sizeof(float) + 128
+                      : (size_t)(row_block(batch) + kXsumStride) * batch * sizeof(float) + 64;
+}
+
 // Items of the MFMA path that each wavefront of a workgroup takes (contiguous runs).
 __host__ __device__ __forceinline__ int mfma_items_per_wave(int nitems, int waves) { return (nitems + waves - 1) / waves; }
 
-template <int DT, int BATCH, bool MFMA, int THREADS, bool SINGLE>
+// ARITH: 0 = matmul-free (dot2 on the VALU), 1 = MFMA with 16-bit operands, 2 = MFMA with one-bit fp4 weights
+// and fp8 pieces of the input (batch <= 4).
+template <int DT, int BATCH, int ARITH, int THREADS, bool SINGLE>
 __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __restrict__ stages, int nstages,
                                                                      int nphases, const int* __restrict__ seg_index,
                                                                      const RunSegment* __restrict__ segs,
@@ -102,11 +111,16 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
     constexpr int kWaves = THREADS / kWave;
     constexpr int kRowBlock = row_block(BATCH);
     extern __shared__ uint4 lds_raw[];
-    constexpr bool kPow2Mfma = MFMA && DT == 0;                 // fp16 MFMA path: single-bit operands, pair-major x
+    constexpr bool MFMA = ARITH != 0;
+    constexpr bool kQ8 = ARITH == 2;
+    constexpr bool kPow2Mfma = ARITH == 1 && DT == 0;           // fp16 MFMA path: single-bit operands, pair-major x
+    constexpr bool kTotals = kPow2Mfma || kQ8;                  // signed sum = (sum of x) - 2 (sum of b x)
+    static_assert(!kQ8 || BATCH * kQ8Pieces <= 16, "pieces of all batch rows must fit the 16 operand columns");
     float* racc = (float*)lds_raw;                              // [kRowBlock][BATCH] row sums
     float* xtot = racc + kRowBlock * BATCH;                     // [16] sum of the staged input per batch row
     float* xsum = xtot + 16;                                    // [BATCH][kXsumStride] per-unit input sums
-    uint4* xs = lds_raw + ((kRowBlock + kXsumStride) * BATCH * sizeof(float) + 64) / sizeof(uint4);
+    uint32_t* smax = (uint32_t*)xsum;                           // kQ8: [16] largest |input| per batch row (bits)
+    uint4* xs = lds_raw + stream_head_bytes(BATCH, ARITH) / sizeof(uint4);
     __shared__ int s_flag;
     const int tid = threadIdx.x;
     const int wg = blockIdx.x;
@@ -149,7 +163,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
             }
             const BitsView bv = bits_view(st);
             const int chunk_units = min(st.units, chunk_cap);
-            const int upad = chunk_units | 1;
+            const int upad = kQ8 ? q8_pitch(q8_units4(chunk_units)) : (chunk_units | 1);
             const bool one_chunk = chunk_units == st.units;
             StageInput sin;
             sin.in = st.in; sin.s_col = st.s_col; sin.K = st.K; sin.in_stride = st.in_stride;
@@ -223,13 +237,15 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                         const int cu_n = min(chunk_units, st.units - c0);
                         if (!(one_chunk && staged)) {
                             if (c0) lds_barrier();
-                            if (kPow2Mfma && c0 == 0) {
-                                // every reader of the previous total has passed a barrier by now
-                                if (tid < 16) xtot[tid] = 0.f;
+                            if (kTotals && (c0 == 0 || kQ8)) {
+                                // every reader of the previous totals has passed a barrier by now
+                                if (tid < 16 && c0 == 0) xtot[tid] = 0.f;
+                                if (kQ8 && tid >= 16 && tid < 32) smax[tid - 16] = 0u;
                                 lds_barrier();
                             }
-                            stage_units<DT, BATCH, kPow2Mfma>(xs, xsum, sin, c0, cu_n, upad, kStreamThreads,
-                                                              kPow2Mfma ? xtot : nullptr);
+                            if constexpr (kQ8) stage_units_q8<DT, BATCH>(xs, smax, xtot, sin, c0, cu_n, upad, kStreamThreads);
+                            else stage_units<DT, BATCH, kPow2Mfma>(xs, xsum, sin, c0, cu_n, upad, kStreamThreads,
+                                                                   kPow2Mfma ? xtot : nullptr);
                             staged = true;
                         }
                         lds_barrier();                           // xs / xsum / zeroed racc visible
@@ -244,7 +260,13 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                             const int nitems = ((nr + 15) >> 4) * ngroups;
                             const int per = mfma_items_per_wave(nitems, kWaves);
                             const int it_begin = wave * per, it_end = min(it_begin + per, nitems);
-                            constexpr int kAccs = kPow2Mfma ? kPow2Classes : kMfmaAccs;
+                            constexpr int kAccs = kQ8 ? kQ8Accs : kPow2Mfma ? kPow2Classes : kMfmaAccs;
+                            // kQ8: operand column of this lane (batch row, piece), its first chunk, and the factor
+                            // that takes its accumulator back to the unscaled signed sum
+                            const int qcol = min(r16, BATCH * kQ8Pieces - 1);
+                            const uint4* qbase = xs + (size_t)qcol * upad + 8 * (g >> 1) + (g & 1);
+                            float qfac = 0.f;
+                            if constexpr (kQ8) qfac = q8_unscale_neg2(q8_exponent(smax[qcol / kQ8Pieces]));
                             // (row group, unit group) of the current and of the next item, advanced without divisions
                             int rg = 16 * (it_begin / ngroups), ub = it_begin % ngroups;
                             int rg_n = rg, ub_n = ub + 1;
@@ -266,7 +288,8 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                                     const uint4 wpre = load_unit(bv, min(rb + rg_n + r16, st.rows - 1), c0 + un,
                                                                  it + 1 < it_end && un < cu_n);
                                     trim_unit(bv, w, c0 + u);
-                                    if constexpr (kPow2Mfma) unit_mfma_pow2<BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
+                                    if constexpr (kQ8) unit_mfma_q8(w, qbase + 32 * ub, acc);     // w = 0 beyond cu_n, padding staged as 0
+                                    else if constexpr (kPow2Mfma) unit_mfma_pow2<BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
                                     else unit_mfma<DT, BATCH>(w, xs, upad, u, u < cu_n, acc);
                                     w = wpre;
                                     rg = rg_n; ub = ub_n;
@@ -274,9 +297,18 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                                 }
                                 // sum[v] = partial sum of row rg_run + 4*g + v for batch row r16
                                 float4_t sum;
-                                if constexpr (kPow2Mfma) sum = pow2_combine(acc) * -2.f;   // + sum of x at the end
+                                if constexpr (kQ8) sum = q8_combine(acc) * qfac;           // + sum of x at the end
+                                else if constexpr (kPow2Mfma) sum = pow2_combine(acc) * -2.f;
                                 else sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
-                                if (r16 < BATCH) {
+                                if constexpr (kQ8) {
+                                    // the pieces of a batch row are neighbouring columns: their sum lands in one address
+                                    if (r16 < BATCH * kQ8Pieces) {
+#pragma unroll
+                                        for (int v = 0; v < 4; ++v)
+                                            if (rg_run + 4 * g + v < nr)
+                                                atomicAdd(&racc[(rg_run + 4 * g + v) * BATCH + r16 / kQ8Pieces], sum[v]);
+                                    }
+                                } else if (r16 < BATCH) {
 #pragma unroll
                                     for (int v = 0; v < 4; ++v)
                                         if (rg_run + 4 * g + v < nr) atomicAdd(&racc[(rg_run + 4 * g + v) * BATCH + r16], sum[v]);
@@ -356,7 +388,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                     for (int i = tid; i < nr * BATCH; i += kStreamThreads) {
                         const int row = rb + i / BATCH, b = i % BATCH;
                         float v = racc[i];
-                        if constexpr (kPow2Mfma) v += xtot[b];
+                        if constexpr (kTotals) v += xtot[b];
                         if (st.s_row) v *= E::to_float(st.s_row[row]);
                         const size_t o = (size_t)b * st.out_stride + row;
                         if (st.addend) {
@@ -407,8 +439,17 @@ size_t stream_counter_bytes(int nstages) {
 }
 
 // ---- host side --------------------------------------------------------------------------------
-static void stream_lds_plan(int batch, int max_units, int* chunk_cap_out, size_t* lds_out) {
-    const int racc_bytes = (row_block(batch) + kXsumStride) * batch * (int)sizeof(float) + 64;
+static void stream_lds_plan(int batch, int arith, int max_units, int* chunk_cap_out, size_t* lds_out) {
+    const int racc_bytes = (int)stream_head_bytes(batch, arith);
+    if (arith == 2) {
+        // kQ8Pieces bytes per column and batch row, staged in whole groups of four units
+        int chunk_cap = (kStreamLdsMax - racc_bytes - batch * kQ8Pieces * (int)sizeof(uint4)) / (batch * kQ8Pieces * 128);
+        chunk_cap &= ~3;
+        const int chunk_units = max_units < chunk_cap ? max_units : chunk_cap;
+        *chunk_cap_out = chunk_cap;
+        *lds_out = (size_t)racc_bytes + (size_t)q8_chunks(batch, q8_units4(chunk_units)) * sizeof(uint4);
+        return;
+    }
     int chunk_cap = (kStreamLdsMax - racc_bytes - batch * (int)sizeof(uint4)) / (batch * 16 * (int)sizeof(uint4));
     chunk_cap = (chunk_cap - 1) & ~1;
     if (chunk_cap > kXsumStride - 2) chunk_cap = kXsumStride - 2;
@@ -426,19 +467,19 @@ static void stream_lds_plan(int batch, int max_units, int* chunk_cap_out, size_t
 // traffic per row: decisive for the MFMA path (batch 16: 211 -> 80 us per layer going from 256 to 1024
 // lanes).  The matmul-free batch-1 kernel prefers four independent 256-lane workgroups per CU, which overlap
 // each other's staging and arithmetic (32.7 vs 35.0 us with one 1024-lane workgroup).
-#ifndef NQ_STREAM_MFMA
-#define NQ_STREAM_MFMA(DT, BATCH) ((BATCH) >= 2 || (DT) == 0)
+#ifndef NQ_STREAM_ARITH
+#define NQ_STREAM_ARITH(DT, BATCH) ((BATCH) <= 4 ? 2 : 1)
 #endif
 #ifndef NQ_STREAM_THREADS
-#define NQ_STREAM_THREADS(DT, BATCH) ((BATCH) >= 2 ? 1024 : (DT) == 0 ? 512 : 256)
+#define NQ_STREAM_THREADS(DT, BATCH) ((BATCH) >= 2 ? 1024 : 512)
 #endif
 
 template <int DT, int BATCH>
 struct StreamKernel {
-    static constexpr bool kMfma = NQ_STREAM_MFMA(DT, BATCH);
+    static constexpr int kArith = NQ_STREAM_ARITH(DT, BATCH);
     static constexpr int kThreads = NQ_STREAM_THREADS(DT, BATCH);
-    static constexpr auto fn = gemv_stream_kernel<DT, BATCH, kMfma, kThreads, false>;
-    static constexpr auto fn_single = gemv_stream_kernel<DT, BATCH, kMfma, kThreads, true>;
+    static constexpr auto fn = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false>;
+    static constexpr auto fn_single = gemv_stream_kernel<DT, BATCH, kArith, kThreads, true>;
 };
 
 template <int DT, int BATCH>
@@ -457,7 +498,7 @@ template <int DT, int BATCH>
 static int capacity_of(int max_units) {
     int chunk_cap;
     size_t lds;
-    stream_lds_plan(BATCH, max_units, &chunk_cap, &lds);
+    stream_lds_plan(BATCH, StreamKernel<DT, BATCH>::kArith, max_units, &chunk_cap, &lds);
     if (prepare_kernel<DT, BATCH>(lds) != hipSuccess) return 0;
     int per_cu = 0, dev = 0, cus = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)StreamKernel<DT, BATCH>::fn, StreamKernel<DT, BATCH>::kThreads,
@@ -474,7 +515,7 @@ static hipError_t launch_stream(const RunStage* stages, int nstages, int nphases
                                 int max_units, hipStream_t stream) {
     int chunk_cap;
     size_t lds;
-    stream_lds_plan(BATCH, max_units, &chunk_cap, &lds);
+    stream_lds_plan(BATCH, StreamKernel<DT, BATCH>::kArith, max_units, &chunk_cap, &lds);
     hipError_t e = prepare_kernel<DT, BATCH>(lds);
     if (e != hipSuccess) return e;
 #ifdef NQ_TRACE
@@ -512,7 +553,7 @@ static hipError_t launch_single(const RunStage& st, hipStream_t stream) {
     using SK = StreamKernel<DT, BATCH>;
     int chunk_cap;
     size_t lds;
-    stream_lds_plan(BATCH, st.units, &chunk_cap, &lds);
+    stream_lds_plan(BATCH, SK::kArith, st.units, &chunk_cap, &lds);
     static bool attr_done = false;
     if (lds > 64 * 1024 && !attr_done) {
         hipError_t e = hipFuncSetAttribute((const void*)SK::fn_single, hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);

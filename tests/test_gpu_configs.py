@@ -108,11 +108,12 @@ def test_cfg4_llama3_70b_shapes_in_one_run_list(dev, batch):
         for (rows, ref, xt, ops_dev), y in zip(cases, ys):
             err = np.abs(y.float().cpu().numpy()[:, rows] - ref).max() / np.abs(ref).max()
             assert err < 1e-3, err
-    # full-size property: every row agrees with the per-linear entry point (different summation tree)
+    # full-size property: every row agrees with the per-linear entry point (other arithmetic: 16-bit staging of x
+    # and h there, fp8 pieces here; each is within 1e-3 of the exact result, both errors add up here)
     for (rows, ref, xt, ops_dev), y in zip(cases, ys):
         y_op = torch.ops.binary_kernels.nanoquant_dyn_forward(xt, *ops_dev, 128, 128, 2, 2, 1, 1, 8, 8)
         torch.cuda.synchronize()
-        assert torch.allclose(y.float(), y_op.float(), rtol=2e-3, atol=2e-4 * float(np.abs(ref).max()))
+        assert torch.allclose(y.float(), y_op.float(), rtol=2e-3, atol=1e-3 * float(np.abs(ref).max()))
 
 
 def test_cfg1_full_size_linearity_in_output_scale(dev):

@@ -43,9 +43,9 @@ def test_independent_linears(dev, batch, interleave):
             assert err < (TIGHT if r >= 256 else 1e-2), (rep, m, n, r, err)
 
 
-def test_matches_per_linear_entry_point_bitwise(dev):
-    # same arithmetic per 16-byte unit, different summation tree across units: agreement to fp32
-    # rounding of the row sums, i.e. far below one fp16 ulp of the output for almost all elements
+def test_matches_per_linear_entry_point(dev):
+    # different arithmetic (the run list stages fp8 pieces of the input, the per-linear kernel 16-bit values)
+    # and different summation trees: agreement far below one fp16 ulp of the output for most elements
     m, n, r, batch = 1024, 4096, 512, 2
     npt, ops = _term(dev, m, n, r, seed=7)
     x = torch.from_numpy(oracle.synth_x(batch, n, 7)).to(dev)
@@ -54,8 +54,7 @@ def test_matches_per_linear_entry_point_bitwise(dev):
     y_rl = rl.run()[0].float()
     y_op = torch.ops.binary_kernels.nanoquant_dyn_forward(x, *ops, 128, 128, 2, 2, 1, 1, 8, 8).float()
     torch.cuda.synchronize()
-    assert torch.allclose(y_rl, y_op, rtol=2e-3, atol=0)
-    assert (y_rl == y_op).float().mean() > 0.9
+    assert torch.allclose(y_rl, y_op, rtol=2e-3, atol=2e-4 * float(y_op.abs().max()))
 
 
 def test_chained_linears_depend_on_each_other(dev):
@@ -143,7 +142,10 @@ def test_graph_replay_of_a_run_list(dev):
         torch.cuda.synchronize()
         assert rl.status() == 0
         for y, e in zip(rl.outputs, eager):
-            assert torch.equal(y, e), rep
+            # row sums are finished with LDS float atomics whose order varies from run to run: equal up to an
+            # fp32 rounding of the sum, i.e. at most one fp16 ulp of the output here and there
+            assert torch.allclose(y.float(), e.float(), rtol=2e-3, atol=1e-4 * float(e.float().abs().max())), rep
+            assert (y == e).float().mean() > 0.9, rep
 
 
 @pytest.mark.parametrize("batch", [2, 16])
