@@ -511,17 +511,21 @@ __device__ __forceinline__ uint32_t quad_transpose_rev(uint32_t m, bool odd, boo
 __device__ __forceinline__ uint32_t q8_exponent(uint32_t max_bits) { return max(max_bits >> 23, 32u); }
 __device__ __forceinline__ float q8_scale(uint32_t eb) { return as_float((261u - eb) << 23); }
 __device__ __forceinline__ float q8_unscale_neg2(uint32_t eb) { return as_float(0x80000000u | ((eb - 6u) << 23)); }
+// the same for accumulators that hold 0.5 * sum b * u
+__device__ __forceinline__ float q8_unscale_neg4(uint32_t eb) { return as_float(0x80000000u | ((eb - 5u) << 23)); }
 
 // Stage units [c0, c0 + cu_n) (plus zero padding up to q8_units4(cu_n)) of BATCH rows.  smax[b] (uint32,
 // zeroed by the caller, barrier before) receives the bit pattern of max |u| per batch row, xtot[b] the sum of
 // the staged values.  The wavefronts of the workgroup are divided among the batch rows (nthreads / 64 must be a
 // multiple of BATCH), so a lane reduces maximum and sum over all its chunks before anything crosses lanes.
 // Contains one workgroup barrier; a barrier must follow before the staged data is read.
-template <int DT, int BATCH>
+template <int DT, int BATCH, int THREADS>
 __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* smax, float* xtot, const StageInput& st, int c0,
-                                               int cu_n, int pitch, int nthreads) {
+                                               int cu_n, int pitch) {
     using E = Elem<DT>;
-    constexpr int kBurst = BATCH >= 4 ? 6 : 3;
+    constexpr int nthreads = THREADS;
+    // chunks per lane that stay in registers across the barrier: enough for 11264 columns (88 units) per batch row
+    constexpr int kBurst = (88 * 16 * BATCH + THREADS - 1) / THREADS;
     const int nchunks = q8_units4(cu_n) * 16;            // 8-column chunks per batch row, a multiple of 64
     const int tpr = nthreads / BATCH;                    // lanes per batch row
     const int b = threadIdx.x / tpr, tl = threadIdx.x - b * tpr;
@@ -672,26 +676,51 @@ __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* smax, float*
     }
 }
 
-// acc[p] += (single-bit fp4 operand of class p of this lane's unit) x (fp8 pieces); bp = this lane's first
-// chunk of the item: xq + column * pitch + 8 * (4 ub + (g >> 1)) + (g & 1).  Class values 0.5, 1, 2, 2.
-constexpr int kQ8Accs = 4;
-__device__ __forceinline__ void unit_mfma_q8(const uint4& w, const uint4* bp, float4_t (&acc)[kQ8Accs]) {
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const uint32_t mask = p == 3 ? 0x44444444u : (0x11111111u << p);
-        const int sh = p == 3 ? 1 : 0;
-        v8i_t a = {0, 0, 0, 0, 0, 0, 0, 0};
-        a[0] = (int)((w.x >> sh) & mask);
-        a[1] = (int)((w.y >> sh) & mask);
-        a[2] = (int)((w.z >> sh) & mask);
-        a[3] = (int)((w.w >> sh) & mask);
-        const uint4 b0 = bp[2 * p], b1 = bp[2 * p + 16];
-        const v8i_t b = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
-        acc[p] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[p], 4 /* A: fp4 */, 0 /* B: fp8 */, 0, 0, 0, 0);
-    }
+// The B operand of one unit group held in registers: per class p the two 16-byte halves read from
+// xq + column * pitch + 8 * (4 ub + (g >> 1)) + (g & 1) + 2 p (lo) and 16 chunks further (hi).  Named native
+// vectors on purpose: arrays of uint4 captured by a lambda end up in scratch memory.
+struct Q8Operand {
+    u32x4_t lo0, lo1, lo2, lo3, hi0, hi1, hi2, hi3;
+};
+
+__device__ __forceinline__ void q8_read_operand(Q8Operand& o, const uint4* bp) {
+    const u32x4_t* p = (const u32x4_t*)bp;
+    o.lo0 = p[0]; o.hi0 = p[16];
+    o.lo1 = p[2]; o.hi1 = p[18];
+    o.lo2 = p[4]; o.hi2 = p[20];
+    o.lo3 = p[6]; o.hi3 = p[22];
 }
-__device__ __forceinline__ float4_t q8_combine(const float4_t (&acc)[kQ8Accs]) {
-    return acc[0] * 2.f + acc[1] + (acc[2] + acc[3]) * 0.5f;   // undo the class values 0.5, 1, 2, 2
+
+// One class of two row groups that share the input operand: (w >> P) & 0x11111111 is the fp4 operand of
+// value 0.5 per set bit whatever the class, so all four classes add into ONE accumulator per row group; the two
+// row groups alternate, which keeps dependent MFMAs two issues apart.
+template <int P>
+__device__ __forceinline__ void q8_class_pair(const uint4& wa, const uint4& wb, const u32x4_t& lo, const u32x4_t& hi,
+                                              float4_t& acc_a, float4_t& acc_b) {
+    constexpr uint32_t M = 0x11111111u;
+    const v8i_t b = {(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+    const v8i_t aa = {(int)((wa.x >> P) & M), (int)((wa.y >> P) & M), (int)((wa.z >> P) & M), (int)((wa.w >> P) & M), 0, 0, 0, 0};
+    const v8i_t ab = {(int)((wb.x >> P) & M), (int)((wb.y >> P) & M), (int)((wb.z >> P) & M), (int)((wb.w >> P) & M), 0, 0, 0, 0};
+    acc_a = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aa, b, acc_a, 4 /* A: fp4 */, 0 /* B: fp8 */, 0, 0, 0, 0);
+    acc_b = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ab, b, acc_b, 4, 0, 0, 0, 0, 0);
+}
+
+// acc += 0.5 * sum b * u per (row, column) of the lane, for the units wa / wb of two row groups 16 rows apart
+__device__ __forceinline__ void unit_mfma_q8_pair(const uint4& wa, const uint4& wb, const Q8Operand& o, float4_t& acc_a,
+                                                  float4_t& acc_b) {
+    q8_class_pair<0>(wa, wb, o.lo0, o.hi0, acc_a, acc_b);
+    q8_class_pair<1>(wa, wb, o.lo1, o.hi1, acc_a, acc_b);
+    q8_class_pair<2>(wa, wb, o.lo2, o.hi2, acc_a, acc_b);
+    q8_class_pair<3>(wa, wb, o.lo3, o.hi3, acc_a, acc_b);
+}
+
+// Sum over the kQ8Pieces neighbouring columns of a batch row; valid in the lane of the last piece.
+__device__ __forceinline__ float q8_piece_sum(float v) {
+    static_assert(kQ8Pieces == 3, "two shifted adds");
+    const int i = __builtin_bit_cast(int, v);
+    const float s1 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, i, 0x111 /* row_shr:1 */, 0xF, 0xF, true));
+    const float s2 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, i, 0x112 /* row_shr:2 */, 0xF, 0xF, true));
+    return v + s1 + s2;
 }
 
 }  // namespace nq

@@ -50,12 +50,18 @@ constexpr int kCounterStride = 8;              // 64-bit words between sub-count
 // in [g*members_k, (g+1)*members_k) for as long as the reading workgroup itself has not left, so
 // g = value / members_k needs no reset between launches and no atomic that returns a value; stage s
 // is complete in launch g when its sub-counters add up to (g+1) * seg_count(s).
+constexpr int kQ8Depth = 3;                    // items (2 KB of packed words each) in flight per wavefront, fp4 x fp8 path
 constexpr int kStreamLdsMax = 144 * 1024;      // staged activations + row accumulators, upper bound
 
 // The packed words of one stage as a raw buffer: one 16-byte load per unit whatever the row alignment
 // (buffer loads need dword alignment only), zeros past the end of the matrix, and "no load" expressed
 // as an offset past the end instead of a branch -- with exactly one load instruction per loop trip the
 // compiler can leave younger fetches in flight (vmcnt counting) instead of waiting for all of them.
+// Cache policy of the packed-word fetches: default.  The non-temporal hint costs a fifth of the read bandwidth here
+// (a wave-load is 16 rows x 64 bytes, so every 128-byte line is asked for twice, and the hint drops it in between).
+#ifndef NQ_BITS_AUX
+#define NQ_BITS_AUX 0
+#endif
 struct BitsView {
     __amdgpu_buffer_rsrc_t rsrc;
     int words;      // 32-bit words per row
@@ -72,7 +78,7 @@ __device__ __forceinline__ BitsView bits_view(const RunStage& st) {
 
 __device__ __forceinline__ uint4 load_unit(const BitsView& v, int row, int unit, bool live) {
     const uint32_t off = live ? ((uint32_t)row * (uint32_t)v.words + 4u * (uint32_t)unit) * 4u : kPastEnd;
-    const u32x4_t w = __builtin_amdgcn_raw_buffer_load_b128(v.rsrc, off, 0, 2 /* nt: streamed once */);
+    const u32x4_t w = __builtin_amdgcn_raw_buffer_load_b128(v.rsrc, off, 0, NQ_BITS_AUX);
     return make_uint4(w.x, w.y, w.z, w.w);
 }
 
@@ -169,9 +175,30 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
             sin.in = st.in; sin.s_col = st.s_col; sin.K = st.K; sin.in_stride = st.in_stride;
             sin.in_f32 = st.in_f32; sin.in_coherent = st.in_coherent; sin.vec_in = st.vec_in;
 
-            // First fetch of the slice, issued before any wait: the weights are always ready.
+            // First fetches of the slice, issued before any wait: the weights are always ready.  The fp4 x fp8 path
+            // keeps kQ8Depth fetches per wavefront in flight (a slice of one decoder layer is about three items per
+            // wavefront, so its weights stream in while the input is still being waited for and staged).
             uint4 wnext = make_uint4(0, 0, 0, 0);
-            if constexpr (MFMA) {
+            uint4 wqa0 = wnext, wqb0 = wnext, wqa1 = wnext, wqb1 = wnext, wqa2 = wnext, wqb2 = wnext;
+            if constexpr (kQ8) {
+                // items of the first row block: (pair of 16-row groups, 4-unit group), unit group fastest; wavefront
+                // w starts with item w * per; lane (row l & 15 of both groups, unit l >> 4)
+                const int ng0 = (chunk_units + 3) >> 2;
+                const int nrp0 = (min(seg.row_end - seg.row_begin, kRowBlock) + 31) >> 5;
+                const int per0 = mfma_items_per_wave(ng0 * nrp0, kWaves);
+                const int item0 = __builtin_amdgcn_readfirstlane(tid >> 6) * per0;
+                const int end0 = min(item0 + per0, ng0 * nrp0);
+                auto first = [&](int it, uint4& wa, uint4& wb) {
+                    const int u = 4 * (it % ng0) + ((tid & 63) >> 4);
+                    const int row = seg.row_begin + 32 * (it / ng0) + (tid & 15);
+                    const bool live = it < end0 && u < chunk_units;
+                    wa = load_unit(bv, min(row, st.rows - 1), u, live);
+                    wb = load_unit(bv, min(row + 16, st.rows - 1), u, live);
+                };
+                first(item0, wqa0, wqb0);
+                first(item0 + 1, wqa1, wqb1);
+                first(item0 + 2, wqa2, wqb2);
+            } else if constexpr (MFMA) {
                 // wavefront w starts with item w of the first row block: 16 rows x 4 units, lane (row l & 15,
                 // unit l >> 4)
                 const int ng0 = (chunk_units + 3) >> 2;
@@ -243,14 +270,95 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                                 if (kQ8 && tid >= 16 && tid < 32) smax[tid - 16] = 0u;
                                 lds_barrier();
                             }
-                            if constexpr (kQ8) stage_units_q8<DT, BATCH>(xs, smax, xtot, sin, c0, cu_n, upad, kStreamThreads);
+                            if constexpr (kQ8) stage_units_q8<DT, BATCH, THREADS>(xs, smax, xtot, sin, c0, cu_n, upad);
                             else stage_units<DT, BATCH, kPow2Mfma>(xs, xsum, sin, c0, cu_n, upad, kStreamThreads,
                                                                    kPow2Mfma ? xtot : nullptr);
                             staged = true;
                         }
                         lds_barrier();                           // xs / xsum / zeroed racc visible
                         if (sg == seg_begin && ph < 3 && rb == seg.row_begin && c0 == 0) NQ_MARK(2 + 4 * ph);
-                        if constexpr (MFMA) {
+                        if constexpr (kQ8) {
+                            // Items = (pair of 16-row groups, 4-unit group), unit group fastest: one read of the input
+                            // operand (eight 16-byte LDS reads per lane) serves two row groups, and a wavefront takes a
+                            // contiguous run of items, so it adds its two accumulators to the row sums only when the
+                            // pair changes (LDS float atomics cost about 2.5 cycles per lane).
+                            const int lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+                            const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar item arithmetic
+                            const int ngroups = (cu_n + 3) >> 2, nrp = (nr + 31) >> 5;
+                            const int nitems = ngroups * nrp;
+                            const int per = mfma_items_per_wave(nitems, kWaves);
+                            const int it_begin = wave * per, it_end = min(it_begin + per, nitems);
+                            // operand column of this lane (batch row, piece), its first chunk, and the factor that takes
+                            // an accumulator back to the unscaled signed sum; columns beyond the last piece are never
+                            // read back, so their lanes skip the LDS reads (40 % less LDS time per read)
+                            const bool qlive = r16 < BATCH * kQ8Pieces;
+                            const int qcol = min(r16, BATCH * kQ8Pieces - 1);
+                            const uint4* qbase = xs + (size_t)qcol * upad + 8 * (g >> 1) + (g & 1);
+                            const float qfac = q8_unscale_neg4(q8_exponent(smax[qcol / kQ8Pieces]));
+                            const bool qlast = qlive && r16 % kQ8Pieces == kQ8Pieces - 1;   // holds the sum over the pieces
+                            float* rdst = racc + (4 * g) * BATCH + qcol / kQ8Pieces;
+                            // fetch cursor (kQ8Depth items ahead) and compute cursor, advanced without divisions
+                            int it_f = it_begin, rp_f = it_begin / ngroups, ub_f = it_begin - rp_f * ngroups;
+                            int rp = rp_f, ub = ub_f;
+                            auto fetch = [&](uint4& wa, uint4& wb) {
+                                const int u = 4 * ub_f + g;
+                                const int row = rb + 32 * rp_f + r16;
+                                const bool live = it_f < it_end && u < cu_n;
+                                wa = load_unit(bv, min(row, st.rows - 1), c0 + u, live);
+                                wb = load_unit(bv, min(row + 16, st.rows - 1), c0 + u, live);
+                                ++it_f;
+                                if (++ub_f == ngroups) { ub_f = 0; ++rp_f; }
+                            };
+                            // kQ8Depth register pairs in rotation, each refilled right after its use: nothing in flight
+                            // is ever copied, and the main loop has no early exit.
+                            static_assert(kQ8Depth == 3, "the rotation below is written out for three register pairs");
+                            uint4 wa0, wb0, wa1, wb1, wa2, wb2;
+                            if (rb == seg.row_begin && c0 == 0) {            // fetched before the wait
+                                wa0 = wqa0; wb0 = wqb0; wa1 = wqa1; wb1 = wqb1; wa2 = wqa2; wb2 = wqb2;
+#pragma unroll
+                                for (int k = 0; k < kQ8Depth; ++k) {
+                                    ++it_f;
+                                    if (++ub_f == ngroups) { ub_f = 0; ++rp_f; }
+                                }
+                            } else {
+                                fetch(wa0, wb0); fetch(wa1, wb1); fetch(wa2, wb2);
+                            }
+                            Q8Operand opnd = {};
+                            float4_t acc_a = {0.f, 0.f, 0.f, 0.f}, acc_b = {0.f, 0.f, 0.f, 0.f};
+                            int rp_run = rp;
+                            auto flush = [&]() {
+                                // acc[v] = partial sum of row 32 rp_run + 4 g + v (acc_b: 16 rows further) for column r16
+#pragma unroll
+                                for (int v = 0; v < 4; ++v) {
+                                    const float sa = q8_piece_sum(acc_a[v] * qfac), sb = q8_piece_sum(acc_b[v] * qfac);
+                                    const int row = 32 * rp_run + 4 * g + v;
+                                    if (qlast && row < nr) atomicAdd(&rdst[(32 * rp_run + v) * BATCH], sa);
+                                    if (qlast && row + 16 < nr) atomicAdd(&rdst[(32 * rp_run + 16 + v) * BATCH], sb);
+                                }
+                            };
+                            auto step = [&](uint4& wa, uint4& wb) {
+                                if (rp != rp_run) {
+                                    flush();
+                                    acc_a = acc_b = (float4_t){0.f, 0.f, 0.f, 0.f};
+                                    rp_run = rp;
+                                }
+                                if (qlive) q8_read_operand(opnd, qbase + 32 * ub);
+                                trim_unit(bv, wa, c0 + 4 * ub + g);       // w = 0 beyond cu_n, padding staged as 0
+                                trim_unit(bv, wb, c0 + 4 * ub + g);
+                                unit_mfma_q8_pair(wa, wb, opnd, acc_a, acc_b);
+                                if (++ub == ngroups) { ub = 0; ++rp; }
+                                fetch(wa, wb);
+                            };
+                            int it = it_begin;
+#pragma unroll 1
+                            for (; it + kQ8Depth <= it_end; it += kQ8Depth) {
+                                step(wa0, wb0); step(wa1, wb1); step(wa2, wb2);
+                            }
+                            if (it < it_end) step(wa0, wb0);
+                            if (it + 1 < it_end) step(wa1, wb1);
+                            if (it_begin < it_end) flush();              // + sum of x at the end
+                            if (ph == 0 && sg == seg_begin) NQ_MARK(14);
+                        } else if constexpr (MFMA) {
                             // Items = (16-row group, 4-unit group), unit group fastest; every wavefront takes a
                             // contiguous run of items, so it mostly stays on one row group and adds its
                             // accumulator to the row sums only when the row group changes.
@@ -260,13 +368,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                             const int nitems = ((nr + 15) >> 4) * ngroups;
                             const int per = mfma_items_per_wave(nitems, kWaves);
                             const int it_begin = wave * per, it_end = min(it_begin + per, nitems);
-                            constexpr int kAccs = kQ8 ? kQ8Accs : kPow2Mfma ? kPow2Classes : kMfmaAccs;
-                            // kQ8: operand column of this lane (batch row, piece), its first chunk, and the factor
-                            // that takes its accumulator back to the unscaled signed sum
-                            const int qcol = min(r16, BATCH * kQ8Pieces - 1);
-                            const uint4* qbase = xs + (size_t)qcol * upad + 8 * (g >> 1) + (g & 1);
-                            float qfac = 0.f;
-                            if constexpr (kQ8) qfac = q8_unscale_neg2(q8_exponent(smax[qcol / kQ8Pieces]));
+                            constexpr int kAccs = kPow2Mfma ? kPow2Classes : kMfmaAccs;
                             // (row group, unit group) of the current and of the next item, advanced without divisions
                             int rg = 16 * (it_begin / ngroups), ub = it_begin % ngroups;
                             int rg_n = rg, ub_n = ub + 1;
@@ -288,8 +390,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                                     const uint4 wpre = load_unit(bv, min(rb + rg_n + r16, st.rows - 1), c0 + un,
                                                                  it + 1 < it_end && un < cu_n);
                                     trim_unit(bv, w, c0 + u);
-                                    if constexpr (kQ8) unit_mfma_q8(w, qbase + 32 * ub, acc);     // w = 0 beyond cu_n, padding staged as 0
-                                    else if constexpr (kPow2Mfma) unit_mfma_pow2<BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
+                                    if constexpr (kPow2Mfma) unit_mfma_pow2<BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
                                     else unit_mfma<DT, BATCH>(w, xs, upad, u, u < cu_n, acc);
                                     w = wpre;
                                     rg = rg_n; ub = ub_n;
@@ -297,18 +398,9 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                                 }
                                 // sum[v] = partial sum of row rg_run + 4*g + v for batch row r16
                                 float4_t sum;
-                                if constexpr (kQ8) sum = q8_combine(acc) * qfac;           // + sum of x at the end
-                                else if constexpr (kPow2Mfma) sum = pow2_combine(acc) * -2.f;
+                                if constexpr (kPow2Mfma) sum = pow2_combine(acc) * -2.f;   // + sum of x at the end
                                 else sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
-                                if constexpr (kQ8) {
-                                    // the pieces of a batch row are neighbouring columns: their sum lands in one address
-                                    if (r16 < BATCH * kQ8Pieces) {
-#pragma unroll
-                                        for (int v = 0; v < 4; ++v)
-                                            if (rg_run + 4 * g + v < nr)
-                                                atomicAdd(&racc[(rg_run + 4 * g + v) * BATCH + r16 / kQ8Pieces], sum[v]);
-                                    }
-                                } else if (r16 < BATCH) {
+                                if (r16 < BATCH) {
 #pragma unroll
                                     for (int v = 0; v < 4; ++v)
                                         if (rg_run + 4 * g + v < nr) atomicAdd(&racc[(rg_run + 4 * g + v) * BATCH + r16], sum[v]);
@@ -471,7 +563,7 @@ static void stream_lds_plan(int batch, int arith, int max_units, int* chunk_cap_
 #define NQ_STREAM_ARITH(DT, BATCH) ((BATCH) <= 4 ? 2 : 1)
 #endif
 #ifndef NQ_STREAM_THREADS
-#define NQ_STREAM_THREADS(DT, BATCH) ((BATCH) >= 2 ? 1024 : 512)
+#define NQ_STREAM_THREADS(DT, BATCH) 1024
 #endif
 
 template <int DT, int BATCH>
