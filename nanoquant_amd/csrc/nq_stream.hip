@@ -180,7 +180,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
             // decoder layer is two or three items per wavefront, so its weights stream in while the input is still
             // being waited for and staged.  (A third item here would push the kernel over its 128 registers.)
             uint4 wnext = make_uint4(0, 0, 0, 0);
-            uint4 wqa0 = wnext, wqb0 = wnext, wqa1 = wnext, wqb1 = wnext;
+            uint4 wqa0 = wnext, wqb0 = wnext;
             if constexpr (kQ8) {
                 // items of the first row block: (pair of 16-row groups, 4-unit group), unit group fastest; wavefront
                 // w starts with item w * per; lane (row l & 15 of both groups, unit l >> 4)
@@ -197,7 +197,6 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                     wb = load_unit(bv, min(row + 16, st.rows - 1), u, live);
                 };
                 first(item0, wqa0, wqb0);
-                first(item0 + 1, wqa1, wqb1);
             } else if constexpr (MFMA) {
                 // wavefront w starts with item w of the first row block: 16 rows x 4 units, lane (row l & 15,
                 // unit l >> 4)
@@ -314,12 +313,10 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                             static_assert(kQ8Depth == 3, "the rotation below is written out for three register pairs");
                             uint4 wa0, wb0, wa1, wb1, wa2, wb2;
                             if (rb == seg.row_begin && c0 == 0) {            // fetched before the wait
-                                wa0 = wqa0; wb0 = wqb0; wa1 = wqa1; wb1 = wqb1;
-#pragma unroll
-                                for (int k = 0; k < kQ8Depth - 1; ++k) {
-                                    ++it_f;
-                                    if (++ub_f == ngroups) { ub_f = 0; ++rp_f; }
-                                }
+                                wa0 = wqa0; wb0 = wqb0;
+                                ++it_f;
+                                if (++ub_f == ngroups) { ub_f = 0; ++rp_f; }
+                                fetch(wa1, wb1);
                                 fetch(wa2, wb2);
                             } else {
                                 fetch(wa0, wb0); fetch(wa1, wb1); fetch(wa2, wb2);
