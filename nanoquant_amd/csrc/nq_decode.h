@@ -524,8 +524,9 @@ __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* smax, float*
                                                int cu_n, int pitch) {
     using E = Elem<DT>;
     constexpr int nthreads = THREADS;
-    // chunks per lane that stay in registers across the barrier: enough for 11264 columns (88 units) per batch row
-    constexpr int kBurst = (88 * 16 * BATCH + THREADS - 1) / THREADS;
+    // chunks per lane and round trip.  When a batch row fits into one round trip (16384 columns at batch 1 and 1024
+    // lanes, 8192 at batch 2) the values stay in registers across the barrier; longer inputs are read twice.
+    constexpr int kBurst = 2;
     const int nchunks = q8_units4(cu_n) * 16;            // 8-column chunks per batch row, a multiple of 64
     const int tpr = nthreads / BATCH;                    // lanes per batch row
     const int b = threadIdx.x / tpr, tl = threadIdx.x - b * tpr;
@@ -653,25 +654,33 @@ __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* smax, float*
             if (q - lane < nchunks) quantize(q, v[j], S);
         }
     } else {
-        // long inputs: one pass for the maximum, a second one (re-reading the input) for the pieces
+        // long inputs: one pass for the maximum, a second one (re-reading the input) for the pieces, kBurst chunks
+        // per lane and round trip
         float m = 0.f, tot = 0.f;
 #pragma unroll 1
-        for (int q = tl; q - lane < nchunks; q += tpr) {
-            u32x4_t ra, rb;
+        for (int q0 = tl; q0 - lane < nchunks; q0 += kBurst * tpr) {
+            u32x4_t ra[kBurst], rb[kBurst];
             float v[8];
-            issue(q, ra, rb);
-            values(q, ra, rb, v, m, tot);
+#pragma unroll
+            for (int j = 0; j < kBurst; ++j) issue(q0 + j * tpr, ra[j], rb[j]);
+#pragma unroll
+            for (int j = 0; j < kBurst; ++j) values(q0 + j * tpr, ra[j], rb[j], v, m, tot);
         }
         publish(m, tot);
         lds_barrier();
         const float S = q8_scale(q8_exponent(smax[b]));
 #pragma unroll 1
-        for (int q = tl; q - lane < nchunks; q += tpr) {
-            u32x4_t ra, rb;
-            float v[8], m2 = 0.f, t2 = 0.f;
-            issue(q, ra, rb);
-            values(q, ra, rb, v, m2, t2);
-            quantize(q, v, S);
+        for (int q0 = tl; q0 - lane < nchunks; q0 += kBurst * tpr) {
+            u32x4_t ra[kBurst], rb[kBurst];
+#pragma unroll
+            for (int j = 0; j < kBurst; ++j) issue(q0 + j * tpr, ra[j], rb[j]);
+#pragma unroll
+            for (int j = 0; j < kBurst; ++j) {
+                float v[8], m2 = 0.f, t2 = 0.f;
+                const int q = q0 + j * tpr;
+                values(q, ra[j], rb[j], v, m2, t2);
+                if (q - lane < nchunks) quantize(q, v, S);
+            }
         }
     }
 }

@@ -175,28 +175,12 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
             sin.in = st.in; sin.s_col = st.s_col; sin.K = st.K; sin.in_stride = st.in_stride;
             sin.in_f32 = st.in_f32; sin.in_coherent = st.in_coherent; sin.vec_in = st.vec_in;
 
-            // First fetches of the slice, issued before any wait: the weights are always ready.  The fp4 x fp8 path
-            // issues two items (4 KB) per wavefront here and keeps kQ8Depth in flight in the loop: a slice of one
-            // decoder layer is two or three items per wavefront, so its weights stream in while the input is still
-            // being waited for and staged.  (A third item here would push the kernel over its 128 registers.)
+            // First fetch of the slice, issued before any wait: the weights are always ready.  Not on the fp4 x fp8
+            // path: its staging needs the registers, and holding fetched words across it (measured with one, two and
+            // three items per wavefront) costs more in spills than the head start gains.
             uint4 wnext = make_uint4(0, 0, 0, 0);
-            uint4 wqa0 = wnext, wqb0 = wnext;
             if constexpr (kQ8) {
-                // items of the first row block: (pair of 16-row groups, 4-unit group), unit group fastest; wavefront
-                // w starts with item w * per; lane (row l & 15 of both groups, unit l >> 4)
-                const int ng0 = (chunk_units + 3) >> 2;
-                const int nrp0 = (min(seg.row_end - seg.row_begin, kRowBlock) + 31) >> 5;
-                const int per0 = mfma_items_per_wave(ng0 * nrp0, kWaves);
-                const int item0 = __builtin_amdgcn_readfirstlane(tid >> 6) * per0;
-                const int end0 = min(item0 + per0, ng0 * nrp0);
-                auto first = [&](int it, uint4& wa, uint4& wb) {
-                    const int u = 4 * (it % ng0) + ((tid & 63) >> 4);
-                    const int row = seg.row_begin + 32 * (it / ng0) + (tid & 15);
-                    const bool live = it < end0 && u < chunk_units;
-                    wa = load_unit(bv, min(row, st.rows - 1), u, live);
-                    wb = load_unit(bv, min(row + 16, st.rows - 1), u, live);
-                };
-                first(item0, wqa0, wqb0);
+                // nothing: see the loop (registers are scarcer than the head start is worth)
             } else if constexpr (MFMA) {
                 // wavefront w starts with item w of the first row block: 16 rows x 4 units, lane (row l & 15,
                 // unit l >> 4)
@@ -312,15 +296,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                             // is ever copied, and the main loop has no early exit.
                             static_assert(kQ8Depth == 3, "the rotation below is written out for three register pairs");
                             uint4 wa0, wb0, wa1, wb1, wa2, wb2;
-                            if (rb == seg.row_begin && c0 == 0) {            // fetched before the wait
-                                wa0 = wqa0; wb0 = wqb0;
-                                ++it_f;
-                                if (++ub_f == ngroups) { ub_f = 0; ++rp_f; }
-                                fetch(wa1, wb1);
-                                fetch(wa2, wb2);
-                            } else {
-                                fetch(wa0, wb0); fetch(wa1, wb1); fetch(wa2, wb2);
-                            }
+                            fetch(wa0, wb0); fetch(wa1, wb1); fetch(wa2, wb2);
                             Q8Operand opnd = {};
                             float4_t acc_a = {0.f, 0.f, 0.f, 0.f}, acc_b = {0.f, 0.f, 0.f, 0.f};
                             int rp_run = rp;
