@@ -27,7 +27,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the headline kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
 # copy kernel of known size (profiles/gemv_stream_llama2_7b_layer_b1.md); valid for the default workload only.
-MEASURED_TRAFFIC_BYTES = 33966528
+MEASURED_TRAFFIC_BYTES = 30667520
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 LLAMA2_7B_LAYER = (("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096),
@@ -190,7 +190,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f16 operands, f32 accumulate",
+        "dtype": "f16 in/out; one-bit fp4 x fp8-piece MFMA products (exact), f32 accumulate",
         "data": "synthetic",
         "config": {
             "workload": "cfg1: decode GEMV over the 7 linears of one Llama-2-7B decoder layer, batch 1, 1.0 bpw "
@@ -204,8 +204,8 @@ def main():
         "us_per_layer": round(ms * 1e3, 3),
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_stream_kernel<fp16, batch 1, MFMA, 512 lanes> (one launch per layer: 14 stages in 2 phases, "
-                      "512 resident workgroups)",
+            "kernel": "gemv_stream_kernel<fp16, batch 1, fp4 x fp8 MFMA, 1024 lanes> (one launch per layer: 14 stages in "
+                      "2 phases, 256 resident workgroups)",
             "achieved": round(bytes1 / launches_per_step / (launch_us * 1e-6) / 1e9, 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
