@@ -472,7 +472,8 @@ __device__ __forceinline__ float4_t pow2_combine(const float4_t (&acc)[kPow2Clas
 // element, u = x * s * S ~ q0 + q1 + q2 with q_k = fp8(u - q_0 - .. - q_{k-1}) and S a power of two that brings
 // the largest |u| of the staged slice into [128, 256): every piece carries 4 significant bits, three of them
 // reproduce u to 2^-12 relative or 2^-17 of the slice maximum, whichever is larger (fp16 staging keeps 2^-11
-// relative); all products are exact and accumulate in fp32.  Pieces and batch rows
+// relative); products are exact and accumulators fp32, but the instruction's internal 128-term sum keeps 13 bits
+// below its largest product (measured), which cuts elements far below the largest of their group at 2^-14 of it.  Pieces and batch rows
 // are columns of the B operand: column j = b * kQ8Pieces + piece, at most 16.
 //
 // Operand geometry (measured on gfx950 with one-hot operands): lane (i = l & 15, g = l >> 4) supplies

@@ -22,6 +22,12 @@ checkout):
   nominal_rank / checkpoint_rank   round(mn/(m+n)) and src/nanoquant/utils/utils.py:132-159
   torch_dense_forward     the same _compute_forward with torch.nn.functional.linear on dense
                           +-1 factors: the reference's CPU path, timed as the CPU baseline
+  fp8_e4m3_round / fp8_pieces / staged_input   no counterpart in the reference: the number format (OCP e4m3,
+                          round to nearest even) and the three-piece decomposition in which the gfx950 run-list
+                          kernel stages its input; lets a test state exactly what that kernel must compute
+
+Pinning of the fp8 helpers: against torch.float8_e4m3fn conversion on every finite fp8 value, on midpoints and on
+random inputs, and against the closed-form error bound of the decomposition (tests/test_oracle_layer.py).
 
 Pinning (tests/test_oracle_*.py): pack/unpack against hand-derived known-answer words and the
 committed fixtures in tests/golden/, a brute-force per-bit Python loop, the popcount and
@@ -251,3 +257,43 @@ def torch_dense_forward(x, vt, u, s_in, s_mid, s_out):
         y = y * s_mid
     y = F.linear(y, u)
     return y * s_out
+
+
+# ---- the input format of the gfx950 run-list kernel (batch <= 2) --------------------------------------
+def fp8_e4m3_round(v) -> np.ndarray:
+    """Round float64 values to the nearest OCP e4m3 number (ties to even, subnormals down to 2^-9, |v| <= 448
+    expected).  Returned as float64."""
+    v = np.asarray(v, dtype=np.float64)
+    a = np.abs(v)
+    e = np.floor(np.log2(np.where(a > 0, a, 1.0)))
+    e = np.clip(e, -6, 8)                       # binade of the value; below 2^-6 the spacing stays 2^-9
+    q = np.exp2(e - 3)                          # spacing: 3 mantissa bits
+    r = np.round(a / q) * q                     # numpy rounds halves to even
+    return np.sign(v) * np.minimum(r, 448.0)
+
+
+def fp8_pieces(u, pieces: int = 3) -> np.ndarray:
+    """[pieces, ...]: q_k = fp8(u - q_0 - ... - q_{k-1})."""
+    u = np.asarray(u, dtype=np.float64)
+    out = []
+    rest = u.copy()
+    for _ in range(pieces):
+        q = fp8_e4m3_round(rest)
+        out.append(q)
+        rest = rest - q
+    return np.stack(out)
+
+
+def staged_input(v, pieces: int = 3) -> np.ndarray:
+    """What the run-list kernel multiplies the signs with, per row of v [batch, K]: v scaled by the power of two
+    S that brings max |v| of the row into [128, 256), cut into fp8 pieces, summed and scaled back."""
+    v = np.asarray(v, dtype=np.float64)
+    out = np.zeros_like(v)
+    for b in range(v.shape[0]):
+        mx = np.abs(v[b]).max()
+        if mx == 0:
+            continue
+        s = np.exp2(7 - np.floor(np.log2(mx)))
+        out[b] = fp8_pieces(v[b] * s, pieces).sum(axis=0) / s
+    return out
+

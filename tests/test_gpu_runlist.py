@@ -57,6 +57,42 @@ def test_matches_per_linear_entry_point(dev):
     assert torch.allclose(y_rl, y_op, rtol=2e-3, atol=2e-4 * float(y_op.abs().max()))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("batch", [1, 2])
+def test_small_batches_compute_exactly_on_the_fp8_pieces(dev, batch, dtype):
+    # Up to batch 2 the kernel multiplies the signs with three fp8 pieces of x * s_in (resp. h * s_mid), scaled by
+    # the largest magnitude of the vector.  Restating that staging in the oracle predicts the output ten times
+    # closer than the 1e-3 budget of the dense definition: a missing or misplaced piece (7e-4), a wrong column,
+    # scale or class weight (O(1)) cannot hide in the tolerance.  What remains (1e-5 .. 5e-5 measured) is the
+    # instruction's own 128-term sum, which keeps 13 bits below its largest product (2^5 + 2^-9 gives 2^5).
+    m, n, r = 768, 1504, 416                       # ragged: 47 and 13 words per row
+    vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, 77)
+    x = oracle.synth_x(batch, n, 78)
+    to = lambda a: torch.from_numpy(a).to(dev).to(dtype)
+    xd, sd_in, sd_mid, sd_out = to(x), to(s_in), to(s_mid), to(s_out)
+    f64 = lambda t: t.float().cpu().numpy().astype(np.float64)
+
+    def stage(v, signs):
+        # sum +-v = (sum of v, taken exactly while staging) - 2 (sum of b * pieces of v), b = (1 - sign) / 2
+        q = oracle.staged_input(v)
+        return q @ signs.T.astype(np.float64) + (v - q).sum(axis=1, keepdims=True)
+
+    h = stage(f64(xd) * f64(sd_in)[None, :], vt).astype(np.float32).astype(np.float64)   # h is stored as fp32
+    ref = stage(h * f64(sd_mid)[None, :], u) * f64(sd_out)[None, :]
+    rl = DecodeRunList(batch, dtype, dev)
+    i = rl.add(xd, sd_in, packing.binary_packer(torch.from_numpy(vt), "half2").to(dev), sd_mid,
+               packing.binary_packer(torch.from_numpy(u), "half2").to(dev), sd_out, out_f32=True)
+    y = rl.run()[i]
+    torch.cuda.synchronize()
+    assert rl.status() == 0 and y.dtype == torch.float32
+    err = np.abs(y.cpu().numpy() - ref).max() / np.abs(ref).max()
+    print(f"exact-staging check batch={batch} {dtype}: {err:.3g}", flush=True)
+    assert err < 1e-4, err
+    # and the dense definition within the layer's budget
+    dense = oracle.layer_forward(f64(xd), vt, u, f64(sd_in), f64(sd_mid), f64(sd_out), dtype=np.float64)
+    assert np.abs(y.cpu().numpy() - dense).max() / np.abs(dense).max() < 1e-3
+
+
 def test_chained_linears_depend_on_each_other(dev):
     # y of linear i is x of linear i+1: the in-kernel dependency counters order them
     dims = [768, 512, 1024, 256]

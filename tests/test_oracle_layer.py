@@ -131,3 +131,40 @@ def test_rank_rules():
 def test_max_rel_err_metric():
     ref = np.array([[1.0, -4.0]])
     assert oracle.max_rel_err(ref + np.array([[0.02, 0.0]]), ref) == pytest.approx(0.005)
+
+
+# ---- the fp8 input format of the run-list kernel ------------------------------------------------------
+def test_fp8_rounding_matches_the_library_type():
+    # every finite e4m3 number is a fixed point; random values and all midpoints round as torch's type does
+    bits = torch.arange(256, dtype=torch.uint8)
+    vals = bits.view(torch.float8_e4m3fn).float().numpy().astype(np.float64)
+    vals = vals[np.isfinite(vals)]
+    assert len(vals) == 254 and np.abs(vals).max() == 448.0
+    assert np.array_equal(oracle.fp8_e4m3_round(vals), vals)
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.normal(0, 50, 20000), rng.normal(0, 0.01, 20000), rng.uniform(-448, 448, 20000)])
+    x = x[np.abs(x) <= 448].astype(np.float32).astype(np.float64)
+    t = torch.from_numpy(x).float().to(torch.float8_e4m3fn).float().numpy().astype(np.float64)
+    assert np.array_equal(oracle.fp8_e4m3_round(x), t)
+    grid = np.unique(np.abs(vals))
+    mid = (grid[:-1] + grid[1:]) / 2            # ties go to the even mantissa
+    t = torch.from_numpy(mid).float().to(torch.float8_e4m3fn).float().numpy().astype(np.float64)
+    assert np.array_equal(oracle.fp8_e4m3_round(mid), t)
+
+
+def test_three_fp8_pieces_reproduce_the_input():
+    # q0 + q1 + q2 = u up to 2^-12 relative, or the subnormal floor 2^-10 absolute (2^-17 of a maximum >= 128)
+    rng = np.random.default_rng(1)
+    u = np.concatenate([rng.uniform(-255.9, 255.9, 100000), rng.normal(0, 1e-2, 20000), [0.0, 255.99, -128.0, 2.0 ** -9]])
+    q = oracle.fp8_pieces(u, 3)
+    assert np.abs(q).max() <= 256               # never near the format's 448
+    err = np.abs(q.sum(axis=0) - u)
+    assert np.all(err <= np.maximum(2.0 ** -12 * np.abs(u), 2.0 ** -10))
+    # two pieces are not enough for the 1e-3 budget of the layer (worst element 2^-9), three are
+    assert np.max(np.abs(oracle.fp8_pieces(u, 2).sum(axis=0) - u) / np.maximum(np.abs(u), 1.0)) > 1e-3
+    # a whole vector: scaled by a power of two, so the decomposition of v is that of v * S
+    v = rng.normal(0, 0.02, (2, 512))
+    sv = oracle.staged_input(v)
+    assert np.all(np.abs(sv - v) <= np.maximum(2.0 ** -12 * np.abs(v), 2.0 ** -17 * np.abs(v).max(axis=1, keepdims=True)))
+    assert np.array_equal(oracle.staged_input(v * 8.0), sv * 8.0)
+    assert np.array_equal(oracle.staged_input(np.zeros((1, 64))), np.zeros((1, 64)))
