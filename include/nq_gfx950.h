@@ -56,6 +56,13 @@ int nq_gemv_forward(const void* x, const void* s_in, const uint32_t* vt_bits, co
                     const uint32_t* u_bits, const void* s_out, float* h_scratch, void* y,
                     int batch, int n, int r, int m, int dtype, void* stream);
 
+/* The same with y += bias (bias [m] of `dtype`, may be NULL), added in the epilogue of the second stage.  The
+ * reference's kernel paths drop the bias of a module (modules/linear.py:121-141 returns before :248-257 adds it);
+ * this entry point is what a caller uses to keep it. */
+int nq_gemv_forward_bias(const void* x, const void* s_in, const uint32_t* vt_bits, const void* s_mid,
+                         const uint32_t* u_bits, const void* s_out, const void* bias, float* h_scratch, void* y,
+                         int batch, int n, int r, int m, int dtype, void* stream);
+
 /* Decode path, sum of `nterms` terms that share x (the mixture-of-rank layer; no counterpart in the
  * reference's code, defined as the sum of single-term layers).  Arrays hold one pointer / rank per
  * term; s_mid[t] may be NULL.  h_scratch: fp32 [batch, max r]; y_scratch: fp32 [batch, m]. */
@@ -101,6 +108,7 @@ typedef struct nq_linear {
     int x_from;             /* -1: x is an external input */
     int y_from;             /* -1: addend (if any) is an external input */
     int out_f32;
+    const void* bias;       /* [m] of the list's dtype, added after s_out (before addend); may be NULL */
 } nq_linear;
 
 /* Launch geometry of a built run list; filled by nq_runlist_build, passed back to nq_runlist_run. */
@@ -133,6 +141,10 @@ int nq_gemv_stage(const void* in, const void* s_col, const uint32_t* bits, const
 size_t nq_gemm_scratch_bytes(int tokens, int k, int rows);
 int nq_gemm_onebit(const void* x, const uint32_t* tiles, const void* s_in, const void* s_out, void* y,
                    void* scratch, size_t scratch_bytes, int tokens, int k, int rows, int dtype, void* stream);
+/* The same with y[t, j] += bias[j] (bias [rows] of `dtype`, 16-byte aligned, may be NULL). */
+int nq_gemm_onebit_bias(const void* x, const uint32_t* tiles, const void* s_in, const void* s_out, const void* bias,
+                        void* y, void* scratch, size_t scratch_bytes, int tokens, int k, int rows, int dtype,
+                        void* stream);
 
 /* Prefill path, one term: two chained one-bit GEMMs with the intermediate h [tokens, r] (`dtype`,
  * caller-owned) between them.  Replaces marlin_nanoquant_cuda (kernel/cuda/gemm.cpp:112-122; schema
@@ -142,6 +154,10 @@ int nq_gemm_onebit(const void* x, const uint32_t* tiles, const void* s_in, const
 int nq_gemm_nanoquant(const void* x, const uint32_t* vt_tiles, const uint32_t* u_tiles, const void* s_in,
                       const void* s_mid, const void* s_out, void* h, void* y, void* scratch,
                       size_t scratch_bytes, int tokens, int n, int r, int m, int dtype, void* stream);
+/* The same with the bias [m] added in the epilogue of the second GEMM (may be NULL). */
+int nq_gemm_nanoquant_bias(const void* x, const uint32_t* vt_tiles, const uint32_t* u_tiles, const void* s_in,
+                           const void* s_mid, const void* s_out, const void* bias, void* h, void* y, void* scratch,
+                           size_t scratch_bytes, int tokens, int n, int r, int m, int dtype, void* stream);
 
 /* Word-order conversion on the device, in place allowed (dst == src): the checkpoint format
  * ("lsb_first", modules/linear.py:298) to the kernel format ("half2", modules/linear.py:171-172)

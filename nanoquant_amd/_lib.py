@@ -23,6 +23,7 @@ _SIGNATURES = {
     "nq_abi_version": (_i, []),
     "nq_device_query": (_i, [_i, ctypes.POINTER(_i)]),
     "nq_gemv_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "nq_gemv_forward_bias": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "nq_gemv_mixture": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "nq_runlist_workspace_bytes": (_sz, [_vp, _i]),
     "nq_runlist_build": (_i, [_vp, _i, _i, _i, _i, _vp, _sz, _vp, _vp]),
@@ -32,6 +33,8 @@ _SIGNATURES = {
     "nq_gemm_scratch_bytes": (_sz, [_i, _i, _i]),
     "nq_gemm_onebit": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),
     "nq_gemm_nanoquant": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
+    "nq_gemm_onebit_bias": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),
+    "nq_gemm_nanoquant_bias": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
     "nq_repack_words": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
     "nq_stream_copy": (_i, [_vp, _vp, _sz, _vp]),
 }

@@ -38,7 +38,7 @@ const char* nq_status_string(int status) {
 
 int nq_last_hip_error(void) { return g_last_hip_error; }
 
-int nq_abi_version(void) { return 1; }
+int nq_abi_version(void) { return 2; }
 
 int nq_device_query(int attr, int* value) {
     if (!value) return NQ_ERR_NULL;
@@ -58,6 +58,12 @@ int nq_device_query(int attr, int* value) {
 int nq_gemv_forward(const void* x, const void* s_in, const uint32_t* vt_bits, const void* s_mid,
                     const uint32_t* u_bits, const void* s_out, float* h_scratch, void* y,
                     int batch, int n, int r, int m, int dtype, void* stream) {
+    return nq_gemv_forward_bias(x, s_in, vt_bits, s_mid, u_bits, s_out, nullptr, h_scratch, y, batch, n, r, m, dtype, stream);
+}
+
+int nq_gemv_forward_bias(const void* x, const void* s_in, const uint32_t* vt_bits, const void* s_mid,
+                         const uint32_t* u_bits, const void* s_out, const void* bias, float* h_scratch, void* y,
+                         int batch, int n, int r, int m, int dtype, void* stream) {
     if (dtype != NQ_F16 && dtype != NQ_BF16) return NQ_ERR_DTYPE;
     if (batch < 0 || n < 0 || r < 0 || m < 0) return NQ_ERR_SHAPE;
     if (batch == 0 || m == 0) return NQ_OK;
@@ -67,7 +73,7 @@ int nq_gemv_forward(const void* x, const void* s_in, const uint32_t* vt_bits, co
                                   words_of(n), n, n, r, st);
     if (e != hipSuccess) return hip_status(e);
     e = nq::gemv_stage(dtype, false, u_bits, h_scratch, nullptr, s_out, nullptr, y, false, batch, m,
-                       words_of(r), r, r, m, st);
+                       words_of(r), r, r, m, st, bias);
     return hip_status(e);
 }
 
@@ -180,7 +186,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
 
         nq::RunStage b{};
         b.bits = l.u_bits; b.in = l.h; b.s_col = nullptr; b.s_row = (const uint16_t*)l.s_out;
-        b.out = l.y; b.addend = l.addend;
+        b.out = l.y; b.addend = l.addend; b.bias = (const uint16_t*)l.bias;
         b.rows = l.m; b.K = l.r; b.words = (l.r + 31) / 32; b.units = (b.words + 3) / 4;
         b.in_stride = l.r; b.out_stride = l.m; b.in_f32 = 1; b.out_f32 = l.out_f32 ? 1 : 0;
         b.dep = 2 * i;
@@ -374,25 +380,39 @@ size_t nq_gemm_scratch_bytes(int tokens, int k, int rows) { return nq::gemm_scra
 
 int nq_gemm_onebit(const void* x, const uint32_t* tiles, const void* s_in, const void* s_out, void* y,
                    void* scratch, size_t scratch_bytes, int tokens, int k, int rows, int dtype, void* stream) {
+    return nq_gemm_onebit_bias(x, tiles, s_in, s_out, nullptr, y, scratch, scratch_bytes, tokens, k, rows, dtype, stream);
+}
+
+int nq_gemm_onebit_bias(const void* x, const uint32_t* tiles, const void* s_in, const void* s_out, const void* bias,
+                        void* y, void* scratch, size_t scratch_bytes, int tokens, int k, int rows, int dtype,
+                        void* stream) {
     if (dtype != NQ_F16 && dtype != NQ_BF16) return NQ_ERR_DTYPE;
     if (tokens < 0 || k < 0 || rows < 0) return NQ_ERR_SHAPE;
     if (k % 256 != 0 || rows % 32 != 0) return NQ_ERR_PROB_SHAPE;
     if (tokens == 0 || rows == 0 || k == 0) return NQ_OK;
     if (!x || !tiles || !y) return NQ_ERR_NULL;
-    if (((uintptr_t)x | (uintptr_t)tiles | (uintptr_t)y | (uintptr_t)s_in | (uintptr_t)scratch) & 15u) return NQ_ERR_ALIGN;
+    if (((uintptr_t)x | (uintptr_t)tiles | (uintptr_t)y | (uintptr_t)s_in | (uintptr_t)scratch | (uintptr_t)bias) & 15u)
+        return NQ_ERR_ALIGN;
     const size_t need = nq::gemm_scratch_bytes(tokens, k, rows);
     if (need > 0 && (!scratch || scratch_bytes < need)) return NQ_ERR_WORKSPACE;
     return hip_status(nq::gemm_onebit(dtype, x, tiles, s_in, s_out, y, (float*)scratch, tokens, k, rows,
-                                      (hipStream_t)stream));
+                                      (hipStream_t)stream, bias));
 }
 
 int nq_gemm_nanoquant(const void* x, const uint32_t* vt_tiles, const uint32_t* u_tiles, const void* s_in,
                       const void* s_mid, const void* s_out, void* h, void* y, void* scratch,
                       size_t scratch_bytes, int tokens, int n, int r, int m, int dtype, void* stream) {
+    return nq_gemm_nanoquant_bias(x, vt_tiles, u_tiles, s_in, s_mid, s_out, nullptr, h, y, scratch, scratch_bytes, tokens, n, r,
+                                  m, dtype, stream);
+}
+
+int nq_gemm_nanoquant_bias(const void* x, const uint32_t* vt_tiles, const uint32_t* u_tiles, const void* s_in,
+                           const void* s_mid, const void* s_out, const void* bias, void* h, void* y, void* scratch,
+                           size_t scratch_bytes, int tokens, int n, int r, int m, int dtype, void* stream) {
     if (!h) return (tokens == 0 || m == 0) ? NQ_OK : NQ_ERR_NULL;
     int st = nq_gemm_onebit(x, vt_tiles, s_in, s_mid, h, scratch, scratch_bytes, tokens, n, r, dtype, stream);
     if (st != NQ_OK) return st;
-    return nq_gemm_onebit(h, u_tiles, nullptr, s_out, y, scratch, scratch_bytes, tokens, r, m, dtype, stream);
+    return nq_gemm_onebit_bias(h, u_tiles, nullptr, s_out, bias, y, scratch, scratch_bytes, tokens, r, m, dtype, stream);
 }
 
 int nq_repack_words(const uint32_t* src, uint32_t* dst, size_t nwords, int src_order, int dst_order, void* stream) {

@@ -28,6 +28,7 @@ struct GemmArgs {
     const uint4* tiles;     // [R/32][K/256][64 lanes] 16 bytes each
     const uint16_t* s_in;   // [K] or null
     const uint16_t* s_out;  // [R] or null
+    const uint16_t* bias;   // [R] added after the output scale, or null
     void* y;                // [T, R] 16-bit
     float* acc;             // [T, R] fp32 partial sums (k-split only)
     int T, K, R;
@@ -195,8 +196,9 @@ __global__ __launch_bounds__(256) void gemm_onebit_kernel(GemmArgs a) {
     for (int r = 0; r < RT; ++r) {
         if (r >= ntiles) break;
         const int row = (rt + r) * 32 + (lane & 31);
-        float sc = 1.f;
+        float sc = 1.f, bs = 0.f;
         if (!SPLIT && a.s_out) sc = E::to_float(a.s_out[row]);
+        if (!SPLIT && a.bias) bs = E::to_float(a.bias[row]);
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) {
 #pragma unroll
@@ -205,7 +207,7 @@ __global__ __launch_bounds__(256) void gemm_onebit_kernel(GemmArgs a) {
                 if (tok < a.T) {
                     const size_t o = (size_t)tok * a.R + row;
                     if (SPLIT) atomicAdd(a.acc + o, acc[r][tt][v]);
-                    else ((uint16_t*)a.y)[o] = E::from_float_sat(acc[r][tt][v] * sc);
+                    else ((uint16_t*)a.y)[o] = E::from_float_sat(acc[r][tt][v] * sc + bs);
                 }
             }
         }
@@ -331,13 +333,15 @@ __global__ __launch_bounds__(256) void gemm_kwave_kernel(GemmArgs a) {
                 sums[j] = (pr[(0 * 16 + v) * 64 + l0 + j] + pr[(1 * 16 + v) * 64 + l0 + j]) +
                           (pr[(2 * 16 + v) * 64 + l0 + j] + pr[(3 * 16 + v) * 64 + l0 + j]);
             u32x4_t sc = {E::kOnePair, E::kOnePair, E::kOnePair, E::kOnePair};
+            u32x4_t bs = {0u, 0u, 0u, 0u};
             if (a.s_out) sc = *(const u32x4_t*)(a.s_out + row0);
+            if (a.bias) bs = *(const u32x4_t*)(a.bias + row0);
             u32x4_t outv;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const uint32_t sw = sc[j];
-                const uint16_t lo = E::from_float_sat(sums[2 * j] * E::to_float((uint16_t)(sw & 0xFFFFu)));
-                const uint16_t hi = E::from_float_sat(sums[2 * j + 1] * E::to_float((uint16_t)(sw >> 16)));
+                const uint32_t sw = sc[j], bw = bs[j];
+                const uint16_t lo = E::from_float_sat(sums[2 * j] * E::to_float((uint16_t)(sw & 0xFFFFu)) + E::to_float((uint16_t)(bw & 0xFFFFu)));
+                const uint16_t hi = E::from_float_sat(sums[2 * j + 1] * E::to_float((uint16_t)(sw >> 16)) + E::to_float((uint16_t)(bw >> 16)));
                 outv[j] = (uint32_t)lo | ((uint32_t)hi << 16);
             }
             if (tok < a.T) *(u32x4_t*)((uint16_t*)a.y + (size_t)tok * a.R + row0) = outv;
@@ -348,7 +352,8 @@ __global__ __launch_bounds__(256) void gemm_kwave_kernel(GemmArgs a) {
 // Scales, converts and stores the accumulated sums, and puts the accumulator back to zero: the scratch
 // is zero on entry of every GEMM call and zero again when the call has finished.
 template <int DT>
-__global__ __launch_bounds__(256) void gemm_finish_kernel(float4* acc, const uint16_t* s_out, uint16_t* y, int R, size_t n4) {
+__global__ __launch_bounds__(256) void gemm_finish_kernel(float4* acc, const uint16_t* s_out, const uint16_t* bias, uint16_t* y, int R,
+                                                          size_t n4) {
     using E = Elem<DT>;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
@@ -360,9 +365,14 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(float4* acc, const uin
             s0 = E::to_float(s_out[row]); s1 = E::to_float(s_out[row + 1]);
             s2 = E::to_float(s_out[row + 2]); s3 = E::to_float(s_out[row + 3]);
         }
+        float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
+        if (bias) {
+            b0 = E::to_float(bias[row]); b1 = E::to_float(bias[row + 1]);
+            b2 = E::to_float(bias[row + 2]); b3 = E::to_float(bias[row + 3]);
+        }
         uint2 o;
-        o.x = (uint32_t)E::from_float_sat(v.x * s0) | ((uint32_t)E::from_float_sat(v.y * s1) << 16);
-        o.y = (uint32_t)E::from_float_sat(v.z * s2) | ((uint32_t)E::from_float_sat(v.w * s3) << 16);
+        o.x = (uint32_t)E::from_float_sat(v.x * s0 + b0) | ((uint32_t)E::from_float_sat(v.y * s1 + b1) << 16);
+        o.y = (uint32_t)E::from_float_sat(v.z * s2 + b2) | ((uint32_t)E::from_float_sat(v.w * s3 + b3) << 16);
         ((uint2*)y)[i] = o;
     }
 }
@@ -459,7 +469,7 @@ static hipError_t launch_gemm(const GemmArgs& a, const GemmPlan& p, hipStream_t 
         size_t zb = (n4 + 255) / 256;
         if (zb > 2048) zb = 2048;
         hipLaunchKernelGGL(gemm_finish_kernel<DT>, dim3((unsigned)zb), dim3(256), 0, stream, (float4*)a.acc, a.s_out,
-                           (uint16_t*)a.y, a.R, n4);
+                           a.bias, (uint16_t*)a.y, a.R, n4);
     } else {
         e = scaled ? launch_variant<DT, TT, RT, KS, false, true>(a, grid, lds, stream)
                    : launch_variant<DT, TT, RT, KS, false, false>(a, grid, lds, stream);
@@ -471,10 +481,10 @@ static hipError_t launch_gemm(const GemmArgs& a, const GemmPlan& p, hipStream_t 
 // Shapes must satisfy K % 256 == 0 and R % 32 == 0 (checked by the caller).  `scratch` (when
 // gemm_scratch_bytes > 0) must be zero on entry and is zero again when the enqueued work has finished.
 hipError_t gemm_onebit(int dtype, const void* x, const uint32_t* tiles, const void* s_in, const void* s_out,
-                       void* y, float* scratch, int T, int K, int R, hipStream_t stream) {
+                       void* y, float* scratch, int T, int K, int R, hipStream_t stream, const void* bias) {
     GemmArgs a;
     a.x = x; a.tiles = (const uint4*)tiles;
-    a.s_in = (const uint16_t*)s_in; a.s_out = (const uint16_t*)s_out;
+    a.s_in = (const uint16_t*)s_in; a.s_out = (const uint16_t*)s_out; a.bias = (const uint16_t*)bias;
     a.y = y; a.acc = scratch;
     a.T = T; a.K = K; a.R = R;
     a.ktiles = K / kTileK;

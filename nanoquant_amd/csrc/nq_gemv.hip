@@ -34,6 +34,7 @@ struct StageArgs {
     int vec_bits;           // rows of `bits` are 16-byte aligned and words % 4 == 0
     int vec_in;             // rows of `in` (and s_col) allow 16-byte loads
     const float* addend;    // [batch, out_stride] fp32 added before the store (sum over terms), may be null
+    const uint16_t* bias;   // [rows] added after the row scale, may be null
     int out_f32;            // store fp32 instead of the 16-bit activation type
 };
 
@@ -118,11 +119,12 @@ __global__ __launch_bounds__(256) void gemv_stage_kernel(StageArgs a) {
 #pragma unroll
     for (int rr = 0; rr < RPW; ++rr) {
         const int row = row0 + rr;
-        float sc = 1.f;
+        float sc = 1.f, bs = 0.f;
         if (a.s_row && row < a.rows) sc = E::to_float(a.s_row[row]);
+        if (a.bias && row < a.rows) bs = E::to_float(a.bias[row]);
 #pragma unroll
         for (int b = 0; b < BATCH; ++b) {
-            float v = group_sum(acc[rr][b], G) * sc;
+            float v = group_sum(acc[rr][b], G) * sc + bs;
             if (g == 0 && row < a.rows) {
                 const size_t o = (size_t)b * a.out_stride + row;
                 if (a.addend) v += a.addend[o];
@@ -194,10 +196,11 @@ static bool use_stream_kernel(int piece) { return piece >= 16; }
 // One stage over `batch` input rows, any batch >= 1: split into power-of-two pieces of at most 16.
 hipError_t gemv_stage(int dtype, bool first, const uint32_t* bits, const void* in, const void* s_col,
                       const void* s_row, const float* addend, void* out, bool out_f32, int batch, int rows,
-                      int words, int K, int in_stride, int out_stride, hipStream_t stream) {
+                      int words, int K, int in_stride, int out_stride, hipStream_t stream, const void* bias) {
     if (rows <= 0 || batch <= 0) return hipSuccess;
     StageArgs a;
     a.bits = bits;
+    a.bias = (const uint16_t*)bias;
     a.s_col = (const uint16_t*)s_col;
     a.s_row = (const uint16_t*)s_row;
     a.rows = rows; a.words = words; a.K = K;
@@ -223,7 +226,7 @@ hipError_t gemv_stage(int dtype, bool first, const uint32_t* bits, const void* i
         hipError_t e;
         if (use_stream_kernel(piece) && (size_t)rows * words * 4 < 0x7FFFFFF0ull) {
             RunStage st{};
-            st.bits = bits; st.in = a.in; st.s_col = a.s_col; st.s_row = a.s_row; st.out = a.out; st.addend = a.addend;
+            st.bits = bits; st.in = a.in; st.s_col = a.s_col; st.s_row = a.s_row; st.out = a.out; st.addend = a.addend; st.bias = a.bias;
             st.rows = rows; st.words = words; st.K = K; st.units = a.units;
             st.in_stride = in_stride; st.out_stride = out_stride;
             st.in_f32 = first ? 0 : 1; st.out_f32 = a.out_f32;

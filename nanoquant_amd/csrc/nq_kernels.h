@@ -10,7 +10,8 @@ namespace nq {
 // activation type (clamped); `addend` (fp32, same shape as out) is added before the store.
 hipError_t gemv_stage(int dtype, bool first, const uint32_t* bits, const void* in, const void* s_col,
                       const void* s_row, const float* addend, void* out, bool out_f32, int batch, int rows,
-                      int words, int K, int in_stride, int out_stride, hipStream_t stream);
+                      int words, int K, int in_stride, int out_stride, hipStream_t stream,
+                      const void* bias = nullptr);
 
 // nq_stream.hip: one launch over a table of stages (see the file header).
 struct RunStage {
@@ -20,6 +21,7 @@ struct RunStage {
     const uint16_t* s_row;  // [rows] per-row scale, may be null
     void* out;              // [batch, out_stride]: fp32 when out_f32, else 16-bit (clamped)
     const float* addend;    // fp32 [batch, out_stride] added before the store, may be null
+    const uint16_t* bias;   // [rows] added after the row scale, may be null
     int rows, words, K, units;
     int in_stride, out_stride;
     int in_f32, out_f32;
@@ -50,7 +52,7 @@ hipError_t gemv_stream_single(int dtype, int batch, const RunStage& st, hipStrea
 // scratch: fp32 [T,R] when gemm_scratch_bytes(T,K,R) > 0.
 size_t gemm_scratch_bytes(int T, int K, int R);
 hipError_t gemm_onebit(int dtype, const void* x, const uint32_t* tiles, const void* s_in, const void* s_out,
-                       void* y, float* scratch, int T, int K, int R, hipStream_t stream);
+                       void* y, float* scratch, int T, int K, int R, hipStream_t stream, const void* bias = nullptr);
 
 // nq_util.hip
 hipError_t stream_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);

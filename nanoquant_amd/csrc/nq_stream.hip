@@ -456,6 +456,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                         float v = racc[i];
                         if constexpr (kTotals) v += xtot[b];
                         if (st.s_row) v *= E::to_float(st.s_row[row]);
+                        if (st.bias) v += E::to_float(st.bias[row]);
                         const size_t o = (size_t)b * st.out_stride + row;
                         if (st.addend) {
                             if (st.dep2 >= 0)

@@ -39,6 +39,9 @@ class NanoQuantLinear(nn.Module):
         self.do_train = False
         self._binarized = True
         self.dtype = dtype
+        # False mirrors the reference, whose kernel paths return before the bias is added; True adds it in the
+        # epilogue of the last kernel (decode and prefill alike).
+        self.kernel_path_bias = False
         self.register_parameter("weight", None)
         if bias:
             self.bias = nn.Parameter(torch.zeros(out_features, device=device, dtype=dtype), requires_grad=False)
@@ -104,16 +107,28 @@ class NanoQuantLinear(nn.Module):
             else:
                 raise ValueError(f"Expected 2D or 3D input tensor, got {x.ndim}D")
 
+            # As in the reference (linear.py:121-141) the kernel paths do not add the bias, unless
+            # `kernel_path_bias` is set: then it is added in the epilogue of the last kernel.
+            bias = None
+            if self.kernel_path_bias and self.bias is not None:
+                bias = self.bias if self.bias.dtype == self.dtype else self.bias.to(self.dtype)
             if self.kernel_type == "gemv":
-                y = self.kernel_forward(x, self.scale_pre, self.V_int8, self.scale_mid, self.U_int8,
-                                        self.scale_post, **self.kernel_kwargs)
+                if bias is not None:
+                    y = ops.gemv_forward_with_bias(x, self.scale_pre, self.V_int8, self.scale_mid, self.U_int8,
+                                                   self.scale_post, bias)
+                else:
+                    y = self.kernel_forward(x, self.scale_pre, self.V_int8, self.scale_mid, self.U_int8,
+                                            self.scale_post, **self.kernel_kwargs)
             elif self.kernel_type == "gemm":
-                y = self.kernel_forward(x, self.V_int8, self.U_int8, self.s1, self.s2, self.s3, self.workspace)
+                if bias is not None:
+                    y = ops.gemm_forward_with_bias(x, self.V_int8, self.U_int8, self.s1, self.s2, self.s3, self.workspace,
+                                                   bias)
+                else:
+                    y = self.kernel_forward(x, self.V_int8, self.U_int8, self.s1, self.s2, self.s3, self.workspace)
             else:
                 raise ValueError(f"Unknown kernel_type: {self.kernel_type}")
             if original_shape is not None:
                 y = y.view(original_shape[0], original_shape[1], -1)
-            # As in the reference (linear.py:121-141), the kernel paths do not add the bias.
             return y.to(orig_dtype) if y.dtype != orig_dtype else y
 
         s_mid = getattr(self, "scale_mid", None)

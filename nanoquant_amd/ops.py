@@ -121,22 +121,17 @@ def _check_gemv_args(x, scale_g, Ubits, scale_l, Vbits, scale_h):
     return n, r, m
 
 
-def nanoquant_dyn_forward(x, scale_g, Ubits, scale_l, Vbits, scale_h,
-                          num_thread_stage1=128, num_thread_stage2=128,
-                          num_row_per_warp_stage1=2, num_row_per_warp_stage2=2,
-                          num_acc_stage1=4, num_acc_stage2=4,
-                          num_pipeline_stage1=2, num_pipeline_stage2=2):
-    """y = scale_h * (Vbits (scale_l * (Ubits (scale_g * x)))): `Ubits` [r, n/32] is the FIRST stage,
-    `Vbits` [m, r/32] the second (the reference's argument names, pybind.cpp:86-90)."""
+def _check_bias(bias, m, x):
+    if bias is None:
+        return
+    _check_dev_cont(bias, "bias", x.dtype, "Bias")
+    if bias.dim() != 1 or bias.size(0) != m:
+        raise RuntimeError(f"bias must be [{m}], got {list(bias.shape)}")
+
+
+def _gemv_forward(x, scale_g, Ubits, scale_l, Vbits, scale_h, bias=None):
     n, r, m = _check_gemv_args(x, scale_g, Ubits, scale_l, Vbits, scale_h)
-    _sweep("n_th1", num_thread_stage1)
-    _sweep("n_rpw1", num_row_per_warp_stage1)
-    _sweep("n_acc1", num_acc_stage1)
-    _sweep("n_pipe1", num_pipeline_stage1)
-    _sweep("n_th2", num_thread_stage2)
-    _sweep("n_rpw2", num_row_per_warp_stage2)
-    _sweep("n_acc2", num_acc_stage2)
-    _sweep("n_pipe2", num_pipeline_stage2)
+    _check_bias(bias, m, x)
     lead = x.shape[:-1]
     batch = 1
     for d in lead:
@@ -145,10 +140,29 @@ def nanoquant_dyn_forward(x, scale_g, Ubits, scale_l, Vbits, scale_h,
     if batch > 0 and m > 0:
         h = torch.empty((batch, max(r, 1)), dtype=torch.float32, device=x.device)
         with torch.cuda.device(x.device):
-            _lib.check(_lib.lib().nq_gemv_forward(_ptr(x), _ptr(scale_g), _ptr(Ubits), _ptr(scale_l), _ptr(Vbits),
-                                                  _ptr(scale_h), _ptr(h), _ptr(y), batch, n, r, m, _dtype_id(x),
-                                                  _stream(x.device)))
+            _lib.check(_lib.lib().nq_gemv_forward_bias(_ptr(x), _ptr(scale_g), _ptr(Ubits), _ptr(scale_l), _ptr(Vbits),
+                                                       _ptr(scale_h), _ptr(bias), _ptr(h), _ptr(y), batch, n, r, m,
+                                                       _dtype_id(x), _stream(x.device)))
     return y.reshape(*lead, m)
+
+
+def nanoquant_dyn_forward(x, scale_g, Ubits, scale_l, Vbits, scale_h,
+                          num_thread_stage1=128, num_thread_stage2=128,
+                          num_row_per_warp_stage1=2, num_row_per_warp_stage2=2,
+                          num_acc_stage1=4, num_acc_stage2=4,
+                          num_pipeline_stage1=2, num_pipeline_stage2=2):
+    """y = scale_h * (Vbits (scale_l * (Ubits (scale_g * x)))): `Ubits` [r, n/32] is the FIRST stage,
+    `Vbits` [m, r/32] the second (the reference's argument names, pybind.cpp:86-90)."""
+    _check_gemv_args(x, scale_g, Ubits, scale_l, Vbits, scale_h)
+    _sweep("n_th1", num_thread_stage1)
+    _sweep("n_rpw1", num_row_per_warp_stage1)
+    _sweep("n_acc1", num_acc_stage1)
+    _sweep("n_pipe1", num_pipeline_stage1)
+    _sweep("n_th2", num_thread_stage2)
+    _sweep("n_rpw2", num_row_per_warp_stage2)
+    _sweep("n_acc2", num_acc_stage2)
+    _sweep("n_pipe2", num_pipeline_stage2)
+    return _gemv_forward(x, scale_g, Ubits, scale_l, Vbits, scale_h)
 
 
 def _nanoquant_dyn_forward_meta(x, scale_g, Ubits, scale_l, Vbits, scale_h, *hints, **kw):
@@ -236,9 +250,7 @@ def _marlin_onebit_meta(x, weight, scale_g, scale_h, workspace):
     return x.new_empty((m, n))
 
 
-def marlin_nanoquant_forward(x, weight_u, weight_v, scale_g, scale_l, scale_h, workspace):
-    """Two chained one-bit GEMMs (gemm.cpp:112-122): `weight_u` is the FIRST stage [n -> r],
-    `weight_v` the second [r -> m] (the order marlin_nanoquant_packer returns them)."""
+def _gemm_nanoquant_forward(x, weight_u, weight_v, scale_g, scale_l, scale_h, workspace, bias=None):
     dt = _gemm_dtype(x)
     t, r, n = _onebit_check(x, weight_u, scale_g, scale_l, workspace)
     _check_gemm_tensor(x, "x")
@@ -248,16 +260,23 @@ def marlin_nanoquant_forward(x, weight_u, weight_v, scale_g, scale_l, scale_h, w
         _check_gemm_tensor(s, name, x.dtype)
     imm = torch.empty((t, r), dtype=x.dtype, device=x.device)
     _, m, _ = _onebit_check(imm, weight_v, None, scale_h, workspace)
+    _check_bias(bias, m, x)
     out = torch.empty((t, m), dtype=x.dtype, device=x.device)
     if t == 0 or m == 0:
         return out
     nbytes = max(int(_lib.lib().nq_gemm_scratch_bytes(t, n, r)), int(_lib.lib().nq_gemm_scratch_bytes(t, r, m)))
     scratch = _scratch(nbytes, x.device)
     with torch.cuda.device(x.device):
-        _lib.check(_lib.lib().nq_gemm_nanoquant(_ptr(x), _ptr(weight_u), _ptr(weight_v), _ptr(scale_g), _ptr(scale_l),
-                                                _ptr(scale_h), _ptr(imm), _ptr(out), _ptr(scratch), nbytes,
-                                                t, n, r, m, dt, _stream(x.device)))
+        _lib.check(_lib.lib().nq_gemm_nanoquant_bias(_ptr(x), _ptr(weight_u), _ptr(weight_v), _ptr(scale_g), _ptr(scale_l),
+                                                     _ptr(scale_h), _ptr(bias), _ptr(imm), _ptr(out), _ptr(scratch), nbytes,
+                                                     t, n, r, m, dt, _stream(x.device)))
     return out
+
+
+def marlin_nanoquant_forward(x, weight_u, weight_v, scale_g, scale_l, scale_h, workspace):
+    """Two chained one-bit GEMMs (gemm.cpp:112-122): `weight_u` is the FIRST stage [n -> r],
+    `weight_v` the second [r -> m] (the order marlin_nanoquant_packer returns them)."""
+    return _gemm_nanoquant_forward(x, weight_u, weight_v, scale_g, scale_l, scale_h, workspace)
 
 
 def _marlin_nanoquant_meta(x, weight_u, weight_v, scale_g, scale_l, scale_h, workspace):
@@ -270,6 +289,17 @@ def _marlin_nanoquant_meta(x, weight_u, weight_v, scale_g, scale_l, scale_h, wor
 # ---------------------------------------------------------------------------------------------
 # extras above the reference's surface (plain functions, not dispatcher ops)
 # ---------------------------------------------------------------------------------------------
+def gemv_forward_with_bias(x, scale_g, Ubits, scale_l, Vbits, scale_h, bias):
+    """nanoquant_dyn_forward + bias [m], added in the epilogue of the second stage.  The reference's kernel paths
+    return before the module's bias is added (modules/linear.py:121-141); this keeps it."""
+    return _gemv_forward(x, scale_g, Ubits, scale_l, Vbits, scale_h, bias)
+
+
+def gemm_forward_with_bias(x, weight_u, weight_v, scale_g, scale_l, scale_h, workspace, bias):
+    """marlin_nanoquant_forward + bias [m], added in the epilogue of the second GEMM."""
+    return _gemm_nanoquant_forward(x, weight_u, weight_v, scale_g, scale_l, scale_h, workspace, bias)
+
+
 def gemv_mixture_forward(x, terms):
     """Sum of several binary low-rank terms sharing x.  terms: sequence of
     (scale_g, Ubits, scale_l | None, Vbits, scale_h) with the operand meaning of nanoquant_dyn_forward."""

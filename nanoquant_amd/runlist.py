@@ -24,6 +24,7 @@ class NqLinear(ctypes.Structure):
         ("addend", ctypes.c_void_p),
         ("n", ctypes.c_int), ("r", ctypes.c_int), ("m", ctypes.c_int),
         ("x_from", ctypes.c_int), ("y_from", ctypes.c_int), ("out_f32", ctypes.c_int),
+        ("bias", ctypes.c_void_p),
     ]
 
 
@@ -54,10 +55,10 @@ class DecodeRunList:
     def add(self, x: torch.Tensor, scale_pre: torch.Tensor, V_int8: torch.Tensor, scale_mid: Optional[torch.Tensor],
             U_int8: torch.Tensor, scale_post: torch.Tensor, y: Optional[torch.Tensor] = None,
             x_from: int = -1, addend: Optional[torch.Tensor] = None, y_from: int = -1,
-            out_f32: bool = False) -> int:
+            out_f32: bool = False, bias: Optional[torch.Tensor] = None) -> int:
         """Append one linear (operands as `NanoQuantLinear` holds them after `_prepare_kernel('gemv')`:
         V_int8 [r, n/32] first stage, U_int8 [m, r/32] second stage).  Returns its index; `y` is
-        allocated when not given and is available as `outputs[index]`."""
+        allocated when not given and is available as `outputs[index]`.  `bias` [m] is added after `scale_post`."""
         n = x.shape[-1]
         r, m = V_int8.shape[0], U_int8.shape[0]
         for name, t, dt in (("x", x, self.dtype), ("scale_pre", scale_pre, self.dtype), ("scale_post", scale_post, self.dtype),
@@ -70,12 +71,15 @@ class DecodeRunList:
             raise RuntimeError("packed factor shapes do not match x / each other")
         if scale_pre.numel() != n or scale_post.numel() != m or (scale_mid is not None and scale_mid.numel() != r):
             raise RuntimeError("scale size mismatch")
+        if bias is not None and (not bias.is_cuda or not bias.is_contiguous() or bias.dtype != self.dtype or bias.numel() != m):
+            raise RuntimeError(f"bias must be a contiguous {self.dtype} tensor of {m} elements on the GPU")
         if y is None:
             y = torch.empty((self.batch, m), dtype=torch.float32 if out_f32 else self.dtype, device=self.device)
         h = torch.empty((self.batch, r), dtype=torch.float32, device=self.device)
-        self._keep += [x, scale_pre, V_int8, scale_mid, U_int8, scale_post, y, h, addend]
+        self._keep += [x, scale_pre, V_int8, scale_mid, U_int8, scale_post, y, h, addend, bias]
         self._entries.append(dict(x=x, s_in=scale_pre, vt=V_int8, s_mid=scale_mid, u=U_int8, s_out=scale_post, h=h, y=y,
-                                  addend=addend, n=n, r=r, m=m, x_from=x_from, y_from=y_from, out_f32=int(out_f32)))
+                                  addend=addend, n=n, r=r, m=m, x_from=x_from, y_from=y_from, out_f32=int(out_f32),
+                                  bias=bias))
         self._workspace = None
         return len(self._entries) - 1
 
@@ -91,7 +95,8 @@ class DecodeRunList:
         p = lambda t: None if t is None else t.data_ptr()
         for i, e in enumerate(self._entries):
             arr[i] = NqLinear(p(e["x"]), p(e["s_in"]), p(e["vt"]), p(e["s_mid"]), p(e["u"]), p(e["s_out"]), p(e["h"]),
-                              p(e["y"]), p(e["addend"]), e["n"], e["r"], e["m"], e["x_from"], e["y_from"], e["out_f32"])
+                              p(e["y"]), p(e["addend"]), e["n"], e["r"], e["m"], e["x_from"], e["y_from"], e["out_f32"],
+                              p(e["bias"]))
         lib = _lib.lib()
         nbytes = int(lib.nq_runlist_workspace_bytes(arr, n))
         ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
