@@ -1,16 +1,14 @@
-// Decode path, run-list form: ONE launch covers a whole list of matmul-free stages.
+// Decode path, run-list form: ONE launch covers a whole list of stages (out[b, row] = s_row[row] * sum of
+// signed, scaled inputs; two stages per linear).
 //
 // A decoder stack at batch 1 is a stream of small sign matrices (1-6 MB each) and a 4096x4096 layer
 // is worth 0.3 us of HBM time, so launching one kernel per stage (as the reference does,
 // src/nanoquant/kernel/cuda/gemv_kernel.cu:406-425: two launches per linear) leaves the memory system
-// idle most of the time.  Here the grid is exactly as large as the device can keep resident (a few
-// workgroups per CU) and the stages are grouped into phases by dependency depth (all first stages of
+// idle most of the time.  Here the grid is exactly as large as the device can keep resident (one 1024-lane
+// workgroup per CU) and the stages are grouped into phases by dependency depth (all first stages of
 // independent linears are phase 0, their second stages phase 1, ...):
 //   * every workgroup owns a balanced slice (in units of sign words) of every phase, cut at row
-//     boundaries by the host: no workgroup slot ever idles while another phase is running, and the
-//     several workgroups of a CU cover each other's latencies;
-//   * the sign words of a slice do not depend on any activation, so each lane issues its first
-//     128-bit fetch before the slice waits for the producer of its input;
+//     boundaries by the host: no workgroup slot ever idles while another phase is running;
 //   * a slice whose input is produced by an earlier stage waits on that stage's completion counters
 //     (device-scope atomics), not on a kernel boundary.  All workgroups are resident, so the producers
 //     are always running; the wait is bounded all the same and an expiry is reported through the
@@ -18,8 +16,8 @@
 //   * the intermediate h is handed over with relaxed device-scope atomics (coherent 32/64-bit
 //     accesses) instead of cache-wide release/acquire fences, which on this part write back and
 //     invalidate a whole L2 per workgroup;
-//   * inside a workgroup the (row, 16-byte unit) pairs are dealt round-robin to the 256 lanes,
-//     whatever the shape, and per-row sums are finished with LDS float atomics.
+//   * inside a workgroup the sign words go to the MFMA units as (16 rows x 4 units) items, one row and unit
+//     per lane; wavefronts take contiguous runs of items and finish per-row sums with LDS float atomics.
 // The arithmetic per 16-byte unit is in nq_decode.h.
 #include "nq_decode.h"
 #include "nq_kernels.h"
@@ -103,8 +101,7 @@ __host__ __device__ constexpr size_t stream_head_bytes(int batch, int arith) {
 // Items of the MFMA path that each wavefront of a workgroup takes (contiguous runs).
 __host__ __device__ __forceinline__ int mfma_items_per_wave(int nitems, int waves) { return (nitems + waves - 1) / waves; }
 
-// ARITH: 0 = matmul-free (dot2 on the VALU), 1 = MFMA with 16-bit operands, 2 = MFMA with one-bit fp4 weights
-// and fp8 pieces of the input (batch <= 4).
+// ARITH: 1 = MFMA with 16-bit operands, 2 = MFMA with one-bit fp4 weights and fp8 pieces of the input (batch <= 4).
 template <int DT, int BATCH, int ARITH, int THREADS, bool SINGLE>
 __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __restrict__ stages, int nstages,
                                                                      int nphases, const int* __restrict__ seg_index,
@@ -117,7 +114,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
     constexpr int kWaves = THREADS / kWave;
     constexpr int kRowBlock = row_block(BATCH);
     extern __shared__ uint4 lds_raw[];
-    constexpr bool MFMA = ARITH != 0;
+    static_assert(ARITH == 1 || ARITH == 2, "unknown arithmetic");
     constexpr bool kQ8 = ARITH == 2;
     constexpr bool kPow2Mfma = ARITH == 1 && DT == 0;           // fp16 MFMA path: single-bit operands, pair-major x
     constexpr bool kTotals = kPow2Mfma || kQ8;                  // signed sum = (sum of x) - 2 (sum of b x)
@@ -181,7 +178,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
             uint4 wnext = make_uint4(0, 0, 0, 0);
             if constexpr (kQ8) {
                 // nothing: see the loop (registers are scarcer than the head start is worth)
-            } else if constexpr (MFMA) {
+            } else {
                 // wavefront w starts with item w of the first row block: 16 rows x 4 units, lane (row l & 15,
                 // unit l >> 4)
                 const int ng0 = (chunk_units + 3) >> 2;
@@ -190,9 +187,6 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                 const int u0 = 4 * (item0 % ng0) + ((tid & 63) >> 4);
                 wnext = load_unit(bv, min(seg.row_begin + 16 * (item0 / ng0) + (tid & 15), st.rows - 1), u0,
                                   item0 < ((nr0 + 15) >> 4) * ng0 && u0 < chunk_units);
-            } else {
-                const int nr0 = min(seg.row_end - seg.row_begin, kRowBlock);
-                wnext = load_unit(bv, seg.row_begin + tid / chunk_units, tid % chunk_units, tid < nr0 * chunk_units);
             }
 
             if ((st.dep >= 0 || st.dep2 >= 0) && !aborted) {
@@ -332,7 +326,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                             if (it + 1 < it_end) step(wa1, wb1);
                             if (it_begin < it_end) flush();              // + sum of x at the end
                             if (ph == 0 && sg == seg_begin) NQ_MARK(14);
-                        } else if constexpr (MFMA) {
+                        } else {
                             // Items = (16-row group, 4-unit group), unit group fastest; every wavefront takes a
                             // contiguous run of items, so it mostly stays on one row group and adds its
                             // accumulator to the row sums only when the row group changes.
@@ -379,73 +373,6 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                                     for (int v = 0; v < 4; ++v)
                                         if (rg_run + 4 * g + v < nr) atomicAdd(&racc[(rg_run + 4 * g + v) * BATCH + r16], sum[v]);
                                 }
-                            }
-                        } else {
-                            const int total = nr * cu_n;
-                            // Lane t takes the (row, unit) pairs t, t + T, t + 2T, ... of the block (row-major), so
-                            // the lanes of a wavefront hold consecutive units of one to a few rows.  Two fetches
-                            // are kept in flight ahead of the arithmetic.  Row sums: lanes of the same row are
-                            // summed across the wavefront first and one lane adds the total to the row
-                            // accumulator -- 64 lanes adding to one LDS address serialise and cost a third of the
-                            // loop otherwise.  Every lane of a wavefront takes every trip (cross-lane sums).
-                            const int lane = tid & 63;
-                            // 0: per-lane adds (a wavefront spans many rows); 1: cu_n is 16, 32 or a multiple of 64,
-                            // rows coincide with aligned lane groups; 2: rows start anywhere in the wavefront
-                            const int sum_group = (cu_n & 63) == 0 ? 64 : cu_n;
-                            const int sum_mode = cu_n < 16 ? 0 : (sum_group == 16 || sum_group == 32 || sum_group == 64) ? 1 : 2;
-                            // Three fetch registers in rotation (trip k uses A, k+1 uses B, k+2 uses C, each
-                            // refilled for three trips later right after its use): nothing in flight is ever
-                            // copied, so the wait before a unit's arithmetic leaves the two younger fetches out.
-                            const int srow = kStreamThreads / cu_n, scu = kStreamThreads % cu_n;
-                            const int srow3 = 3 * kStreamThreads / cu_n, scu3 = 3 * kStreamThreads % cu_n;
-                            int row_a = tid / cu_n, cu_a = tid % cu_n;
-                            int row_b = row_a + srow, cu_b = cu_a + scu;
-                            if (cu_b >= cu_n) { cu_b -= cu_n; ++row_b; }
-                            int row_c = row_b + srow, cu_c = cu_b + scu;
-                            if (cu_c >= cu_n) { cu_c -= cu_n; ++row_c; }
-                            uint4 wa = wnext;                        // first block, chunk 0: fetched before the wait
-                            if (rb != seg.row_begin || c0 != 0) wa = load_unit(bv, rb + row_a, c0 + cu_a, tid < total);
-                            uint4 wb = load_unit(bv, rb + row_b, c0 + cu_b, tid + kStreamThreads < total);
-                            uint4 wc = load_unit(bv, rb + row_c, c0 + cu_c, tid + 2 * kStreamThreads < total);
-                            auto step = [&](uint4& w, int& row_l, int& cu, int f) {
-                                const bool valid = f < total;
-                                float part[BATCH];
-                                trim_unit(bv, w, c0 + cu);
-                                UnitDot<DT, BATCH>::run(w, xs, xsum, upad, valid ? cu : 0, part);
-                                const int row_now = row_l;
-                                // refill this register for three trips later
-                                row_l += srow3; cu += scu3;
-                                if (cu >= cu_n) { cu -= cu_n; ++row_l; }
-                                w = load_unit(bv, rb + row_l, c0 + cu, f + 3 * kStreamThreads < total);
-                                if (sum_mode == 1) {
-                                    // the group's total arrives in its last 16 lanes; the first of them adds it
-#pragma unroll
-                                    for (int b = 0; b < BATCH; ++b) {
-                                        const float tot = group_sum_tail(valid ? part[b] : 0.f, sum_group);
-                                        if (valid && (lane & (sum_group - 1)) == sum_group - 16) atomicAdd(&racc[row_now * BATCH + b], tot);
-                                    }
-                                } else if (sum_mode == 2) {
-                                    const int r_lo = __builtin_amdgcn_readfirstlane(row_now);
-                                    const int r_hi = (f - lane + 63 < total) ? __builtin_amdgcn_readlane(row_now, 63) : nr - 1;
-                                    for (int r = r_lo; r <= r_hi; ++r) {
-#pragma unroll
-                                        for (int b = 0; b < BATCH; ++b) {
-                                            const float tot = group_sum_tail((valid && row_now == r) ? part[b] : 0.f, 64);
-                                            if (lane == 63) atomicAdd(&racc[r * BATCH + b], tot);
-                                        }
-                                    }
-                                } else if (valid) {
-#pragma unroll
-                                    for (int b = 0; b < BATCH; ++b) atomicAdd(&racc[row_now * BATCH + b], part[b]);
-                                }
-                            };
-#pragma unroll 1
-                            for (int f = tid; f - lane < total; f += 3 * kStreamThreads) {   // wave-uniform trip counts
-                                step(wa, row_a, cu_a, f);
-                                if (f + kStreamThreads - lane >= total) break;
-                                step(wb, row_b, cu_b, f + kStreamThreads);
-                                if (f + 2 * kStreamThreads - lane >= total) break;
-                                step(wc, row_c, cu_c, f + 2 * kStreamThreads);
                             }
                         }
                         }
