@@ -109,6 +109,7 @@ typedef struct nq_linear {
     int y_from;             /* -1: addend (if any) is an external input */
     int out_f32;
     const void* bias;       /* [m] of the list's dtype, added after s_out (before addend); may be NULL */
+    int tiled;              /* vt_bits and u_bits are in the tile order of nq_tile_words (16-byte aligned) */
 } nq_linear;
 
 /* Launch geometry of a built run list; filled by nq_runlist_build, passed back to nq_runlist_run. */
@@ -163,6 +164,16 @@ int nq_gemm_nanoquant_bias(const void* x, const uint32_t* vt_tiles, const uint32
  * ("lsb_first", modules/linear.py:298) to the kernel format ("half2", modules/linear.py:171-172)
  * without the dense round trip of utils/load_utils.py:269-293.  order ids: nq_word_order. */
 int nq_repack_words(const uint32_t* src, uint32_t* dst, size_t nwords, int src_order, int dst_order, void* stream);
+
+/* Tile order of the packed words for run lists (no counterpart in the reference, whose kernels read the row-major
+ * words of kernel/utils.py:51-113 directly): 16-byte units indexed [row/32][unit/4][(row/16)&1][unit&3][row&15],
+ * rows padded to a multiple of 32 and units (4 words) to a multiple of 4 with zero words.  The 64 units a wavefront
+ * fetches for one MFMA operand are then 1 KiB contiguous instead of 16 pieces of 64 bytes, worth 15-25 % of read
+ * bandwidth in long run lists.  nq_tiled_words: 32-bit words of the tiled buffer.  nq_tile_words: row-major
+ * [rows, words] -> tile order, or back with inverse != 0; src and dst must differ; the tiled side must be 16-byte
+ * aligned. */
+size_t nq_tiled_words(int rows, int words);
+int nq_tile_words(const uint32_t* src, uint32_t* dst, int rows, int words, int inverse, void* stream);
 
 /* Plain device copy kernel of known traffic (bytes read + bytes written); used to calibrate the
  * memory counters of a profiler.  bytes must be a multiple of 16. */

@@ -199,15 +199,25 @@ class LinearStack:
         return [torch.randn(batch, lin["n"], device=self.device, generator=gen).to(self.dtype) for lin in self.layers[0]]
 
     # -- decode ----------------------------------------------------------------------------------
-    def make_runlist_step(self, batch: int, xs, per_layer: bool):
+    def make_runlist_step(self, batch: int, xs, per_layer: bool, tiled: bool = True):
+        """tiled: hand the words over in the run list's tile order (packing.tile_words; permuted once, here)."""
         from .runlist import DecodeRunList
+        if tiled:
+            for layer in self.layers:
+                for lin in layer:
+                    if "vt_tiled" not in lin:
+                        lin["vt_tiled"] = self._packing.tile_words(lin["vt"])
+                        lin["u_tiled"] = self._packing.tile_words(lin["u"])
         lists = []
         groups = [[layer] for layer in self.layers] if per_layer else [self.layers]
         for group in groups:
             rl = DecodeRunList(batch, self.dtype, self.device)
             for layer in group:
                 for lin, x in zip(layer, xs):
-                    rl.add(x, lin["s_in"], lin["vt"], lin["s_mid"], lin["u"], lin["s_out"])
+                    if tiled:
+                        rl.add(x, lin["s_in"], lin["vt_tiled"], lin["s_mid"], lin["u_tiled"], lin["s_out"], tiled=True)
+                    else:
+                        rl.add(x, lin["s_in"], lin["vt"], lin["s_mid"], lin["u"], lin["s_out"])
             rl.build()
             lists.append(rl)
 
@@ -265,9 +275,9 @@ def run_config(stack: LinearStack, args, bs: int, pt: int, new: int, power: bool
     xs = stack.inputs(bs, args.seed + 1)
     kind = args.quant_kernel_type
     if kind == "runlist":
-        step = stack.make_runlist_step(bs, xs, per_layer=False)
+        step = stack.make_runlist_step(bs, xs, per_layer=False, tiled=args.tiled)
     elif kind == "runlist-per-layer":
-        step = stack.make_runlist_step(bs, xs, per_layer=True)
+        step = stack.make_runlist_step(bs, xs, per_layer=True, tiled=args.tiled)
     else:
         step = stack.make_op_step(xs)
     graph = None
@@ -349,6 +359,8 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--gpu_id", type=int, default=0)
     p.add_argument("--no_graph", dest="graph", action="store_false", help="launch from Python instead of replaying a graph")
     p.add_argument("--skip_prefill", action="store_true")
+    p.add_argument("--row_major", dest="tiled", action="store_false",
+                   help="run lists read the reference's row-major words instead of the tile order")
     p.add_argument("--profile_energy", action="store_true")
     return p
 

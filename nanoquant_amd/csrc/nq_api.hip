@@ -3,6 +3,7 @@
 #include "../../include/nq_gfx950.h"
 #include "nq_kernels.h"
 
+#include <algorithm>
 #include <vector>
 
 namespace {
@@ -38,7 +39,7 @@ const char* nq_status_string(int status) {
 
 int nq_last_hip_error(void) { return g_last_hip_error; }
 
-int nq_abi_version(void) { return 2; }
+int nq_abi_version(void) { return 3; }
 
 int nq_device_query(int attr, int* value) {
     if (!value) return NQ_ERR_NULL;
@@ -170,7 +171,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         const nq_linear& l = linears[i];
         nq::RunStage a{};
         a.bits = l.vt_bits; a.in = l.x; a.s_col = (const uint16_t*)l.s_in; a.s_row = (const uint16_t*)l.s_mid;
-        a.out = l.h; a.addend = nullptr;
+        a.out = l.h; a.addend = nullptr; a.tiled = l.tiled ? 1 : 0;
         a.rows = l.r; a.K = l.n; a.words = (l.n + 31) / 32; a.units = (a.words + 3) / 4;
         a.in_stride = l.n; a.out_stride = l.r; a.in_f32 = 0; a.out_f32 = 1;
         a.dep = l.x_from >= 0 ? 2 * l.x_from + 1 : -1;
@@ -186,7 +187,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
 
         nq::RunStage b{};
         b.bits = l.u_bits; b.in = l.h; b.s_col = nullptr; b.s_row = (const uint16_t*)l.s_out;
-        b.out = l.y; b.addend = l.addend; b.bias = (const uint16_t*)l.bias;
+        b.out = l.y; b.addend = l.addend; b.bias = (const uint16_t*)l.bias; b.tiled = l.tiled ? 1 : 0;
         b.rows = l.m; b.K = l.r; b.words = (l.r + 31) / 32; b.units = (b.words + 3) / 4;
         b.in_stride = l.r; b.out_stride = l.m; b.in_f32 = 1; b.out_f32 = l.out_f32 ? 1 : 0;
         b.dep = 2 * i;
@@ -197,7 +198,10 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         b.phase = a.phase + 1;
         if (b.dep2 >= 0 && table[b.dep2].phase + 1 > b.phase) b.phase = table[b.dep2].phase + 1;
         // the kernel addresses the packed words of a stage with 32-bit byte offsets
-        if ((size_t)a.rows * a.words * 4 >= 0x7FFFFFF0ull || (size_t)b.rows * b.words * 4 >= 0x7FFFFFF0ull) return NQ_ERR_SHAPE;
+        const size_t bytes_a = l.tiled ? nq::tiled_word_count(a.rows, a.words) * 4 : (size_t)a.rows * a.words * 4;
+        const size_t bytes_b = l.tiled ? nq::tiled_word_count(b.rows, b.words) * 4 : (size_t)b.rows * b.words * 4;
+        if (bytes_a >= 0x7FFFFFF0ull || bytes_b >= 0x7FFFFFF0ull) return NQ_ERR_SHAPE;
+        if (l.tiled && (((uintptr_t)l.vt_bits | (uintptr_t)l.u_bits) & 15u)) return NQ_ERR_ALIGN;
         table[2 * i + 1] = b;
         if (a.units > max_units) max_units = a.units;
         if (b.units > max_units) max_units = b.units;
@@ -232,6 +236,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
             while (k + 1 < ids.size() && prefix[k + 1] <= c) ++k;
             if (c >= total) { k = ids.size() - 1; row = table[ids[k]].rows; return; }
             row = (int)((c - prefix[k]) / table[ids[k]].units);
+            if (table[ids[k]].tiled) row &= ~31;      // tile order: cut between 32-row tiles
         };
         if (ids.size() * 2 <= (size_t)nwg) {
             // Few stages, many workgroups: give every stage whole workgroups, so that no workgroup stages
@@ -288,9 +293,16 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
             int w = 0;
             for (size_t k = 0; k < ids.size(); ++k) {
                 const int rows = table[ids[k]].rows;
+                // tile order: cut between 32-row tiles, so that every wave-load is one contiguous KiB
+                const bool tiled = table[ids[k]].tiled != 0;
+                const int ntile = (rows + 31) / 32;
                 for (int j = 0; j < share[k]; ++j, ++w) {
-                    const int rb = (int)((long long)rows * j / share[k]);
-                    const int re = (int)((long long)rows * (j + 1) / share[k]);
+                    int rb = (int)((long long)rows * j / share[k]);
+                    int re = (int)((long long)rows * (j + 1) / share[k]);
+                    if (tiled) {
+                        rb = (int)std::min<long long>(rows, 32LL * ((long long)ntile * j / share[k]));
+                        re = (int)std::min<long long>(rows, 32LL * ((long long)ntile * (j + 1) / share[k]));
+                    }
                     if (re > rb) {
                         slice[ph][(size_t)w].push_back(nq::RunSegment{ids[k], rb, re, 0});
                         table[ids[k]].seg_count += 1;
@@ -413,6 +425,20 @@ int nq_gemm_nanoquant_bias(const void* x, const uint32_t* vt_tiles, const uint32
     int st = nq_gemm_onebit(x, vt_tiles, s_in, s_mid, h, scratch, scratch_bytes, tokens, n, r, dtype, stream);
     if (st != NQ_OK) return st;
     return nq_gemm_onebit_bias(h, u_tiles, nullptr, s_out, bias, y, scratch, scratch_bytes, tokens, r, m, dtype, stream);
+}
+
+size_t nq_tiled_words(int rows, int words) {
+    if (rows <= 0 || words <= 0) return 0;
+    return nq::tiled_word_count(rows, words);
+}
+
+int nq_tile_words(const uint32_t* src, uint32_t* dst, int rows, int words, int inverse, void* stream) {
+    if (rows < 0 || words < 0) return NQ_ERR_SHAPE;
+    if (rows == 0 || words == 0) return NQ_OK;
+    if (!src || !dst) return NQ_ERR_NULL;
+    if (src == dst) return NQ_ERR_SHAPE;             // a permutation across rows: not in place
+    if (((uintptr_t)(inverse ? src : dst)) & 15u) return NQ_ERR_ALIGN;
+    return hip_status(nq::tile_words(src, dst, rows, words, inverse ? 1 : 0, (hipStream_t)stream));
 }
 
 int nq_repack_words(const uint32_t* src, uint32_t* dst, size_t nwords, int src_order, int dst_order, void* stream) {

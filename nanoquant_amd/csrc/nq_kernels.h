@@ -33,7 +33,7 @@ struct RunStage {
     int in_coherent;        // fp32 input written by another stage of the same launch
     int heavy_release;      // 16-bit output read by a later stage: full device-scope release on completion
     int heavy_acquire;      // 16-bit input written by an earlier stage: full device-scope acquire after the wait
-    int pad_;
+    int tiled;              // `bits` is in the tile order of tile_words() instead of row-major
 };
 // One workgroup's share of one stage: rows [row_begin, row_end).
 struct RunSegment {
@@ -58,5 +58,7 @@ hipError_t gemm_onebit(int dtype, const void* x, const uint32_t* tiles, const vo
 hipError_t stream_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);
 hipError_t repack_words(const uint32_t* src, uint32_t* dst, size_t nwords, int src_order, int dst_order,
                         hipStream_t stream);
+size_t tiled_word_count(int rows, int words);
+hipError_t tile_words(const uint32_t* src, uint32_t* dst, int rows, int words, int inverse, hipStream_t stream);
 
 }  // namespace nq

@@ -63,20 +63,32 @@ constexpr int kStreamLdsMax = 144 * 1024;      // staged activations + row accum
 struct BitsView {
     __amdgpu_buffer_rsrc_t rsrc;
     int words;      // 32-bit words per row
-    int ragged;     // words % 4 != 0: the last unit of a row holds fewer than 4 words
+    int ragged;     // row-major and words % 4 != 0: the last unit of a row holds fewer than 4 words
+    int groups;     // > 0: tile order (see tile_kernel), value = 4-unit groups per row; 0: row-major
 };
 
 __device__ __forceinline__ BitsView bits_view(const RunStage& st) {
     BitsView v;
-    v.rsrc = raw_buffer(st.bits, (uint32_t)((size_t)st.rows * st.words * sizeof(uint32_t)));
     v.words = st.words;
-    v.ragged = (st.words & 3) != 0;
+    v.groups = st.tiled ? (st.words + 15) >> 4 : 0;
+    const size_t bytes = st.tiled ? (size_t)((st.rows + 31) >> 5) * v.groups * 2048 : (size_t)st.rows * st.words * sizeof(uint32_t);
+    v.rsrc = raw_buffer(st.bits, (uint32_t)bytes);
+    v.ragged = !st.tiled && (st.words & 3) != 0;
     return v;
 }
 
+// In tile order the 64 units of a wave-load (16 rows x 4 units) are 1 KiB contiguous and every line is read once:
+// streamed with the non-temporal hint (6.5 TB/s in a read-only probe against 5.9 row-major with default policy).
 __device__ __forceinline__ uint4 load_unit(const BitsView& v, int row, int unit, bool live) {
-    const uint32_t off = live ? ((uint32_t)row * (uint32_t)v.words + 4u * (uint32_t)unit) * 4u : kPastEnd;
-    const u32x4_t w = __builtin_amdgcn_raw_buffer_load_b128(v.rsrc, off, 0, NQ_BITS_AUX);
+    u32x4_t w;
+    if (v.groups) {
+        const uint32_t r = (uint32_t)row, u = (uint32_t)unit;
+        const uint32_t idx = ((((r >> 5) * (uint32_t)v.groups + (u >> 2)) * 2u + ((r >> 4) & 1u)) * 4u + (u & 3u)) * 16u + (r & 15u);
+        w = __builtin_amdgcn_raw_buffer_load_b128(v.rsrc, live ? idx * 16u : kPastEnd, 0, 2 /* nt */);
+    } else {
+        const uint32_t off = live ? ((uint32_t)row * (uint32_t)v.words + 4u * (uint32_t)unit) * 4u : kPastEnd;
+        w = __builtin_amdgcn_raw_buffer_load_b128(v.rsrc, off, 0, NQ_BITS_AUX);
+    }
     return make_uint4(w.x, w.y, w.z, w.w);
 }
 

@@ -45,4 +45,56 @@ hipError_t repack_words(const uint32_t* src, uint32_t* dst, size_t nwords, int s
     return hipGetLastError();
 }
 
+// Tile order of the run-list kernel: 16-byte units (4 words) indexed [row / 32][unit / 4][(row / 16) & 1][unit & 3]
+// [row & 15], rows padded to a multiple of 32 and units to a multiple of 4 with zero words.  The 64 units that
+// one wavefront fetches for an MFMA operand (16 rows x 4 units) are 1 KiB contiguous, the two row groups of a
+// 32-row pair adjacent.  One thread per destination (tile: tiled, else row-major) unit.
+__host__ __device__ __forceinline__ size_t tiled_unit_index(int row, int unit, int groups) {
+    return (((((size_t)(row >> 5) * groups + (unit >> 2)) * 2 + ((row >> 4) & 1)) * 4 + (unit & 3)) * 16) + (row & 15);
+}
+
+size_t tiled_word_count(int rows, int words) {
+    const size_t groups = ((size_t)words + 15) / 16;
+    return (((size_t)rows + 31) / 32) * groups * 128 * 4;
+}
+
+__global__ __launch_bounds__(256) void tile_kernel(const uint32_t* src, uint32_t* dst, int rows, int words, int groups,
+                                                   int inverse, size_t nunits) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nunits; i += stride) {
+        if (!inverse) {
+            // i = tiled unit index -> (row, unit)
+            const int r16 = (int)(i & 15), g = (int)((i >> 4) & 3), half = (int)((i >> 6) & 1);
+            const size_t t = i >> 7;
+            const int ub = (int)(t % (size_t)groups), rp = (int)(t / (size_t)groups);
+            const int row = 32 * rp + 16 * half + r16, unit = 4 * ub + g;
+            uint32_t w[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int c = 4 * unit + k;
+                w[k] = (row < rows && c < words) ? src[(size_t)row * words + c] : 0u;
+            }
+            ((uint4*)dst)[i] = make_uint4(w[0], w[1], w[2], w[3]);
+        } else {
+            // i = row-major unit index over [rows][ceil(words / 4)]
+            const int upr = (words + 3) / 4;
+            const int row = (int)(i / (size_t)upr), unit = (int)(i % (size_t)upr);
+            const uint4 v = ((const uint4*)src)[tiled_unit_index(row, unit, groups)];
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+            for (int k = 0; k < 4; ++k)
+                if (4 * unit + k < words) dst[(size_t)row * words + 4 * unit + k] = w[k];
+        }
+    }
+}
+
+hipError_t tile_words(const uint32_t* src, uint32_t* dst, int rows, int words, int inverse, hipStream_t stream) {
+    if (rows <= 0 || words <= 0) return hipSuccess;
+    const int groups = (words + 15) / 16;
+    const size_t nunits = inverse ? (size_t)rows * ((words + 3) / 4) : tiled_word_count(rows, words) / 4;
+    size_t blocks = (nunits + 255) / 256;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    hipLaunchKernelGGL(tile_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, src, dst, rows, words, groups, inverse, nunits);
+    return hipGetLastError();
+}
+
 }  // namespace nq

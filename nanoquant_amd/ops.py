@@ -350,6 +350,21 @@ def repack_words_device(packed: torch.Tensor, src: str, dst: str) -> torch.Tenso
     return out
 
 
+def tile_words_device(packed: torch.Tensor, inverse: bool, shape=None) -> torch.Tensor:
+    """Device pass of packing.tile_words / untile_words."""
+    lib = _lib.lib()
+    if not inverse:
+        rows, words = packed.shape
+        out = torch.empty(int(lib.nq_tiled_words(rows, words)), dtype=torch.int32, device=packed.device)
+    else:
+        rows, words = shape
+        out = torch.empty((rows, words), dtype=torch.int32, device=packed.device)
+    if rows > 0 and words > 0:
+        with torch.cuda.device(packed.device):
+            _lib.check(lib.nq_tile_words(_ptr(packed), _ptr(out), rows, words, int(inverse), _stream(packed.device)))
+    return out
+
+
 def get_kernel_function(namespace: str, dtype: torch.dtype, kernel_type: str):
     """Operator lookup with the reference's naming rule (src/nanoquant/kernel/utils.py:33-48)."""
     mid = "_dyn" if kernel_type != "fixed" else ""

@@ -100,6 +100,46 @@ def repack_words(packed: torch.Tensor, src: str = "lsb_first", dst: str = "half2
 
 
 # ---------------------------------------------------------------------------------------------
+# tile order of the decode run list
+# ---------------------------------------------------------------------------------------------
+def tile_words(packed: torch.Tensor) -> torch.Tensor:
+    """Row-major words [rows, words] ("half2" order) -> flat int32 buffer in the tile order of the run-list kernel:
+    16-byte units (4 words) indexed [row // 32][unit // 4][(row // 16) & 1][unit & 3][row & 15], rows padded to a
+    multiple of 32 and units to a multiple of 4 with zero words.  The 64 units that a wavefront fetches for one MFMA
+    operand (16 rows x 4 units) become 1 KiB contiguous.  The reference has no such layout (its kernels read the
+    row-major words, kernel/utils.py:51-113); this is a fixed permutation done once at load time."""
+    if packed.dtype != torch.int32 or packed.dim() != 2:
+        raise TypeError("packed words must be a 2-D int32 tensor")
+    rows, words = packed.shape
+    if packed.is_cuda:
+        from . import ops
+        return ops.tile_words_device(packed.contiguous(), inverse=False)
+    groups = (words + 15) // 16
+    r32 = (rows + 31) // 32 * 32
+    pad = torch.zeros((r32, groups * 16), dtype=torch.int32)
+    pad[:rows, :words] = packed
+    # [rp, half, r16, ub, g, word] -> [rp, ub, half, g, r16, word]
+    t = pad.view(r32 // 32, 2, 16, groups, 4, 4).permute(0, 3, 1, 4, 2, 5)
+    return t.contiguous().view(-1)
+
+
+def untile_words(tiled: torch.Tensor, shape: Tuple[int, int]) -> torch.Tensor:
+    """Inverse of tile_words for a matrix of `shape` = (rows, words)."""
+    rows, words = int(shape[0]), int(shape[1])
+    if tiled.dtype != torch.int32 or tiled.dim() != 1:
+        raise TypeError("tiled words must be a flat int32 tensor")
+    groups = (words + 15) // 16
+    r32 = (rows + 31) // 32 * 32
+    if tiled.numel() != r32 * groups * 16:
+        raise ValueError(f"expected {r32 * groups * 16} words for shape {(rows, words)}, got {tiled.numel()}")
+    if tiled.is_cuda:
+        from . import ops
+        return ops.tile_words_device(tiled.contiguous(), inverse=True, shape=(rows, words))
+    t = tiled.view(r32 // 32, groups, 2, 4, 16, 4).permute(0, 2, 4, 1, 3, 5)
+    return t.contiguous().view(r32, groups * 16)[:rows, :words].contiguous()
+
+
+# ---------------------------------------------------------------------------------------------
 # prefill (MFMA) layout
 # ---------------------------------------------------------------------------------------------
 def pack_gemm_tiles(weight: torch.Tensor) -> torch.Tensor:

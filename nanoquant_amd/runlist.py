@@ -24,7 +24,7 @@ class NqLinear(ctypes.Structure):
         ("addend", ctypes.c_void_p),
         ("n", ctypes.c_int), ("r", ctypes.c_int), ("m", ctypes.c_int),
         ("x_from", ctypes.c_int), ("y_from", ctypes.c_int), ("out_f32", ctypes.c_int),
-        ("bias", ctypes.c_void_p),
+        ("bias", ctypes.c_void_p), ("tiled", ctypes.c_int),
     ]
 
 
@@ -55,19 +55,29 @@ class DecodeRunList:
     def add(self, x: torch.Tensor, scale_pre: torch.Tensor, V_int8: torch.Tensor, scale_mid: Optional[torch.Tensor],
             U_int8: torch.Tensor, scale_post: torch.Tensor, y: Optional[torch.Tensor] = None,
             x_from: int = -1, addend: Optional[torch.Tensor] = None, y_from: int = -1,
-            out_f32: bool = False, bias: Optional[torch.Tensor] = None) -> int:
+            out_f32: bool = False, bias: Optional[torch.Tensor] = None, tiled: bool = False) -> int:
         """Append one linear (operands as `NanoQuantLinear` holds them after `_prepare_kernel('gemv')`:
         V_int8 [r, n/32] first stage, U_int8 [m, r/32] second stage).  Returns its index; `y` is
         allocated when not given and is available as `outputs[index]`.  `bias` [m] is added after `scale_post`."""
         n = x.shape[-1]
-        r, m = V_int8.shape[0], U_int8.shape[0]
+        if tiled:
+            # tile order (packing.tile_words): flat buffers, the rank comes from scale_mid / the word count
+            if scale_mid is None:
+                raise RuntimeError("tiled factors need scale_mid (its length is the rank)")
+            r, m = scale_mid.numel(), scale_post.numel()
+        else:
+            r, m = V_int8.shape[0], U_int8.shape[0]
         for name, t, dt in (("x", x, self.dtype), ("scale_pre", scale_pre, self.dtype), ("scale_post", scale_post, self.dtype),
                             ("V_int8", V_int8, torch.int32), ("U_int8", U_int8, torch.int32)):
             if not t.is_cuda or not t.is_contiguous() or t.dtype != dt:
                 raise RuntimeError(f"{name} must be a contiguous {dt} tensor on the GPU")
         if x.numel() != self.batch * n:
             raise RuntimeError(f"x must hold {self.batch} rows of {n}")
-        if V_int8.shape[1] != (n + 31) // 32 or U_int8.shape[1] != (r + 31) // 32:
+        if tiled:
+            lib = _lib.lib()
+            if V_int8.numel() != lib.nq_tiled_words(r, (n + 31) // 32) or U_int8.numel() != lib.nq_tiled_words(m, (r + 31) // 32):
+                raise RuntimeError("tiled factor sizes do not match the shapes")
+        elif V_int8.shape[1] != (n + 31) // 32 or U_int8.shape[1] != (r + 31) // 32:
             raise RuntimeError("packed factor shapes do not match x / each other")
         if scale_pre.numel() != n or scale_post.numel() != m or (scale_mid is not None and scale_mid.numel() != r):
             raise RuntimeError("scale size mismatch")
@@ -79,7 +89,7 @@ class DecodeRunList:
         self._keep += [x, scale_pre, V_int8, scale_mid, U_int8, scale_post, y, h, addend, bias]
         self._entries.append(dict(x=x, s_in=scale_pre, vt=V_int8, s_mid=scale_mid, u=U_int8, s_out=scale_post, h=h, y=y,
                                   addend=addend, n=n, r=r, m=m, x_from=x_from, y_from=y_from, out_f32=int(out_f32),
-                                  bias=bias))
+                                  bias=bias, tiled=int(tiled)))
         self._workspace = None
         return len(self._entries) - 1
 
@@ -96,7 +106,7 @@ class DecodeRunList:
         for i, e in enumerate(self._entries):
             arr[i] = NqLinear(p(e["x"]), p(e["s_in"]), p(e["vt"]), p(e["s_mid"]), p(e["u"]), p(e["s_out"]), p(e["h"]),
                               p(e["y"]), p(e["addend"]), e["n"], e["r"], e["m"], e["x_from"], e["y_from"], e["out_f32"],
-                              p(e["bias"]))
+                              p(e["bias"]), e["tiled"])
         lib = _lib.lib()
         nbytes = int(lib.nq_runlist_workspace_bytes(arr, n))
         ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device)

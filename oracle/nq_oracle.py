@@ -297,3 +297,20 @@ def staged_input(v, pieces: int = 3) -> np.ndarray:
         out[b] = fp8_pieces(v[b] * s, pieces).sum(axis=0) / s
     return out
 
+
+# ---- tile order of the gfx950 run-list kernel ---------------------------------------------------------
+def tile_words(packed: np.ndarray) -> np.ndarray:
+    """Row-major words [rows, words] -> flat tile order, by the index formula itself (no counterpart in the
+    reference): 16-byte unit (row, unit) goes to unit index
+    ((((row // 32) * G + unit // 4) * 2 + (row // 16) % 2) * 4 + unit % 4) * 16 + row % 16, G = ceil(words / 16);
+    padding rows / words are zero."""
+    rows, words = packed.shape
+    groups = (words + 15) // 16
+    out = np.zeros(((rows + 31) // 32) * groups * 128 * 4, dtype=packed.dtype)
+    for row in range(rows):
+        for c in range(words):
+            unit = c // 4
+            idx = ((((row // 32) * groups + unit // 4) * 2 + (row // 16) % 2) * 4 + unit % 4) * 16 + row % 16
+            out[idx * 4 + c % 4] = packed[row, c]
+    return out
+

@@ -204,3 +204,53 @@ def test_bf16_batches_on_the_mfma_path(dev, batch):
     assert rl.status() == 0
     for y, ref in zip(ys, refs):
         assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < 1e-2
+
+
+@pytest.mark.parametrize("rows,words", [(33, 17), (70, 47), (4096, 128), (5, 94)])
+def test_tile_order_on_the_device(dev, rows, words):
+    a = np.random.default_rng(rows + words).integers(-2 ** 31, 2 ** 31 - 1, (rows, words), dtype=np.int64).astype(np.int32)
+    t = packing.tile_words(torch.from_numpy(a).to(dev))
+    torch.cuda.synchronize()
+    assert np.array_equal(t.cpu().numpy(), packing.tile_words(torch.from_numpy(a)).numpy())
+    back = packing.untile_words(t, (rows, words))
+    torch.cuda.synchronize()
+    assert np.array_equal(back.cpu().numpy(), a)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("batch", [1, 2, 4, 16])
+def test_tiled_factors_give_the_same_layer(dev, batch, dtype):
+    # ragged shapes (words 47 / 13, rows not a multiple of 32) and a shape with many 32-row tiles per workgroup
+    shapes = [(600, 1504, 416), (2048, 1024, 512), (96, 160, 64)]
+    rl_t, rl_r = DecodeRunList(batch, dtype, dev), DecodeRunList(batch, dtype, dev)
+    refs = []
+    for i, (m, n, r) in enumerate(shapes):
+        vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, 400 + i)
+        x = oracle.synth_x(batch, n, 410 + i)
+        to = lambda a: torch.from_numpy(a).to(dev).to(dtype)
+        f64 = lambda t: t.float().cpu().numpy().astype(np.float64)
+        xd, sc = to(x), (to(s_in), to(s_mid), to(s_out))
+        vb = packing.binary_packer(torch.from_numpy(vt), "half2").to(dev)
+        ub = packing.binary_packer(torch.from_numpy(u), "half2").to(dev)
+        rl_r.add(xd, sc[0], vb, sc[1], ub, sc[2])
+        rl_t.add(xd, sc[0], packing.tile_words(vb), sc[1], packing.tile_words(ub), sc[2], tiled=True)
+        refs.append(oracle.layer_forward(f64(xd), vt, u, f64(sc[0]), f64(sc[1]), f64(sc[2]), dtype=np.float64))
+    print(f"tiled run list batch={batch} {dtype}", flush=True)
+    ys_t, ys_r = rl_t.run(), rl_r.run()
+    torch.cuda.synchronize()
+    assert rl_t.status() == 0 and rl_r.status() == 0
+    tol = 1e-2 if dtype == torch.bfloat16 else 2e-3
+    for (m, n, r), yt, yr, ref in zip(shapes, ys_t, ys_r, refs):
+        assert oracle.max_rel_err(yt.float().cpu().numpy(), ref) < (tol if r >= 256 else 1e-2), (m, n, r)
+        # same arithmetic, other slice boundaries: row sums differ by fp32 rounding at most
+        assert torch.allclose(yt.float(), yr.float(), rtol=4e-3 if dtype == torch.float16 else 2e-2,
+                              atol=2e-4 * float(yr.float().abs().max()))
+
+
+def test_tiled_factor_size_is_checked(dev):
+    m, n, r = 64, 128, 32
+    _, ops = _term(dev, m, n, r, seed=5)
+    x = torch.zeros(1, n, dtype=torch.float16, device=dev)
+    rl = DecodeRunList(1, torch.float16, dev)
+    with pytest.raises(RuntimeError):
+        rl.add(x, ops[0], ops[1].reshape(-1), ops[2], ops[3].reshape(-1), ops[4], tiled=True)   # row-major sizes

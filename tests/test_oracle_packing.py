@@ -163,3 +163,22 @@ def test_empty_inputs():
     z = np.ones((3, 0), dtype=np.int8)
     assert oracle.pack_rows(z, "half2").shape == (3, 0)
     assert packing.pack_binary_gemv(torch.from_numpy(z), "half2").shape == (3, 0)
+
+
+# ---- tile order of the run list -----------------------------------------------------------------------
+@pytest.mark.parametrize("rows,words", [(1, 1), (16, 4), (33, 17), (70, 47), (64, 16), (5, 94)])
+def test_tile_order_matches_the_index_formula_and_round_trips(rows, words):
+    import torch
+
+    from nanoquant_amd import packing
+    rng = np.random.default_rng(rows * 131 + words)
+    a = rng.integers(-2 ** 31, 2 ** 31 - 1, (rows, words), dtype=np.int64).astype(np.int32)
+    t = packing.tile_words(torch.from_numpy(a))
+    groups = (words + 15) // 16
+    assert t.numel() == (rows + 31) // 32 * groups * 512
+    assert np.array_equal(t.numpy(), oracle.tile_words(a))           # reshape/permute == per-element formula
+    assert np.array_equal(packing.untile_words(t, (rows, words)).numpy(), a)
+    # a wave-load (16 rows x 4 units of one 32-row tile) is 256 consecutive words
+    if rows >= 16 and words >= 16:
+        blk = t.numpy()[:256].reshape(4, 16, 4)                      # [unit, row, word]
+        assert np.array_equal(blk[2, 5], a[5, 8:12])
