@@ -213,6 +213,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
     }
 
     // ---- grid = what the device keeps resident; every workgroup gets an equal share of every phase ----
+    const int granule = nq::stream_row_granule(dtype, batch);
     int nwg = nq::stream_capacity(dtype, batch, max_units);
     if (nwg <= 0) return NQ_ERR_HIP;
     if (nwg > kMaxResidentWorkgroups) nwg = kMaxResidentWorkgroups;
@@ -236,7 +237,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
             while (k + 1 < ids.size() && prefix[k + 1] <= c) ++k;
             if (c >= total) { k = ids.size() - 1; row = table[ids[k]].rows; return; }
             row = (int)((c - prefix[k]) / table[ids[k]].units);
-            if (table[ids[k]].tiled) row &= ~31;      // tile order: cut between 32-row tiles
+            if (table[ids[k]].tiled) row &= ~(granule - 1);   // tile order: cut between the row groups of a wave-load
         };
         if (ids.size() * 2 <= (size_t)nwg) {
             // Few stages, many workgroups: give every stage whole workgroups, so that no workgroup stages
@@ -293,15 +294,15 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
             int w = 0;
             for (size_t k = 0; k < ids.size(); ++k) {
                 const int rows = table[ids[k]].rows;
-                // tile order: cut between 32-row tiles, so that every wave-load is one contiguous KiB
+                // tile order: cut between the row groups of a wave-load, so that each is one contiguous KiB
                 const bool tiled = table[ids[k]].tiled != 0;
-                const int ntile = (rows + 31) / 32;
+                const int ntile = (rows + granule - 1) / granule;
                 for (int j = 0; j < share[k]; ++j, ++w) {
                     int rb = (int)((long long)rows * j / share[k]);
                     int re = (int)((long long)rows * (j + 1) / share[k]);
                     if (tiled) {
-                        rb = (int)std::min<long long>(rows, 32LL * ((long long)ntile * j / share[k]));
-                        re = (int)std::min<long long>(rows, 32LL * ((long long)ntile * (j + 1) / share[k]));
+                        rb = (int)std::min<long long>(rows, (long long)granule * ((long long)ntile * j / share[k]));
+                        re = (int)std::min<long long>(rows, (long long)granule * ((long long)ntile * (j + 1) / share[k]));
                     }
                     if (re > rb) {
                         slice[ph][(size_t)w].push_back(nq::RunSegment{ids[k], rb, re, 0});

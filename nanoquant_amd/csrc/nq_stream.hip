@@ -615,6 +615,14 @@ int stream_capacity(int dtype, int batch, int max_units) {
     return 0;
 }
 
+// Rows that one wave-load spans: slices of tile-order stages are cut at multiples of it.
+int stream_row_granule(int dtype, int batch) {
+#define NQ_GRAN(D, B) (StreamKernel<D, B>::kArith == 2 ? 32 : 16)
+    NQ_STREAM_DISPATCH(NQ_GRAN)
+#undef NQ_GRAN
+    return 32;
+}
+
 hipError_t gemv_stream(int dtype, int batch, const RunStage* stages, int nstages, int nphases, const int* seg_index,
                        const RunSegment* segs, unsigned long long* counters, unsigned* status, int nwg, int max_units,
                        hipStream_t stream) {
