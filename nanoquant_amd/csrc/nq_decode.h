@@ -96,7 +96,7 @@ __device__ __forceinline__ void store_chunk(uint4* xs, int b, int i, int upad, i
     }
 }
 
-// Staging variants below: `xtot` (may be null) receives the sum over all staged units per batch row
+// Staging variants below: `xsum` (may be null) receives the per-unit sums, `xtot` (may be null) the sum over all staged units per batch row
 // (LDS float atomics; the caller zeroes it and puts a barrier before and after).
 
 // Coherent fp32 input (the intermediate h written by other workgroups of this launch): 16-byte
@@ -140,7 +140,7 @@ __device__ __forceinline__ void stage_units_coherent(uint4* xs, float* xsum, flo
                 xd[xs_dword<PM>(b, P, upad, cu)] = (uint32_t)r0 | ((uint32_t)r1 << 16);
                 xd[xs_dword<PM>(b, P + 1, upad, cu)] = (uint32_t)r2 | ((uint32_t)r3 << 16);
                 if ((q & 31) == 0) {
-                    xsum[b * upad + cu] = tot;
+                    if (xsum) xsum[b * upad + cu] = tot;
                     if (xtot) atomicAdd(&xtot[b], tot);
                 }
             }
@@ -207,7 +207,7 @@ __device__ __forceinline__ void stage_units_vector(uint4* xs, float* xsum, float
                 const int cu = q >> 4, i = q & 15;
                 store_chunk<PM>(xs, b, i, upad, cu, r);
                 if (i == 0) {
-                    xsum[b * upad + cu] = tot;
+                    if (xsum) xsum[b * upad + cu] = tot;
                     if (xtot) atomicAdd(&xtot[b], tot);
                 }
             }
@@ -252,7 +252,7 @@ __device__ __forceinline__ void stage_units_scalar(uint4* xs, float* xsum, float
             if (q < nchunks) {
                 store_chunk<PM>(xs, b, i, upad, cu, r);
                 if (i == 0) {
-                    xsum[b * upad + cu] = tot;
+                    if (xsum) xsum[b * upad + cu] = tot;
                     if (xtot) atomicAdd(&xtot[b], tot);
                 }
             }

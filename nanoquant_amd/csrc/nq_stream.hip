@@ -36,8 +36,9 @@ __device__ unsigned long long* g_nq_trace = nullptr;
 namespace nq {
 
 // Rows whose sums a workgroup keeps in LDS at a time (then: barrier, scale, store, barrier).  Few large
-// blocks at small batch; 16 KiB of row sums at most.
-__host__ __device__ constexpr int row_block(int batch) { return batch == 1 ? 1024 : batch == 2 ? 512 : batch == 4 ? 256 : 128; }
+// blocks at small batch; 16 KiB of row sums at most.  From batch 4 up 256 rows = 16 row groups = one per wavefront,
+// so a row sum is finished by one wavefront (LDS float atomics cost about 2.5 cycles per lane).
+__host__ __device__ constexpr int row_block(int batch) { return batch == 1 ? 1024 : batch == 2 ? 512 : 256; }
 // Same-address device-scope atomics serialise at the memory side (tens of ns each), so completion
 // counts are spread over kSubCounters addresses per stage and kExitSubs addresses for the exit count,
 // one 64-byte line each.
@@ -103,11 +104,11 @@ __device__ __forceinline__ void trim_unit(const BitsView& v, uint4& w, int unit)
     }
 }
 
-// Bytes of LDS in front of the staged input: row sums, the input totals, and the per-unit input sums (the fp4 x
-// fp8 path keeps the per-row maxima there instead).
+// Bytes of LDS in front of the staged input: row sums, the input totals [16] and the per-row maxima of the fp4 x
+// fp8 path [16].
 __host__ __device__ constexpr size_t stream_head_bytes(int batch, int arith) {
-    return arith == 2 ? (size_t)row_block(batch) * batch * sizeof(float) + 128
-                      : (size_t)(row_block(batch) + kXsumStride) * batch * sizeof(float) + 64;
+    (void)arith;
+    return (size_t)row_block(batch) * batch * sizeof(float) + 128;
 }
 
 // Items of the MFMA path that each wavefront of a workgroup takes (contiguous runs).
@@ -133,8 +134,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
     static_assert(!kQ8 || BATCH * kQ8Pieces <= 16, "pieces of all batch rows must fit the 16 operand columns");
     float* racc = (float*)lds_raw;                              // [kRowBlock][BATCH] row sums
     float* xtot = racc + kRowBlock * BATCH;                     // [16] sum of the staged input per batch row
-    float* xsum = xtot + 16;                                    // [BATCH][kXsumStride] per-unit input sums
-    uint32_t* smax = (uint32_t*)xsum;                           // kQ8: [16] largest |input| per batch row (bits)
+    uint32_t* smax = (uint32_t*)(xtot + 16);                    // kQ8: [16] largest |input| per batch row (bits)
     uint4* xs = lds_raw + stream_head_bytes(BATCH, ARITH) / sizeof(uint4);
     __shared__ int s_flag;
     const int tid = threadIdx.x;
@@ -260,7 +260,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                                 lds_barrier();
                             }
                             if constexpr (kQ8) stage_units_q8<DT, BATCH, THREADS>(xs, smax, xtot, sin, c0, cu_n, upad);
-                            else stage_units<DT, BATCH, kPow2Mfma>(xs, xsum, sin, c0, cu_n, upad, kStreamThreads,
+                            else stage_units<DT, BATCH, kPow2Mfma>(xs, nullptr, sin, c0, cu_n, upad, kStreamThreads,
                                                                    kPow2Mfma ? xtot : nullptr);
                             staged = true;
                         }
@@ -458,7 +458,6 @@ static void stream_lds_plan(int batch, int arith, int max_units, int* chunk_cap_
     }
     int chunk_cap = (kStreamLdsMax - racc_bytes - batch * (int)sizeof(uint4)) / (batch * 16 * (int)sizeof(uint4));
     chunk_cap = (chunk_cap - 1) & ~1;
-    if (chunk_cap > kXsumStride - 2) chunk_cap = kXsumStride - 2;
     const int chunk_units = max_units < chunk_cap ? max_units : chunk_cap;
     *chunk_cap_out = chunk_cap;
     *lds_out = (size_t)racc_bytes + (size_t)xs_chunks(batch, chunk_units | 1) * sizeof(uint4);
