@@ -76,9 +76,9 @@ class SynthLinear:
         return self._tiled
 
     def add_to(self, rl, x, keep_row_major=True, **kw):
-        """Tile order for the HBM-bound small batches; batch >= 4 runs on 16-bit MFMA operands, is bound by its
+        """Tile order for the HBM-bound small batches; batch >= 8 runs on 16-bit MFMA operands, is bound by its
         arithmetic and measures 3 % slower on tiled words, so it reads the row-major ones."""
-        if rl.batch > 2:
+        if rl.batch > 4:
             return rl.add(x, self.s_in, self.vt_bits, self.s_mid, self.u_bits, self.s_out, **kw)
         vt, u = self.runlist_words(keep_row_major)
         return rl.add(x, self.s_in, vt, self.s_mid, u, self.s_out, tiled=True, **kw)

@@ -463,20 +463,21 @@ static void stream_lds_plan(int batch, int arith, int max_units, int* chunk_cap_
     *lds_out = (size_t)racc_bytes + (size_t)xs_chunks(batch, chunk_units | 1) * sizeof(uint4);
 }
 
-// Which arithmetic, by batch and element type (measured on Llama-2-7B layers: one launch per layer / 26 layers per
-// launch, us per layer):
+// Which arithmetic, by batch (measured on Llama-2-7B layers with row-major words: one launch per layer / 26 layers
+// per launch, us per layer):
 //                                          batch 1        batch 2        batch 4
-//   fp4 x fp8 pieces (ARITH 2), any type   20.2 /  6.9    24.1 /  7.4    30.1 / 10.3
-//   16-bit MFMA operands (ARITH 1), fp16   25.4 / 11.5    25.5 / 11.9    27.0 / 13.1
+//   fp4 x fp8 pieces (ARITH 2), any type   20.2 /  6.9    24.1 /  7.4    31.4 / 10.9
+//   16-bit MFMA operands (ARITH 1), fp16   25.4 / 11.5    25.5 / 11.9    29.8 / 14.2
 //                                   bf16   36.4 / 21.1    31.1 / 17.1    32.3 / 18.4
 // The fp4 x fp8 arithmetic is three times cheaper per packed bit, but every workgroup quantises the whole input
-// vector of its stage (about 110 VALU instructions per 8 columns and batch row), which at batch 4 costs more than
-// the arithmetic saves when a launch covers only one layer.  Its staging does not depend on the element type, so
-// bf16 runs as fast as fp16.  Batch 8 and 16 need more operand columns than one MFMA has.
+// vector of its stage (about 110 VALU instructions per 8 columns and batch row): at batch 4 that costs as much as
+// the arithmetic saves when a launch covers only one layer, and a third less time in long run lists (Llama-3-70B
+// stream at batch 4: 2.3 against 3.6 ms).  Its staging does not depend on the element type, so bf16 runs as fast
+// as fp16.  Batch 8 and 16 need more operand columns than one MFMA has.
 // Every workgroup stages the whole input vector of its stage, so larger workgroups mean less staging work per
 // row: 1024 lanes everywhere (batch 16: 211 -> 80 us per layer going from 256 to 1024 lanes).
 #ifndef NQ_STREAM_ARITH
-#define NQ_STREAM_ARITH(DT, BATCH) (((BATCH) <= 2 || ((BATCH) == 4 && (DT) == 1)) ? 2 : 1)
+#define NQ_STREAM_ARITH(DT, BATCH) ((BATCH) <= 4 ? 2 : 1)
 #endif
 #ifndef NQ_STREAM_THREADS
 #define NQ_STREAM_THREADS(DT, BATCH) 1024
