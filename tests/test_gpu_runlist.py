@@ -254,3 +254,27 @@ def test_tiled_factor_size_is_checked(dev):
     rl = DecodeRunList(1, torch.float16, dev)
     with pytest.raises(RuntimeError):
         rl.add(x, ops[0], ops[1].reshape(-1), ops[2], ops[3].reshape(-1), ops[4], tiled=True)   # row-major sizes
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fp8_staging_with_an_outlier_and_a_zero_row(dev, dtype):
+    # batch row 0: one activation 1000x the rest (the scale of the fp8 pieces follows the outlier, the other elements
+    # sit 10 binades lower); batch row 1: all zeros (its scale must stay finite and its output exactly zero)
+    m, n, r = 512, 2048, 256
+    vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, 500)
+    x = oracle.synth_x(2, n, 501)
+    x[0, 777] = 900.0
+    x[1, :] = 0.0
+    to = lambda a: torch.from_numpy(a).to(dev).to(dtype)
+    f64 = lambda t: t.float().cpu().numpy().astype(np.float64)
+    xd, sc = to(x), (to(s_in), to(s_mid), to(s_out))
+    rl = DecodeRunList(2, dtype, dev)
+    i = rl.add(xd, sc[0], packing.binary_packer(torch.from_numpy(vt), "half2").to(dev), sc[1],
+               packing.binary_packer(torch.from_numpy(u), "half2").to(dev), sc[2], out_f32=True)
+    y = rl.run()[i].cpu().numpy()
+    torch.cuda.synchronize()
+    assert rl.status() == 0
+    ref = oracle.layer_forward(f64(xd), vt, u, f64(sc[0]), f64(sc[1]), f64(sc[2]), dtype=np.float64)
+    assert np.all(np.isfinite(y))
+    assert np.array_equal(y[1], np.zeros(m, dtype=np.float32))
+    assert np.abs(y[0] - ref[0]).max() / np.abs(ref[0]).max() < 1e-3
