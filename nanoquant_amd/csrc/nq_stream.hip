@@ -593,6 +593,7 @@ static hipError_t launch_single(const RunStage& st, hipStream_t stream) {
 
 // Only the batch sizes that the per-linear path sends here are instantiated.
 hipError_t gemv_stream_single(int dtype, int batch, const RunStage& st, hipStream_t stream) {
+    if (batch == 8) return dtype == 0 ? launch_single<0, 8>(st, stream) : launch_single<1, 8>(st, stream);
     if (batch != 16) return hipErrorInvalidValue;
     return dtype == 0 ? launch_single<0, 16>(st, stream) : launch_single<1, 16>(st, stream);
 }

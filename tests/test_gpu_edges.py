@@ -40,7 +40,7 @@ def test_empty_batch_and_zero_tokens(dev):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("batch", [16, 21, 48])
 def test_batches_split_into_pieces(dev, dtype, batch):
-    # 16-row pieces go through the run-list kernel on a single stage, the remainder (4 + 1) through the
+    # 16- and 8-row pieces go through the run-list kernel on a single stage, the remainder (4 + 1) through the
     # lane-group kernel; every row must come out as if computed alone
     m, n, r = 1376, 2048, 736          # 23 words per second-stage row: ragged 16-byte units
     term = oracle.synth_term(m, n, r, 50 + batch)
