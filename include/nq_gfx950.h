@@ -95,14 +95,14 @@ int nq_gemv_mixture(const void* x, const void* const* s_in, const uint32_t* cons
  * nq_runlist_status copies the error word back (synchronises): 0 ok, 1 = a bounded dependency wait
  * expired (the results of that run are invalid; call nq_runlist_build again before reuse). */
 typedef struct nq_linear {
-    const void* x;
+    const void* x;          /* NULL: bound at run time (nq_runlist_run_bound) */
     const void* s_in;
     const uint32_t* vt_bits;
     const void* s_mid;      /* may be NULL */
     const uint32_t* u_bits;
     const void* s_out;
     float* h;
-    void* y;
+    void* y;                /* NULL: bound at run time */
     const float* addend;    /* may be NULL */
     int n, r, m;
     int x_from;             /* -1: x is an external input */
@@ -115,12 +115,19 @@ typedef struct nq_linear {
 /* Launch geometry of a built run list; filled by nq_runlist_build, passed back to nq_runlist_run. */
 typedef struct nq_runlist_plan {
     int nlinears, nstages, nphases, workgroups, max_units, batch, dtype, index_words;
+    int bound;              /* bit 0: some x was NULL, bit 1: some y was NULL (nq_runlist_run_bound must supply them) */
 } nq_runlist_plan;
 
 size_t nq_runlist_workspace_bytes(const nq_linear* linears, int nlinears);
 int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtype, int interleave,
                      void* workspace, size_t workspace_bytes, nq_runlist_plan* plan_out, void* stream);
 int nq_runlist_run(const void* workspace, const nq_runlist_plan* plan, void* stream);
+/* The same with the input and output that the list left open: every nq_linear whose x is NULL reads `x`
+ * ([batch, n] of the list's dtype, 16-byte aligned; they must agree on n), at most one linear may leave y NULL and it writes `y`.
+ * Lets one built list serve a module whose activations live somewhere else on every call (one launch per linear
+ * instead of the reference's two, modules/linear.py:121-130).  Linears with a NULL x or y must not be referred to
+ * by x_from / y_from. */
+int nq_runlist_run_bound(const void* workspace, const nq_runlist_plan* plan, const void* x, void* y, void* stream);
 int nq_runlist_status(const void* workspace, int* status_out, void* stream);
 
 /* One matmul-free stage: out[b,row] = s_row[row] * sum_c sgn(bits[row,c]) * in[b,c] * s_col[c].

@@ -39,7 +39,7 @@ const char* nq_status_string(int status) {
 
 int nq_last_hip_error(void) { return g_last_hip_error; }
 
-int nq_abi_version(void) { return 3; }
+int nq_abi_version(void) { return 4; }
 
 int nq_device_query(int attr, int* value) {
     if (!value) return NQ_ERR_NULL;
@@ -153,12 +153,23 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
     for (int i = 0; i < nlinears; ++i) {
         const nq_linear& l = linears[i];
         if (l.n <= 0 || l.r <= 0 || l.m <= 0) return NQ_ERR_SHAPE;
-        if (!l.x || !l.s_in || !l.vt_bits || !l.u_bits || !l.s_out || !l.h || !l.y) return NQ_ERR_NULL;
+        if (!l.s_in || !l.vt_bits || !l.u_bits || !l.s_out || !l.h) return NQ_ERR_NULL;   // x, y NULL: bound at run time
+        if (!l.x && l.x_from >= 0) return NQ_ERR_SHAPE;
         if (l.x_from >= i || l.y_from >= i) return NQ_ERR_SHAPE;
+        if (l.x_from >= 0 && !linears[l.x_from].y) return NQ_ERR_SHAPE;   // a bound output cannot feed another entry
+        if (l.y_from >= 0 && !linears[l.y_from].y) return NQ_ERR_SHAPE;
         if (l.y_from >= 0 && !linears[l.y_from].out_f32) return NQ_ERR_SHAPE;   // addends are fp32 results
         // two linears writing the same h would race inside a phase
         for (int j = 0; j < i; ++j)
             if (linears[j].h == l.h) return NQ_ERR_SHAPE;
+    }
+    int bound_n = 0, bound_outputs = 0;
+    for (int i = 0; i < nlinears; ++i) {         // one bound x (shared by every entry that reads it), one bound y
+        if (!linears[i].x) {
+            if (bound_n && bound_n != linears[i].n) return NQ_ERR_SHAPE;
+            bound_n = linears[i].n;
+        }
+        if (!linears[i].y && ++bound_outputs > 1) return NQ_ERR_SHAPE;
     }
     if (workspace_bytes < nq_runlist_workspace_bytes(linears, nlinears)) return NQ_ERR_WORKSPACE;
     (void)interleave;   // kept for interface stability: phases make the ordering hint unnecessary
@@ -171,13 +182,13 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         const nq_linear& l = linears[i];
         nq::RunStage a{};
         a.bits = l.vt_bits; a.in = l.x; a.s_col = (const uint16_t*)l.s_in; a.s_row = (const uint16_t*)l.s_mid;
-        a.out = l.h; a.addend = nullptr; a.tiled = l.tiled ? 1 : 0;
+        a.out = l.h; a.addend = nullptr; a.tiled = l.tiled ? 1 : 0; a.in_ext = l.x ? 0 : 1;
         a.rows = l.r; a.K = l.n; a.words = (l.n + 31) / 32; a.units = (a.words + 3) / 4;
         a.in_stride = l.n; a.out_stride = l.r; a.in_f32 = 0; a.out_f32 = 1;
         a.dep = l.x_from >= 0 ? 2 * l.x_from + 1 : -1;
         a.dep2 = -1;
         a.vec_bits = (a.words % 4 == 0) && al16(l.vt_bits);
-        a.vec_in = al16(l.x) && ((size_t)l.n * 2) % 16 == 0 && al16(l.s_in);
+        a.vec_in = al16(l.x) && ((size_t)l.n * 2) % 16 == 0 && al16(l.s_in);   // a bound x must be 16-byte aligned
         a.phase = a.dep >= 0 ? table[a.dep].phase + 1 : 0;
         if (a.dep >= 0) {                        // 16-bit y of an earlier linear is this linear's x
             a.heavy_acquire = 1;
@@ -187,7 +198,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
 
         nq::RunStage b{};
         b.bits = l.u_bits; b.in = l.h; b.s_col = nullptr; b.s_row = (const uint16_t*)l.s_out;
-        b.out = l.y; b.addend = l.addend; b.bias = (const uint16_t*)l.bias; b.tiled = l.tiled ? 1 : 0;
+        b.out = l.y; b.addend = l.addend; b.bias = (const uint16_t*)l.bias; b.tiled = l.tiled ? 1 : 0; b.out_ext = l.y ? 0 : 1;
         b.rows = l.m; b.K = l.r; b.words = (l.r + 31) / 32; b.units = (b.words + 3) / 4;
         b.in_stride = l.r; b.out_stride = l.m; b.in_f32 = 1; b.out_f32 = l.out_f32 ? 1 : 0;
         b.dep = 2 * i;
@@ -358,11 +369,19 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
     plan_out->batch = batch;
     plan_out->dtype = dtype;
     plan_out->index_words = (int)seg_index.size();
+    plan_out->bound = 0;
+    for (int i = 0; i < nlinears; ++i) plan_out->bound |= (linears[i].x ? 0 : 1) | (linears[i].y ? 0 : 2);
     return hip_status(hipStreamSynchronize(hs));   // the tables are host memory: finish before they die
 }
 
 int nq_runlist_run(const void* workspace, const nq_runlist_plan* plan, void* stream) {
+    return nq_runlist_run_bound(workspace, plan, nullptr, nullptr, stream);
+}
+
+int nq_runlist_run_bound(const void* workspace, const nq_runlist_plan* plan, const void* x, void* y, void* stream) {
     if (!workspace || !plan) return NQ_ERR_NULL;
+    if (((plan->bound & 1) && !x) || ((plan->bound & 2) && !y)) return NQ_ERR_NULL;
+    if (((uintptr_t)x) & 15u) return NQ_ERR_ALIGN;
     if (plan->dtype != NQ_F16 && plan->dtype != NQ_BF16) return NQ_ERR_DTYPE;
     if (plan->nlinears <= 0 || plan->nstages != 2 * plan->nlinears || plan->workgroups <= 0 || plan->max_units <= 0 ||
         plan->nphases <= 0 || plan->index_words != plan->workgroups * plan->nphases + 1)
@@ -376,7 +395,7 @@ int nq_runlist_run(const void* workspace, const nq_runlist_plan* plan, void* str
     return hip_status(nq::gemv_stream(plan->dtype, batch, (const nq::RunStage*)(base + off_table), plan->nstages,
                                       plan->nphases, (const int*)(base + off_index),
                                       (const nq::RunSegment*)(base + off_segs), (unsigned long long*)(base + 256),
-                                      (unsigned*)base, plan->workgroups, plan->max_units, (hipStream_t)stream));
+                                      (unsigned*)base, plan->workgroups, plan->max_units, (hipStream_t)stream, x, y));
 }
 
 int nq_runlist_status(const void* workspace, int* status_out, void* stream) {

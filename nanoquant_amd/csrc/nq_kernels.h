@@ -34,6 +34,8 @@ struct RunStage {
     int heavy_release;      // 16-bit output read by a later stage: full device-scope release on completion
     int heavy_acquire;      // 16-bit input written by an earlier stage: full device-scope acquire after the wait
     int tiled;              // `bits` is in the tile order of tile_words() instead of row-major
+    int in_ext, out_ext;    // `in` / `out` are given with the launch instead (bound input / output of the list)
+    int pad_;
 };
 // One workgroup's share of one stage: rows [row_begin, row_end).
 struct RunSegment {
@@ -44,7 +46,7 @@ int stream_capacity(int dtype, int batch, int max_units);
 int stream_row_granule(int dtype, int batch);
 hipError_t gemv_stream(int dtype, int batch, const RunStage* stages, int nstages, int nphases, const int* seg_index,
                        const RunSegment* segs, unsigned long long* counters, unsigned* status, int nwg, int max_units,
-                       hipStream_t stream);
+                       hipStream_t stream, const void* ext_in = nullptr, void* ext_out = nullptr);
 
 // One stage on its own through the run-list kernel (no tables, no counters); batch 16 only.
 hipError_t gemv_stream_single(int dtype, int batch, const RunStage& st, hipStream_t stream);

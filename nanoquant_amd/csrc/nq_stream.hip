@@ -121,7 +121,8 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                                                                      const RunSegment* __restrict__ segs,
                                                                      unsigned long long* counters, unsigned* status,
                                                                      unsigned spin_limit, int chunk_cap,
-                                                                     RunStage single, int single_rows) {
+                                                                     RunStage single, int single_rows,
+                                                                     const void* ext_in, void* ext_out) {
     using E = Elem<DT>;
     constexpr int kStreamThreads = THREADS;
     constexpr int kWaves = THREADS / kWave;
@@ -175,6 +176,8 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
             } else {
                 seg = segs[sg];
                 st = stages[seg.stage];
+                if (st.in_ext) st.in = ext_in;          // bound with the launch
+                if (st.out_ext) st.out = ext_out;
             }
             const BitsView bv = bits_view(st);
             const int chunk_units = min(st.units, chunk_cap);
@@ -521,7 +524,7 @@ static int capacity_of(int max_units) {
 template <int DT, int BATCH>
 static hipError_t launch_stream(const RunStage* stages, int nstages, int nphases, const int* seg_index,
                                 const RunSegment* segs, unsigned long long* counters, unsigned* status, int nwg,
-                                int max_units, hipStream_t stream) {
+                                int max_units, hipStream_t stream, const void* ext_in, void* ext_out) {
     int chunk_cap;
     size_t lds;
     stream_lds_plan(BATCH, StreamKernel<DT, BATCH>::kArith, max_units, &chunk_cap, &lds);
@@ -538,7 +541,7 @@ static hipError_t launch_stream(const RunStage* stages, int nstages, int nphases
 #endif
     using SK = StreamKernel<DT, BATCH>;
     hipLaunchKernelGGL((SK::fn), dim3(nwg), dim3(SK::kThreads), lds, stream, stages, nstages,
-                       nphases, seg_index, segs, counters, status, (unsigned)(1u << 21), chunk_cap, RunStage{}, 0);
+                       nphases, seg_index, segs, counters, status, (unsigned)(1u << 21), chunk_cap, RunStage{}, 0, ext_in, ext_out);
 #ifdef NQ_TRACE
     if (tbuf && ++calls == 40) {
         (void)hipStreamSynchronize(stream);
@@ -587,7 +590,7 @@ static hipError_t launch_single(const RunStage& st, hipStream_t stream) {
     const int nwg = (st.rows + rows_per_wg - 1) / rows_per_wg;
     hipLaunchKernelGGL((SK::fn_single), dim3(nwg), dim3(SK::kThreads), lds, stream, (const RunStage*)nullptr, 0, 1,
                        (const int*)nullptr, (const RunSegment*)nullptr, (unsigned long long*)nullptr, (unsigned*)nullptr,
-                       0u, chunk_cap, st, rows_per_wg);
+                       0u, chunk_cap, st, rows_per_wg, (const void*)nullptr, (void*)nullptr);
     return hipGetLastError();
 }
 
@@ -626,8 +629,8 @@ int stream_row_granule(int dtype, int batch) {
 
 hipError_t gemv_stream(int dtype, int batch, const RunStage* stages, int nstages, int nphases, const int* seg_index,
                        const RunSegment* segs, unsigned long long* counters, unsigned* status, int nwg, int max_units,
-                       hipStream_t stream) {
-#define NQ_RUN(D, B) launch_stream<D, B>(stages, nstages, nphases, seg_index, segs, counters, status, nwg, max_units, stream)
+                       hipStream_t stream, const void* ext_in, void* ext_out) {
+#define NQ_RUN(D, B) launch_stream<D, B>(stages, nstages, nphases, seg_index, segs, counters, status, nwg, max_units, stream, ext_in, ext_out)
     NQ_STREAM_DISPATCH(NQ_RUN)
 #undef NQ_RUN
     return hipErrorInvalidValue;

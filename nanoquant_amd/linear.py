@@ -20,6 +20,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import ops
+from .runlist import DecodeRunList
 from .packing import (binary_packer, binary_unpacker, marlin_nanoquant_packer, repack_words)
 
 
@@ -42,6 +43,13 @@ class NanoQuantLinear(nn.Module):
         # False mirrors the reference, whose kernel paths return before the bias is added; True adds it in the
         # epilogue of the last kernel (decode and prefill alike).
         self.kernel_path_bias = False
+        # True: a decode call of 1, 2, 4, 8 or 16 rows is ONE launch of the run-list kernel (both stages, the
+        # scales and the bias) on a list built once per row count, instead of the two launches of the
+        # reference's op (linear.py:121-130).  It bypasses the torch op, so leave it off under torch.compile.
+        self.fused_launch = False
+        self._fused_lists = {}
+        self._fused_tiled = None
+        self._fused_bias = None
         self.register_parameter("weight", None)
         if bias:
             self.bias = nn.Parameter(torch.zeros(out_features, device=device, dtype=dtype), requires_grad=False)
@@ -112,7 +120,9 @@ class NanoQuantLinear(nn.Module):
             bias = None
             if self.kernel_path_bias and self.bias is not None:
                 bias = self.bias if self.bias.dtype == self.dtype else self.bias.to(self.dtype)
-            if self.kernel_type == "gemv":
+            if self.kernel_type == "gemv" and self.fused_launch and x.shape[0] in DecodeRunList.BATCHES:
+                y = self._fused_forward(x, bias)
+            elif self.kernel_type == "gemv":
                 if bias is not None:
                     y = ops.gemv_forward_with_bias(x, self.scale_pre, self.V_int8, self.scale_mid, self.U_int8,
                                                    self.scale_post, bias)
@@ -137,6 +147,41 @@ class NanoQuantLinear(nn.Module):
             y += self.bias
         return y
 
+    def _fused_forward(self, x: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+        """One launch for the whole layer: a one-entry run list per row count whose input and output are
+        bound at launch.  Up to 4 rows the list reads a tile-order copy of the packed factors (made once,
+        one more bit per weight of device memory); above, the row-major words the op reads."""
+        rows = x.shape[0]
+        if not x.is_cuda:
+            raise RuntimeError("the fused decode launch needs GPU tensors")
+        if x.data_ptr() % 16 != 0:
+            x = x.clone()
+        if bias is not None and bias is not self.bias:     # a converted copy: keep one, so that the list can point at it
+            tag = (self.bias.data_ptr(), self.bias._version)
+            if self._fused_bias is None or self._fused_bias[0] != tag:
+                self._fused_bias = (tag, bias.contiguous())
+            bias = self._fused_bias[1]
+        key = (rows, None if bias is None else bias.data_ptr(), x.device)
+        rl = self._fused_lists.get(key)
+        if rl is None:
+            tiled = rows <= 4
+            if tiled:
+                if self._fused_tiled is None:
+                    self._fused_tiled = (ops.tile_words_device(self.V_int8, False), ops.tile_words_device(self.U_int8, False))
+                V, U = self._fused_tiled
+            else:
+                V, U = self.V_int8, self.U_int8
+            scale_mid = self.scale_mid
+            if tiled and scale_mid is None:      # the tile order carries no rank: a unit scale_mid supplies it
+                scale_mid = torch.ones(self.V_int8.shape[0], dtype=self.dtype, device=x.device)
+            rl = DecodeRunList(rows, dtype=self.dtype, device=x.device)
+            rl.add(None, self.scale_pre, V, scale_mid, U, self.scale_post, bias=bias, tiled=tiled, bind_y=True)
+            rl.build()
+            self._fused_lists[key] = rl
+        y = torch.empty((rows, self.scale_post.numel()), dtype=self.dtype, device=x.device)
+        rl.run(x=x, y=y)
+        return y
+
     def _compute_forward(self, x, V, U, scale_pre, scale_mid, scale_post):
         """Dense definition of the layer (reference: linear.py:248-257)."""
         y = F.linear(x * scale_pre, V)
@@ -154,6 +199,7 @@ class NanoQuantLinear(nn.Module):
         self.do_kernel_inference = True
         self.kernel_type = kernel_type
         self.dtype = dtype
+        self._fused_lists, self._fused_tiled, self._fused_bias = {}, None, None
 
         self.scale_pre = nn.Parameter(self.scale_pre.to(dtype).squeeze(0), requires_grad=False)
         self.scale_post = nn.Parameter(self.scale_post.to(dtype).squeeze(0), requires_grad=False)

@@ -32,7 +32,7 @@ class NqRunlistPlan(ctypes.Structure):
     """Mirror of `nq_runlist_plan`."""
     _fields_ = [("nlinears", ctypes.c_int), ("nstages", ctypes.c_int), ("nphases", ctypes.c_int),
                 ("workgroups", ctypes.c_int), ("max_units", ctypes.c_int), ("batch", ctypes.c_int),
-                ("dtype", ctypes.c_int), ("index_words", ctypes.c_int)]
+                ("dtype", ctypes.c_int), ("index_words", ctypes.c_int), ("bound", ctypes.c_int)]
 
 
 class DecodeRunList:
@@ -52,14 +52,22 @@ class DecodeRunList:
         self._workspace: Optional[torch.Tensor] = None
 
     # ---- building -----------------------------------------------------------------------------
-    def add(self, x: torch.Tensor, scale_pre: torch.Tensor, V_int8: torch.Tensor, scale_mid: Optional[torch.Tensor],
+    def add(self, x: Optional[torch.Tensor], scale_pre: torch.Tensor, V_int8: torch.Tensor, scale_mid: Optional[torch.Tensor],
             U_int8: torch.Tensor, scale_post: torch.Tensor, y: Optional[torch.Tensor] = None,
             x_from: int = -1, addend: Optional[torch.Tensor] = None, y_from: int = -1,
-            out_f32: bool = False, bias: Optional[torch.Tensor] = None, tiled: bool = False) -> int:
+            out_f32: bool = False, bias: Optional[torch.Tensor] = None, tiled: bool = False,
+            bind_y: bool = False) -> int:
         """Append one linear (operands as `NanoQuantLinear` holds them after `_prepare_kernel('gemv')`:
         V_int8 [r, n/32] first stage, U_int8 [m, r/32] second stage).  Returns its index; `y` is
-        allocated when not given and is available as `outputs[index]`.  `bias` [m] is added after `scale_post`."""
-        n = x.shape[-1]
+        allocated when not given and is available as `outputs[index]`.  `bias` [m] is added after `scale_post`.
+
+        `x=None` leaves the input unbound and `bind_y=True` the output: `run(x=..., y=...)` supplies them
+        with each launch (one pointer each for the whole list), so one built list serves any tensors."""
+        if x is None and x_from >= 0:
+            raise RuntimeError("an entry fed by another entry cannot take a late-bound input")
+        if bind_y and y is not None:
+            raise RuntimeError("bind_y leaves the output to run(); do not pass y as well")
+        n = scale_pre.numel() if x is None else x.shape[-1]
         if tiled:
             # tile order (packing.tile_words): flat buffers, the rank comes from scale_mid / the word count
             if scale_mid is None:
@@ -69,9 +77,11 @@ class DecodeRunList:
             r, m = V_int8.shape[0], U_int8.shape[0]
         for name, t, dt in (("x", x, self.dtype), ("scale_pre", scale_pre, self.dtype), ("scale_post", scale_post, self.dtype),
                             ("V_int8", V_int8, torch.int32), ("U_int8", U_int8, torch.int32)):
+            if t is None:
+                continue
             if not t.is_cuda or not t.is_contiguous() or t.dtype != dt:
                 raise RuntimeError(f"{name} must be a contiguous {dt} tensor on the GPU")
-        if x.numel() != self.batch * n:
+        if x is not None and x.numel() != self.batch * n:
             raise RuntimeError(f"x must hold {self.batch} rows of {n}")
         if tiled:
             lib = _lib.lib()
@@ -83,7 +93,7 @@ class DecodeRunList:
             raise RuntimeError("scale size mismatch")
         if bias is not None and (not bias.is_cuda or not bias.is_contiguous() or bias.dtype != self.dtype or bias.numel() != m):
             raise RuntimeError(f"bias must be a contiguous {self.dtype} tensor of {m} elements on the GPU")
-        if y is None:
+        if y is None and not bind_y:
             y = torch.empty((self.batch, m), dtype=torch.float32 if out_f32 else self.dtype, device=self.device)
         h = torch.empty((self.batch, r), dtype=torch.float32, device=self.device)
         self._keep += [x, scale_pre, V_int8, scale_mid, U_int8, scale_post, y, h, addend, bias]
@@ -122,14 +132,30 @@ class DecodeRunList:
         return _lib.NQ_F16 if self.dtype == torch.float16 else _lib.NQ_BF16
 
     # ---- running --------------------------------------------------------------------------------
-    def run(self) -> Sequence[torch.Tensor]:
-        """Enqueue the launch on the current stream (no allocation, no synchronisation)."""
+    def run(self, x: Optional[torch.Tensor] = None, y: Optional[torch.Tensor] = None) -> Sequence[torch.Tensor]:
+        """Enqueue the launch on the current stream (no allocation, no synchronisation).  `x` / `y` are
+        the tensors of the entries added with `x=None` / `bind_y=True`."""
         if self._workspace is None:
             self.build()
+        need_x = any(e["x"] is None for e in self._entries)
+        need_y = any(e["y"] is None for e in self._entries)
+        if need_x != (x is not None) or need_y != (y is not None):
+            raise RuntimeError("run(x=, y=) must be given exactly when the list has late-bound entries")
+        for name, t, key in (("x", x, "n"), ("y", y, "m")):
+            if t is None:
+                continue
+            ent = [e for e in self._entries if e[name] is None]
+            width = ent[0][key]
+            dt = torch.float32 if (name == "y" and ent[0]["out_f32"]) else self.dtype
+            if any(e[key] != width for e in ent) or (name == "y" and any(e["out_f32"] != ent[0]["out_f32"] for e in ent)):
+                raise RuntimeError(f"late-bound entries must agree on the shape of {name}")
+            if not t.is_cuda or not t.is_contiguous() or t.dtype != dt or t.numel() != self.batch * width:
+                raise RuntimeError(f"{name} must be a contiguous {dt} tensor of {self.batch} x {width} on the GPU")
+        p = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())
         with torch.cuda.device(self.device):
             stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
-            _lib.check(_lib.lib().nq_runlist_run(ctypes.c_void_p(self._workspace.data_ptr()),
-                                                 ctypes.byref(self._plan), stream))
+            _lib.check(_lib.lib().nq_runlist_run_bound(ctypes.c_void_p(self._workspace.data_ptr()),
+                                                       ctypes.byref(self._plan), p(x), p(y), stream))
         return self.outputs
 
     def status(self) -> int:
