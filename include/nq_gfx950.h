@@ -167,6 +167,30 @@ int nq_gemm_nanoquant_bias(const void* x, const uint32_t* vt_tiles, const uint32
                            const void* s_mid, const void* s_out, const void* bias, void* h, void* y, void* scratch,
                            size_t scratch_bytes, int tokens, int n, int r, int m, int dtype, void* stream);
 
+/* Several terms with the same token count in two launches instead of two per term: the first GEMMs of all
+ * terms, then the second ones (the projections of a decoder block that read the same tokens: q/k/v, gate/up, or
+ * independent linears of a layer).  Up to 128 tokens a single term cannot fill the device and is bound by launch
+ * and load latencies; grouped, the same launches carry several times the work.  Above 128 tokens the call runs
+ * the terms one after another (nq_gemm_nanoquant_bias) and needs their scratch: max over terms of
+ * nq_gemm_scratch_bytes for both GEMMs, may be NULL up to 128 tokens.  count <= nq_gemm_group_max(); h and y of
+ * different terms must not coincide.  No counterpart in the reference, which launches each linear by itself
+ * (modules/linear.py:131-133). */
+typedef struct nq_gemm_term {
+    const void* x;               /* [tokens, n] */
+    const uint32_t* vt_tiles;    /* first stage, [r rows x n] in the prefill tile layout */
+    const uint32_t* u_tiles;     /* second stage, [m rows x r] */
+    const void* s_in;            /* [n] or NULL (all terms alike) */
+    const void* s_mid;           /* [r] or NULL */
+    const void* s_out;           /* [m] or NULL */
+    const void* bias;            /* [m] or NULL */
+    void* h;                     /* [tokens, r] */
+    void* y;                     /* [tokens, m] */
+    int n, r, m;                 /* n % 256 == 0, r % 256 == 0, m % 32 == 0 */
+} nq_gemm_term;
+int nq_gemm_group_max(void);
+int nq_gemm_nanoquant_group(const nq_gemm_term* terms, int count, int tokens, int dtype, void* scratch,
+                            size_t scratch_bytes, void* stream);
+
 /* Word-order conversion on the device, in place allowed (dst == src): the checkpoint format
  * ("lsb_first", modules/linear.py:298) to the kernel format ("half2", modules/linear.py:171-172)
  * without the dense round trip of utils/load_utils.py:269-293.  order ids: nq_word_order. */

@@ -37,6 +37,8 @@ _SIGNATURES = {
     "nq_gemm_onebit_bias": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),
     "nq_gemm_nanoquant_bias": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
     "nq_repack_words": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
+    "nq_gemm_group_max": (_i, []),
+    "nq_gemm_nanoquant_group": (_i, [_vp, _i, _i, _i, _vp, _sz, _vp]),
     "nq_tiled_words": (_sz, [_i, _i]),
     "nq_tile_words": (_i, [_vp, _vp, _i, _i, _i, _vp]),
     "nq_stream_copy": (_i, [_vp, _vp, _sz, _vp]),

@@ -447,6 +447,52 @@ int nq_gemm_nanoquant_bias(const void* x, const uint32_t* vt_tiles, const uint32
     return nq_gemm_onebit_bias(h, u_tiles, nullptr, s_out, bias, y, scratch, scratch_bytes, tokens, r, m, dtype, stream);
 }
 
+int nq_gemm_group_max(void) { return nq::gemm_group_max(); }
+
+int nq_gemm_nanoquant_group(const nq_gemm_term* terms, int count, int tokens, int dtype, void* scratch,
+                            size_t scratch_bytes, void* stream) {
+    if (dtype != NQ_F16 && dtype != NQ_BF16) return NQ_ERR_DTYPE;
+    if (count < 0 || tokens < 0) return NQ_ERR_SHAPE;
+    if (count == 0 || tokens == 0) return NQ_OK;
+    if (!terms) return NQ_ERR_NULL;
+    if (count > nq::gemm_group_max()) return NQ_ERR_SHAPE;
+    bool grouped = tokens <= nq::gemm_group_max_tokens();
+    for (int i = 0; i < count; ++i) {
+        const nq_gemm_term& t = terms[i];
+        if (t.n <= 0 || t.r <= 0 || t.m <= 0) return NQ_ERR_SHAPE;
+        if (t.n % 256 != 0 || t.r % 256 != 0 || t.m % 32 != 0) return NQ_ERR_PROB_SHAPE;
+        if (!t.x || !t.vt_tiles || !t.u_tiles || !t.h || !t.y) return NQ_ERR_NULL;
+        if (((uintptr_t)t.x | (uintptr_t)t.vt_tiles | (uintptr_t)t.u_tiles | (uintptr_t)t.h | (uintptr_t)t.y |
+             (uintptr_t)t.s_in | (uintptr_t)t.s_mid | (uintptr_t)t.s_out | (uintptr_t)t.bias) & 15u)
+            return NQ_ERR_ALIGN;
+        if ((t.s_in == nullptr) != (terms[0].s_in == nullptr)) grouped = false;   // one kernel variant per launch
+        for (int j = 0; j < i; ++j)
+            if (terms[j].h == t.h || terms[j].y == t.y) return NQ_ERR_SHAPE;      // results would overwrite each other
+    }
+    if (!grouped) {                              // many tokens: every GEMM fills the device by itself
+        for (int i = 0; i < count; ++i) {
+            const nq_gemm_term& t = terms[i];
+            int st = nq_gemm_nanoquant_bias(t.x, t.vt_tiles, t.u_tiles, t.s_in, t.s_mid, t.s_out, t.bias, t.h, t.y, scratch,
+                                            scratch_bytes, tokens, t.n, t.r, t.m, dtype, stream);
+            if (st != NQ_OK) return st;
+        }
+        return NQ_OK;
+    }
+    const void* x[8]; const uint32_t* w[8]; const void* si[8]; const void* so[8]; const void* bs[8]; void* out[8];
+    int K[8], R[8];
+    for (int i = 0; i < count; ++i) {
+        const nq_gemm_term& t = terms[i];
+        x[i] = t.x; w[i] = t.vt_tiles; si[i] = t.s_in; so[i] = t.s_mid; bs[i] = nullptr; out[i] = t.h; K[i] = t.n; R[i] = t.r;
+    }
+    hipError_t e = nq::gemm_onebit_group(dtype, count, x, w, si, so, bs, out, tokens, K, R, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_status(e);
+    for (int i = 0; i < count; ++i) {
+        const nq_gemm_term& t = terms[i];
+        x[i] = t.h; w[i] = t.u_tiles; si[i] = nullptr; so[i] = t.s_out; bs[i] = t.bias; out[i] = t.y; K[i] = t.r; R[i] = t.m;
+    }
+    return hip_status(nq::gemm_onebit_group(dtype, count, x, w, si, so, bs, out, tokens, K, R, (hipStream_t)stream));
+}
+
 size_t nq_tiled_words(int rows, int words) {
     if (rows <= 0 || words <= 0) return 0;
     return nq::tiled_word_count(rows, words);

@@ -219,7 +219,7 @@ __global__ __launch_bounds__(256) void gemm_onebit_kernel(GemmArgs a) {
 // No global atomics, no scratch, no second launch; R/32 x T/32 workgroups, and the wavefronts of a workgroup
 // never wait for each other inside the k loop (each stages its own activation slab).
 template <int DT, bool SCALED, int RT>
-__global__ __launch_bounds__(256) void gemm_kwave_kernel(GemmArgs a) {
+__device__ __forceinline__ void kwave_tile(const GemmArgs& a, int row_block, int token_block) {
     using E = Elem<DT>;
     constexpr int kPitch = slab_pitch<kTileK>();
     constexpr int kSlabHalves = 32 * kPitch + kTileK;            // slab + its 256 input scales
@@ -227,9 +227,9 @@ __global__ __launch_bounds__(256) void gemm_kwave_kernel(GemmArgs a) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint16_t* slab = slabs + wave * kSlabHalves;
     uint16_t* scale_lds = slab + 32 * kPitch;
-    const int rt = blockIdx.x * RT;                              // first of the RT 32-row tiles of this workgroup
+    const int rt = row_block * RT;                               // first of the RT 32-row tiles of this workgroup
     const int ntiles = min(RT, a.R / 32 - rt);
-    const int tok0 = blockIdx.y * 32;
+    const int tok0 = token_block * 32;
 
     float16_t acc[RT];
 #pragma unroll
@@ -250,6 +250,7 @@ __global__ __launch_bounds__(256) void gemm_kwave_kernel(GemmArgs a) {
         }
         if constexpr (SCALED) sr = *(const u32x4_t*)(a.s_in + k0 + 8 * (lane & 31));
     };
+
     const uint4* tile_ptr = a.tiles + (size_t)rt * a.ktiles * 64 + lane;
     const size_t tile_pitch = (size_t)a.ktiles * 64;             // uint4 elements between consecutive row tiles
     uint4 wnext[RT];
@@ -347,6 +348,32 @@ __global__ __launch_bounds__(256) void gemm_kwave_kernel(GemmArgs a) {
             if (tok < a.T) *(u32x4_t*)((uint16_t*)a.y + (size_t)tok * a.R + row0) = outv;
         }
     }
+}
+
+template <int DT, bool SCALED, int RT>
+__global__ __launch_bounds__(256) void gemm_kwave_kernel(GemmArgs a) {
+    kwave_tile<DT, SCALED, RT>(a, blockIdx.x, blockIdx.y);
+}
+
+// Several GEMMs of the few-token kind in one launch (the projections that share a layer's tokens): workgroup b
+// belongs to the problem p with first[p] <= b < first[p + 1]; inside a problem the row blocks run fastest, so
+// neighbours share an activation slab.  All problems have the same token count.
+constexpr int kGroupMax = 8;
+struct GemmGroup {
+    GemmArgs a[kGroupMax];
+    int first[kGroupMax + 1];
+    int count;
+};
+
+template <int DT, bool SCALED, int RT>
+__global__ __launch_bounds__(256) void gemm_kwave_group_kernel(GemmGroup g) {
+    const int b = blockIdx.x;
+    int p = 0;
+    while (p + 1 < g.count && b >= g.first[p + 1]) ++p;
+    const GemmArgs a = g.a[p];
+    const int local = b - g.first[p];
+    const int gx = (a.R / 32 + RT - 1) / RT;
+    kwave_tile<DT, SCALED, RT>(a, local % gx, local / gx);
 }
 
 // Scales, converts and stores the accumulated sums, and puts the accumulator back to zero: the scratch
@@ -509,5 +536,57 @@ hipError_t gemm_onebit(int dtype, const void* x, const uint32_t* tiles, const vo
     if (dtype == 0) return p.rt == 2 ? launch_gemm<0, 2, 2, 256>(a, p, stream) : launch_gemm<0, 2, 1, 256>(a, p, stream);
     return p.rt == 2 ? launch_gemm<1, 2, 2, 256>(a, p, stream) : launch_gemm<1, 2, 1, 256>(a, p, stream);
 }
+
+// Few-token GEMMs of several problems in one launch; every problem: K % 256 == 0, R % 32 == 0, tokens <=
+// kKwaveMaxTokens, and either all have input scales or none (checked by the caller).
+hipError_t gemm_onebit_group(int dtype, int count, const void* const* x, const uint32_t* const* tiles,
+                             const void* const* s_in, const void* const* s_out, const void* const* bias, void* const* y,
+                             int T, const int* K, const int* R, hipStream_t stream) {
+    if (count < 1 || count > kGroupMax || T > kKwaveMaxTokens) return hipErrorInvalidValue;
+    const int gy = (T + 31) / 32;
+    int rt = 4;                                  // widest row blocks that still leave two workgroups per CU
+    for (; rt > 1; rt /= 2) {
+        long total = 0;
+        for (int p = 0; p < count; ++p) total += (long)((R[p] / 32 + rt - 1) / rt) * gy;
+        if (total >= 512) break;
+    }
+    // Longest k first: the workgroups that run longest start first, the short ones fill in behind them.
+    int order[kGroupMax];
+    for (int p = 0; p < count; ++p) order[p] = p;
+    for (int i = 1; i < count; ++i)
+        for (int j = i; j > 0 && K[order[j]] > K[order[j - 1]]; --j) { const int t = order[j]; order[j] = order[j - 1]; order[j - 1] = t; }
+    GemmGroup g;
+    g.count = count;
+    int blocks = 0;
+    for (int p = 0; p < kGroupMax; ++p) {
+        const int q = order[p < count ? p : count - 1];
+        GemmArgs& a = g.a[p];
+        a.x = x[q]; a.tiles = (const uint4*)tiles[q];
+        a.s_in = (const uint16_t*)(s_in ? s_in[q] : nullptr); a.s_out = (const uint16_t*)(s_out ? s_out[q] : nullptr);
+        a.bias = (const uint16_t*)(bias ? bias[q] : nullptr);
+        a.y = y[q]; a.acc = nullptr;
+        a.T = T; a.K = K[q]; a.R = R[q];
+        a.ktiles = K[q] / kTileK; a.ktiles_per_split = a.ktiles; a.xcd_gx = 0;
+        g.first[p] = blocks;
+        if (p < count) blocks += ((R[q] / 32 + rt - 1) / rt) * gy;
+    }
+    g.first[kGroupMax] = blocks;
+    for (int p = count; p < kGroupMax; ++p) g.first[p] = blocks;
+    const bool scaled = g.a[0].s_in != nullptr;
+    const size_t lds = (size_t)4 * (32 * slab_pitch<kTileK>() + kTileK) * sizeof(uint16_t);
+    auto launch = [&](auto kern) -> hipError_t {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds, stream, g);
+        return hipGetLastError();
+    };
+#define NQ_KWG(D, S) (rt == 1 ? launch(gemm_kwave_group_kernel<D, S, 1>) : rt == 2 ? launch(gemm_kwave_group_kernel<D, S, 2>) : launch(gemm_kwave_group_kernel<D, S, 4>))
+    if (dtype == 0) return scaled ? NQ_KWG(0, true) : NQ_KWG(0, false);
+    return scaled ? NQ_KWG(1, true) : NQ_KWG(1, false);
+#undef NQ_KWG
+}
+
+int gemm_group_max() { return kGroupMax; }
+int gemm_group_max_tokens() { return kKwaveMaxTokens; }
 
 }  // namespace nq

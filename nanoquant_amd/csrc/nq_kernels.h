@@ -57,6 +57,13 @@ size_t gemm_scratch_bytes(int T, int K, int R);
 hipError_t gemm_onebit(int dtype, const void* x, const uint32_t* tiles, const void* s_in, const void* s_out,
                        void* y, float* scratch, int T, int K, int R, hipStream_t stream, const void* bias = nullptr);
 
+// Up to gemm_group_max() GEMMs of at most gemm_group_max_tokens() tokens in one launch (s_in: all or none).
+int gemm_group_max();
+int gemm_group_max_tokens();
+hipError_t gemm_onebit_group(int dtype, int count, const void* const* x, const uint32_t* const* tiles,
+                             const void* const* s_in, const void* const* s_out, const void* const* bias, void* const* y,
+                             int T, const int* K, const int* R, hipStream_t stream);
+
 // nq_util.hip
 hipError_t stream_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);
 hipError_t repack_words(const uint32_t* src, uint32_t* dst, size_t nwords, int src_order, int dst_order,

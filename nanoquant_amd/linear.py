@@ -300,6 +300,45 @@ class NanoQuantLinear(nn.Module):
         }
 
 
+def prefill_group(modules: Sequence[NanoQuantLinear], x) -> list:
+    """`[mod(x) for mod in modules]` for modules prepared with `_prepare_kernel("gemm")`, with the GEMMs of all
+    modules sharing launches (`ops.gemm_group_forward`): the projections of a decoder block that read the same
+    tokens (q/k/v, gate/up).  `x` is one tensor for all modules or a list of one tensor per module, 2-D or 3-D as
+    `forward` takes it (linear.py:106-141 of the reference launches each module by itself)."""
+    mods = list(modules)
+    if not mods:
+        return []
+    for mod in mods:
+        if not getattr(mod, "do_kernel_inference", False) or mod.kernel_type != "gemm":
+            raise ValueError("prefill_group needs modules prepared with _prepare_kernel('gemm', dtype)")
+        if mod.dtype != mods[0].dtype:
+            raise ValueError("all modules of a group must be prepared for the same dtype")
+    xs = [x] * len(mods) if isinstance(x, torch.Tensor) else list(x)
+    if len(xs) != len(mods):
+        raise ValueError("one input per module")
+    flat, shapes, cache = [], [], {}
+    for t in xs:
+        if t.ndim not in (2, 3):
+            raise ValueError(f"Expected 2D or 3D input tensor, got {t.ndim}D")
+        if id(t) not in cache:                 # a shared input is converted once
+            v = t if t.dtype == mods[0].dtype else t.to(mods[0].dtype)
+            cache[id(t)] = v.contiguous().view(-1, v.size(-1))
+        flat.append(cache[id(t)])
+        shapes.append(t.shape)
+    biases = []
+    for mod in mods:
+        b = mod.bias if (mod.kernel_path_bias and mod.bias is not None) else None
+        biases.append(None if b is None else (b if b.dtype == mod.dtype else b.to(mod.dtype)))
+    ys = ops.gemm_group_forward(flat, [(m.V_int8, m.U_int8, m.s1, m.s2, m.s3, m.workspace) for m in mods],
+                                biases if any(b is not None for b in biases) else None)
+    outs = []
+    for y, t, shape in zip(ys, xs, shapes):
+        if len(shape) == 3:
+            y = y.view(shape[0], shape[1], -1)
+        outs.append(y.to(t.dtype) if y.dtype != t.dtype else y)
+    return outs
+
+
 class MixtureOfRankLinear(nn.Module):
     """y = sum_t term_t(x): several binary low-rank terms with their own scale vectors."""
 

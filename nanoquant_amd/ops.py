@@ -300,6 +300,66 @@ def gemm_forward_with_bias(x, weight_u, weight_v, scale_g, scale_l, scale_h, wor
     return _gemm_nanoquant_forward(x, weight_u, weight_v, scale_g, scale_l, scale_h, workspace, bias)
 
 
+class NqGemmTerm(ctypes.Structure):
+    """Mirror of `nq_gemm_term` in include/nq_gfx950.h."""
+    _fields_ = [("x", ctypes.c_void_p), ("vt_tiles", ctypes.c_void_p), ("u_tiles", ctypes.c_void_p),
+                ("s_in", ctypes.c_void_p), ("s_mid", ctypes.c_void_p), ("s_out", ctypes.c_void_p),
+                ("bias", ctypes.c_void_p), ("h", ctypes.c_void_p), ("y", ctypes.c_void_p),
+                ("n", ctypes.c_int), ("r", ctypes.c_int), ("m", ctypes.c_int)]
+
+
+def gemm_group_forward(xs, terms, biases=None):
+    """Several `marlin_nanoquant_forward` calls on the same number of tokens in two launches instead of two per
+    call: `terms` is a list of argument tuples (weight_u, weight_v, scale_g, scale_l, scale_h, workspace) as that
+    op takes them after x; `xs` is one tensor [tokens, n] read by every term or a list of one tensor per term;
+    `biases` an optional list of [m] tensors / None.  Returns the list of outputs.  Up to 128 tokens the terms
+    share launches (a single linear leaves most of the device idle there); above, they run one by one.  The
+    reference launches every linear by itself (modules/linear.py:131-133)."""
+    lib = _lib.lib()
+    count = len(terms)
+    if count == 0:
+        return []
+    if isinstance(xs, torch.Tensor):
+        xs = [xs] * count
+    if len(xs) != count or (biases is not None and len(biases) != count):
+        raise RuntimeError("one x (and one bias entry) per term")
+    dt = _gemm_dtype(xs[0])
+    outs, keep, arr_items, nbytes = [], [], [], 0
+    for i, (x, term) in enumerate(zip(xs, terms)):
+        weight_u, weight_v, scale_g, scale_l, scale_h, workspace = term
+        bias = None if biases is None else biases[i]
+        if x.dtype != xs[0].dtype or x.dim() != 2 or x.size(0) != xs[0].size(0) or x.device != xs[0].device:
+            raise RuntimeError("all inputs of a group must be 2-D with the same token count, dtype and device")
+        t, r, n = _onebit_check(x, weight_u, scale_g, scale_l, workspace)
+        _check_gemm_tensor(x, "x")
+        _check_gemm_tensor(weight_u, "weight_u", torch.int32)
+        _check_gemm_tensor(weight_v, "weight_v", torch.int32)
+        for name, s in (("scale_g", scale_g), ("scale_l", scale_l), ("scale_h", scale_h)):
+            _check_gemm_tensor(s, name, x.dtype)
+        imm = torch.empty((t, r), dtype=x.dtype, device=x.device)
+        _, m, _ = _onebit_check(imm, weight_v, None, scale_h, workspace)
+        _check_bias(bias, m, x)
+        out = torch.empty((t, m), dtype=x.dtype, device=x.device)
+        outs.append(out)
+        keep.append(imm)
+        nbytes = max(nbytes, int(lib.nq_gemm_scratch_bytes(t, n, r)), int(lib.nq_gemm_scratch_bytes(t, r, m)))
+        pv = lambda ten: None if ten is None else ten.data_ptr()
+        arr_items.append(NqGemmTerm(pv(x), pv(weight_u), pv(weight_v), pv(scale_g), pv(scale_l), pv(scale_h), pv(bias),
+                                    pv(imm), pv(out), n, r, m))
+    tokens = xs[0].size(0)
+    if tokens == 0:
+        return outs
+    device = xs[0].device
+    group_max = int(lib.nq_gemm_group_max())
+    scratch = _scratch(nbytes, device)
+    with torch.cuda.device(device):
+        for lo in range(0, count, group_max):
+            part = arr_items[lo:lo + group_max]
+            arr = (NqGemmTerm * len(part))(*part)
+            _lib.check(lib.nq_gemm_nanoquant_group(arr, len(part), tokens, dt, _ptr(scratch), nbytes, _stream(device)))
+    return outs
+
+
 def gemv_mixture_forward(x, terms):
     """Sum of several binary low-rank terms sharing x.  terms: sequence of
     (scale_g, Ubits, scale_l | None, Vbits, scale_h) with the operand meaning of nanoquant_dyn_forward."""

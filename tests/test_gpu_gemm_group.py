@@ -1,0 +1,105 @@
+"""Grouped prefill: several linears on the same tokens sharing their launches (nq_gemm_nanoquant_group), against
+the dense definition and against the one-linear operator.  The reference launches each linear by itself
+(src/nanoquant/modules/linear.py:131-133, src/nanoquant/kernel/cuda/gemm.cpp:112-122)."""
+import numpy as np
+import pytest
+import torch
+
+import nanoquant_amd  # noqa: F401
+from nanoquant_amd import NanoQuantLinear, ops, packing, prefill_group
+from oracle import nq_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+TOL = {torch.float16: 2e-3, torch.bfloat16: 1e-2}
+
+
+def _cast(a, dtype):
+    return torch.from_numpy(np.ascontiguousarray(a).astype(np.float32)).to(dtype)
+
+
+def _term(dev, m, n, r, seed, dtype):
+    vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, seed)
+    si, sm, so = (_cast(a, dtype) for a in (s_in, s_mid, s_out))
+    packed = packing.marlin_nanoquant_packer(torch.from_numpy(vt).T.contiguous().to(dev),
+                                             torch.from_numpy(u).T.contiguous().to(dev), si.to(dev), sm.to(dev), so.to(dev))
+    ref = lambda x: oracle.layer_forward(x, vt, u, si.float().numpy(), sm.float().numpy(), so.float().numpy(), dtype=np.float32)
+    return packed, ref
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("tokens", [128, 77, 1, 200])
+def test_group_on_shared_tokens(dev, tokens, dtype):
+    # q, k, v-like: one input, different widths and ranks (one rank padded by the packer); 200 tokens takes the
+    # one-by-one branch of the same entry point
+    n = 1024
+    shapes = [(1024, 512), (256, 100), (320, 256), (2048, 768)]
+    terms = [_term(dev, m, n, r, 500 + i, dtype) for i, (m, r) in enumerate(shapes)]
+    x = _cast(oracle.synth_x(tokens, n, 9), dtype)
+    print(f"group shared tokens={tokens} {dtype}", flush=True)
+    ys = ops.gemm_group_forward(x.to(dev), [p for p, _ in terms])
+    torch.cuda.synchronize()
+    for (m, r), (packed, ref), y in zip(shapes, terms, ys):
+        assert y.shape == (tokens, m) and y.dtype == dtype
+        assert oracle.max_rel_err(y.float().cpu().numpy(), ref(x.float().numpy())) < TOL[dtype], (m, r)
+        single = torch.ops.binary_kernels.marlin_nanoquant_forward(x.to(dev), *packed)
+        if tokens <= 128:
+            assert torch.equal(y, single), (m, r)          # the same tiles in the same order: bit-identical
+        else:
+            assert torch.allclose(y.float(), single.float(), rtol=1e-2, atol=1e-3 * float(single.float().abs().max()))
+
+
+def test_group_with_own_inputs_bias_and_more_terms_than_one_launch_takes(dev):
+    dtype, tokens = torch.float16, 96
+    rng = np.random.default_rng(4)
+    shapes = [(256 + 32 * (i % 3), 512 if i % 2 else 768, 64 + 32 * i) for i in range(11)]   # 11 > 8 terms per launch
+    terms, xs, biases = [], [], []
+    for i, (m, n, r) in enumerate(shapes):
+        terms.append(_term(dev, m, n, r, 600 + i, dtype))
+        xs.append(_cast(oracle.synth_x(tokens, n, 700 + i), dtype))
+        biases.append(_cast(rng.normal(0, 0.05, m), dtype) if i % 2 == 0 else None)
+    ys = ops.gemm_group_forward([x.to(dev) for x in xs], [p for p, _ in terms],
+                                [None if b is None else b.to(dev) for b in biases])
+    torch.cuda.synchronize()
+    for (packed, ref), x, b, y in zip(terms, xs, biases, ys):
+        want = ref(x.float().numpy())
+        if b is not None:
+            want = want + b.float().numpy()[None, :]
+        assert oracle.max_rel_err(y.float().cpu().numpy(), want) < TOL[dtype]
+
+
+def test_group_rejects_mismatched_inputs(dev):
+    dtype = torch.float16
+    (p0, _), (p1, _) = _term(dev, 256, 512, 64, 1, dtype), _term(dev, 256, 768, 64, 2, dtype)
+    x512 = torch.zeros((64, 512), dtype=dtype, device=dev)
+    with pytest.raises(RuntimeError):
+        ops.gemm_group_forward(x512, [p0, p1])                               # second term reads 768 columns
+    with pytest.raises(RuntimeError):
+        ops.gemm_group_forward([x512, torch.zeros((32, 768), dtype=dtype, device=dev)], [p0, p1])   # token counts differ
+    with pytest.raises(RuntimeError):
+        ops.gemm_group_forward([x512], [p0, p1])
+    assert ops.gemm_group_forward(x512, []) == []
+
+
+@pytest.mark.parametrize("ndim", [2, 3])
+def test_prefill_group_of_modules(dev, ndim):
+    dtype, n = torch.float16, 1024
+    mods, refs = [], []
+    for i, (m, r) in enumerate([(1024, 512), (512, 256), (512, 300)]):
+        vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, 800 + i)
+        bias = np.random.default_rng(i).normal(0, 0.05, m).astype(np.float32)
+        f = lambda a: torch.from_numpy(a.astype(np.float32))
+        mod = NanoQuantLinear.from_factors(f(vt), f(u), f(s_in), f(s_mid), f(s_out), bias=f(bias), dtype=dtype).to(dev)
+        mod._prepare_kernel("gemm", dtype)
+        mod.kernel_path_bias = (i == 1)
+        mods.append(mod)
+    x = _cast(oracle.synth_x(2 * 60, n, 12), dtype).to(dev)
+    if ndim == 3:
+        x = x.view(2, 60, n)
+    ys = prefill_group(mods, x)
+    torch.cuda.synchronize()
+    for mod, y in zip(mods, ys):
+        single = mod(x)
+        assert y.shape == single.shape and torch.equal(y, single)
+    unprepared = NanoQuantLinear(256, 256, 64, dtype=dtype)
+    with pytest.raises(ValueError):
+        prefill_group([mods[0], unprepared], x)
