@@ -310,29 +310,34 @@ __device__ __forceinline__ void kwave_tile(const GemmArgs& a, int row_block, int
 
     // ---- add the four partial tiles through LDS (the slabs are free now) ----
     __syncthreads();
-    float* part = (float*)slabs;                                 // [RT][4][16][64] floats = RT x 16 KiB
+    // [RT][4][16] rows of kPartPitch floats; lane l of a row sits at (l & 31) + 33 * (l >> 5).  Pitch 66 and the
+    // odd offset of the upper half make both the stores here and the gathering loads below free of bank conflicts
+    // (the plain [..][64] layout put the 64 gathering lanes on 4 banks: 3600 conflict cycles per workgroup).
+    constexpr int kPartPitch = 66;
+    static_assert(RT * 4 * 16 * kPartPitch * sizeof(float) <= 4 * kSlabHalves * sizeof(uint16_t), "partial tiles must fit the slabs");
+    float* part = (float*)slabs;                                 // RT x 16.25 KiB <= the slabs' 68 KiB
 #pragma unroll
     for (int r = 0; r < RT; ++r)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) part[((r * 4 + wave) * 16 + v) * 64 + lane] = acc[r][v];
+        for (int v = 0; v < 16; ++v) part[((r * 4 + wave) * 16 + v) * kPartPitch + (lane & 31) + 33 * (lane >> 5)] = acc[r][v];
     __syncthreads();
     // Thread (token t, row octet o) of the first 128 threads sums the four partial values of 8 consecutive
     // rows and stores them as one 16-byte chunk.  Accumulator element v of lane l is token
     // 8*(v>>2) + 4*(l>>5) + (v&3), row l&31.
     if (threadIdx.x < 128) {
         const int t = threadIdx.x >> 2, o = threadIdx.x & 3;
-        const int v = 4 * (t >> 3) + (t & 3), l0 = 32 * ((t >> 2) & 1) + 8 * o;
+        const int v = 4 * (t >> 3) + (t & 3), l0 = 33 * ((t >> 2) & 1) + 8 * o;   // lanes 32 h + 8 o + j of the tile row
         const int tok = tok0 + t;
 #pragma unroll
         for (int r = 0; r < RT; ++r) {
             if (r >= ntiles) break;
             const int row0 = (rt + r) * 32 + 8 * o;
-            const float* pr = part + (size_t)r * 4 * 16 * 64;
+            const float* pr = part + (size_t)r * 4 * 16 * kPartPitch;
             float sums[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j)
-                sums[j] = (pr[(0 * 16 + v) * 64 + l0 + j] + pr[(1 * 16 + v) * 64 + l0 + j]) +
-                          (pr[(2 * 16 + v) * 64 + l0 + j] + pr[(3 * 16 + v) * 64 + l0 + j]);
+                sums[j] = (pr[(0 * 16 + v) * kPartPitch + l0 + j] + pr[(1 * 16 + v) * kPartPitch + l0 + j]) +
+                          (pr[(2 * 16 + v) * kPartPitch + l0 + j] + pr[(3 * 16 + v) * kPartPitch + l0 + j]);
             u32x4_t sc = {E::kOnePair, E::kOnePair, E::kOnePair, E::kOnePair};
             u32x4_t bs = {0u, 0u, 0u, 0u};
             if (a.s_out) sc = *(const u32x4_t*)(a.s_out + row0);
