@@ -252,16 +252,27 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         };
         if (ids.size() * 2 <= (size_t)nwg) {
             // Few stages, many workgroups: give every stage whole workgroups, so that no workgroup stages
-            // two input vectors in one phase.  A slice costs units * (rows + kSliceOverheadRows): staging the
-            // input vector takes about as long as the arithmetic of a dozen rows of the same width.  The
-            // workgroup counts n_s minimise the slowest slice, max_s units_s * (rows_s / n_s + overhead).
-            const double kSliceOverheadRows = 12.0;
+            // two input vectors in one phase.  A slice costs units * rows + fixed: staging the input vector takes
+            // about as long as the arithmetic of `overhead_rows` rows of the same width (a dozen at batch 1; every
+            // workgroup stages all batch rows while a row of signs costs the same for 16 columns as for one, so
+            // 48 at batch 8 and 64 at batch 16, from phase timelines of Llama-2-7B layers), and every further pass
+            // of an input too long to be staged at once costs the latency of one more staging round trip
+            // (2 us, 700 row units there).  The workgroup counts n_s minimise the slowest slice,
+            // max_s (units_s * rows_s / n_s + fixed_s).
+            const double overhead_rows = batch >= 16 ? 64.0 : batch >= 8 ? 48.0 : 12.0;
+            const double pass_cost = batch >= 8 ? 700.0 : 0.0;
+            const int chunk_cap = std::max(1, nq::stream_chunk_cap(dtype, batch, max_units));
+            std::vector<double> fixed(ids.size(), 0.0);
+            for (size_t k = 0; k < ids.size(); ++k) {
+                const int u = table[ids[k]].units;
+                fixed[k] = u * overhead_rows + ((u + chunk_cap - 1) / chunk_cap - 1) * pass_cost;
+            }
             std::vector<int> share(ids.size(), 1);
             auto needed = [&](double t) {       // workgroups needed for every slice to cost at most t
                 long long sum = 0;
                 for (size_t k = 0; k < ids.size(); ++k) {
                     const double u = table[ids[k]].units, r = table[ids[k]].rows;
-                    const double room = t - u * kSliceOverheadRows;
+                    const double room = t - fixed[k];
                     if (room <= 0) return (long long)nwg + 1;
                     long long n = (long long)((u * r + room - 1e-9) / room);
                     if (n < 1) n = 1;
@@ -272,7 +283,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
             };
             double lo = 0, hi = 0;
             for (size_t k = 0; k < ids.size(); ++k) {
-                const double t1 = (double)table[ids[k]].units * (table[ids[k]].rows + kSliceOverheadRows);
+                const double t1 = (double)table[ids[k]].units * table[ids[k]].rows + fixed[k];
                 if (t1 > hi) hi = t1;
             }
             for (int iter = 0; iter < 60; ++iter) {
@@ -282,7 +293,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
             int used = 0;
             for (size_t k = 0; k < ids.size(); ++k) {
                 const double u = table[ids[k]].units, r = table[ids[k]].rows;
-                const double room = hi - u * kSliceOverheadRows;
+                const double room = hi - fixed[k];
                 long long n = room > 0 ? (long long)((u * r + room - 1e-9) / room) : 1;
                 if (n < 1) n = 1;
                 if (n > table[ids[k]].rows) n = table[ids[k]].rows;
@@ -295,7 +306,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
                 double worst = -1;
                 for (size_t k = 0; k < ids.size(); ++k) {
                     if (share[k] >= table[ids[k]].rows) continue;
-                    const double t = table[ids[k]].units * ((double)table[ids[k]].rows / share[k] + kSliceOverheadRows);
+                    const double t = table[ids[k]].units * ((double)table[ids[k]].rows / share[k]) + fixed[k];
                     if (t > worst) { worst = t; best = k; }
                 }
                 if (best == ids.size()) break;

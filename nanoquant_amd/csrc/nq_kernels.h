@@ -43,6 +43,7 @@ struct RunSegment {
 };
 size_t stream_counter_bytes(int nstages);
 int stream_capacity(int dtype, int batch, int max_units);
+int stream_chunk_cap(int dtype, int batch, int max_units);
 int stream_row_granule(int dtype, int batch);
 hipError_t gemv_stream(int dtype, int batch, const RunStage* stages, int nstages, int nphases, const int* seg_index,
                        const RunSegment* segs, unsigned long long* counters, unsigned* status, int nwg, int max_units,

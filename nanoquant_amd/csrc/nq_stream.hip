@@ -50,7 +50,7 @@ constexpr int kCounterStride = 8;              // 64-bit words between sub-count
 // g = value / members_k needs no reset between launches and no atomic that returns a value; stage s
 // is complete in launch g when its sub-counters add up to (g+1) * seg_count(s).
 constexpr int kQ8Depth = 3;                    // items (2 KB of packed words each) in flight per wavefront, fp4 x fp8 path
-constexpr int kStreamLdsMax = 144 * 1024;      // staged activations + row accumulators, upper bound
+constexpr int kStreamLdsMax = 160 * 1024 - 512;   // staged activations + row accumulators: the LDS of a CU less the static variables
 
 // The packed words of one stage as a raw buffer: one 16-byte load per unit whatever the row alignment
 // (buffer loads need dword alignment only), zeros past the end of the matrix, and "no load" expressed
@@ -616,6 +616,16 @@ int stream_capacity(int dtype, int batch, int max_units) {
 #define NQ_CAP(D, B) capacity_of<D, B>(max_units)
     NQ_STREAM_DISPATCH(NQ_CAP)
 #undef NQ_CAP
+    return 0;
+}
+
+// Units of an input vector that are staged at once (longer inputs take several passes over the rows of a slice).
+int stream_chunk_cap(int dtype, int batch, int max_units) {
+    int cap = 0;
+    size_t lds = 0;
+#define NQ_CHUNK(D, B) (stream_lds_plan(B, StreamKernel<D, B>::kArith, max_units, &cap, &lds), cap)
+    NQ_STREAM_DISPATCH(NQ_CHUNK)
+#undef NQ_CHUNK
     return 0;
 }
 
