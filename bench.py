@@ -319,28 +319,29 @@ def main():
                                                "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
                 del g, x
             extra[f"prefill_{tokens}_tokens"] = gemm_lines
-        # ---- the 7 linears of the layer at 128 tokens sharing their launches (two per group of <= 8 terms) ----
+        # ---- the 7 linears of the layer sharing their launches (two per group of <= 8 terms) ----
         from nanoquant_amd import ops as nq_ops
         by_mn = {(m, n): (packed, r) for (m, n, r), packed in packed_by_shape.items()}
         group = [by_mn[(m, n)] for (_, m, n) in LLAMA2_7B_LAYER]
-        xs128 = {n: torch.randn(128, n, device=dev, generator=g2).to(torch.float16) for n in (4096, 11008)}
-        group_x = [xs128[n] for (_, _, n) in LLAMA2_7B_LAYER]
-        group_flops = sum(gemm_flops(m, n, by_mn[(m, n)][1], 128) for (_, m, n) in LLAMA2_7B_LAYER)
-        g = capture_rotation([lambda: nq_ops.gemm_group_forward(group_x, [pk for pk, _ in group])] * 5)
-        g.replay()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(5):
+        for tokens in (128, 512):
+            xs_t = {n: torch.randn(tokens, n, device=dev, generator=g2).to(torch.float16) for n in (4096, 11008)}
+            group_x = [xs_t[n] for (_, _, n) in LLAMA2_7B_LAYER]
+            group_flops = sum(gemm_flops(m, n, by_mn[(m, n)][1], tokens) for (_, m, n) in LLAMA2_7B_LAYER)
+            g = capture_rotation([lambda: nq_ops.gemm_group_forward(group_x, [pk for pk, _ in group])] * 5)
             g.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        us = e0.elapsed_time(e1) * 1e3 / 25
-        tf = group_flops / (us * 1e-6) / 1e12
-        extra["prefill_128_tokens_layer_grouped"] = {
-            "us_per_layer": round(us, 2), "TFLOPs": round(tf, 2), "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
-            "note": "7 linears of the layer in two launches (nq_gemm_nanoquant_group); q,k,v,o share one weight copy here"}
-        del g
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(5):
+                g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / 25
+            tf = group_flops / (us * 1e-6) / 1e12
+            extra[f"prefill_{tokens}_tokens_layer_grouped"] = {
+                "us_per_layer": round(us, 2), "TFLOPs": round(tf, 2), "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                "note": "7 linears of the layer in two launches (nq_gemm_nanoquant_group); q,k,v,o share one weight copy here"}
+            del g, xs_t, group_x
         # ---- cfg3: Qwen3-8B-like layer, every weight a sum of two terms (ranks 3:1, ~0.55 bpw), batch 1 ----
         qwen = (("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
                 ("gate", 12288, 4096), ("up", 12288, 4096), ("down", 4096, 12288))

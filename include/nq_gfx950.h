@@ -170,10 +170,12 @@ int nq_gemm_nanoquant_bias(const void* x, const uint32_t* vt_tiles, const uint32
 /* Several terms with the same token count in two launches instead of two per term: the first GEMMs of all
  * terms, then the second ones (the projections of a decoder block that read the same tokens: q/k/v, gate/up, or
  * independent linears of a layer).  Up to 128 tokens a single term cannot fill the device and is bound by launch
- * and load latencies; grouped, the same launches carry several times the work.  Above 128 tokens the call runs
- * the terms one after another (nq_gemm_nanoquant_bias) and needs their scratch: max over terms of
- * nq_gemm_scratch_bytes for both GEMMs, may be NULL up to 128 tokens.  count <= nq_gemm_group_max(); h and y of
- * different terms must not coincide.  No counterpart in the reference, which launches each linear by itself
+ * and load latencies; grouped, the same launches carry several times the work.  Above 128 tokens the group runs
+ * on 64-token block tiles whose workgroups walk the whole k of their term (no k-split, no scratch): together the
+ * terms fill the device where one term needs a k-split and a finish launch to do so.  Only when some terms have
+ * s_in and others do not does the call run the terms one after another (nq_gemm_nanoquant_bias); it then needs
+ * their scratch, max over terms of nq_gemm_scratch_bytes for both GEMMs (may be NULL otherwise).
+ * count <= nq_gemm_group_max(); h and y of different terms must not coincide.  No counterpart in the reference, which launches each linear by itself
  * (modules/linear.py:131-133). */
 typedef struct nq_gemm_term {
     const void* x;               /* [tokens, n] */

@@ -467,7 +467,7 @@ int nq_gemm_nanoquant_group(const nq_gemm_term* terms, int count, int tokens, in
     if (count == 0 || tokens == 0) return NQ_OK;
     if (!terms) return NQ_ERR_NULL;
     if (count > nq::gemm_group_max()) return NQ_ERR_SHAPE;
-    bool grouped = tokens <= nq::gemm_group_max_tokens();
+    bool grouped = true;
     for (int i = 0; i < count; ++i) {
         const nq_gemm_term& t = terms[i];
         if (t.n <= 0 || t.r <= 0 || t.m <= 0) return NQ_ERR_SHAPE;
@@ -480,7 +480,7 @@ int nq_gemm_nanoquant_group(const nq_gemm_term* terms, int count, int tokens, in
         for (int j = 0; j < i; ++j)
             if (terms[j].h == t.h || terms[j].y == t.y) return NQ_ERR_SHAPE;      // results would overwrite each other
     }
-    if (!grouped) {                              // many tokens: every GEMM fills the device by itself
+    if (!grouped) {                              // mixed kernel variants: one linear after the other
         for (int i = 0; i < count; ++i) {
             const nq_gemm_term& t = terms[i];
             int st = nq_gemm_nanoquant_bias(t.x, t.vt_tiles, t.u_tiles, t.s_in, t.s_mid, t.s_out, t.bias, t.h, t.y, scratch,

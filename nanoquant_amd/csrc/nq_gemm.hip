@@ -85,7 +85,7 @@ __device__ __forceinline__ void fetch_slab(const GemmArgs& a, int tok0, int k0, 
 // TT: 32-token tiles per wavefront, RT: 32-row tiles per wavefront, KS: k-values per LDS slab (128 or
 // 256).  A workgroup of 4 wavefronts covers 32*TT tokens x 128*RT rows.
 template <int DT, int TT, int RT, int KS, bool SPLIT, bool SCALED>
-__global__ __launch_bounds__(256) void gemm_onebit_kernel(GemmArgs a) {
+__device__ __forceinline__ void block_tile(const GemmArgs& a, int bx, int by, int bz) {
     using E = Elem<DT>;
     constexpr int kPitch = slab_pitch<KS>();
     constexpr int kSubs = kTileK / KS;       // slabs per weight tile
@@ -93,20 +93,11 @@ __global__ __launch_bounds__(256) void gemm_onebit_kernel(GemmArgs a) {
     extern __shared__ uint16_t slab[];       // [32*TT][kPitch], then the KS input scales of the slab
     uint16_t* scale_lds = slab + 32 * TT * kPitch;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    // Workgroups go to the 8 XCDs round-robin by linear id.  With the flat grid every XCD owns the token
-    // blocks y = xcd (mod 8), so the workgroups that share an activation slab also share an L2.
-    int bx = blockIdx.x, by = blockIdx.y;
-    if (a.xcd_gx > 0) {
-        const int slot = blockIdx.x >> 3;
-        by = (slot / a.xcd_gx) * 8 + (blockIdx.x & 7);
-        bx = slot % a.xcd_gx;
-        if (by * (32 * TT) >= a.T) return;
-    }
     const int rt = (bx * 4 + wave) * RT;           // first of the RT 32-row tiles of this wavefront
     const bool have_rows = rt * 32 < a.R;
     const int ntiles = min(RT, a.R / 32 - rt);     // R % 32 == 0
     const int tok0 = by * (32 * TT);
-    const int kt_begin = blockIdx.z * a.ktiles_per_split;
+    const int kt_begin = bz * a.ktiles_per_split;
     const int kt_end = min(kt_begin + a.ktiles_per_split, a.ktiles);
 
     float16_t acc[RT][TT];
@@ -212,6 +203,20 @@ __global__ __launch_bounds__(256) void gemm_onebit_kernel(GemmArgs a) {
             }
         }
     }
+}
+
+template <int DT, int TT, int RT, int KS, bool SPLIT, bool SCALED>
+__global__ __launch_bounds__(256) void gemm_onebit_kernel(GemmArgs a) {
+    // Workgroups go to the 8 XCDs round-robin by linear id.  With the flat grid every XCD owns the token
+    // blocks y = xcd (mod 8), so the workgroups that share an activation slab also share an L2.
+    int bx = blockIdx.x, by = blockIdx.y;
+    if (a.xcd_gx > 0) {
+        const int slot = blockIdx.x >> 3;
+        by = (slot / a.xcd_gx) * 8 + (blockIdx.x & 7);
+        bx = slot % a.xcd_gx;
+        if (by * (32 * TT) >= a.T) return;
+    }
+    block_tile<DT, TT, RT, KS, SPLIT, SCALED>(a, bx, by, blockIdx.z);
 }
 
 // Few tokens: one 32-row x 32-token output tile per workgroup, the four wavefronts split k among them
@@ -381,6 +386,45 @@ __global__ __launch_bounds__(256) void gemm_kwave_group_kernel(GemmGroup g) {
     kwave_tile<DT, SCALED, RT>(a, local % gx, local / gx);
 }
 
+// The same for more than 128 tokens: block tiles of 64 tokens x 128*RT rows, every workgroup walks the whole k of
+// its problem (no k-split, no scratch).  Workgroups go to the 8 XCDs round-robin by id and first[p] is a multiple
+// of 8, so (id - first[p]) mod 8 is the XCD; the mapping keeps the workgroups that share an activation slab on one
+// XCD (one L2) where the number of token blocks gy allows it: gy a multiple of 8 (or large): XCD = token block
+// mod 8; gy = 1, 2, 4: XCD x owns token block x mod gy and every (8/gy)-th row block; otherwise row blocks run
+// fastest.  a.xcd_gx holds the number of row blocks; group_blocks() is the host's count for the same mapping.
+__host__ __device__ inline int group_mode(int gy) { return (gy % 8 == 0 || gy >= 32) ? 0 : (8 % gy == 0) ? 1 : 2; }
+static int group_blocks(int gx, int gy) {
+    const int mode = group_mode(gy);
+    if (mode == 0) return gx * ((gy + 7) / 8 * 8);
+    if (mode == 1) { const int sub = 8 / gy; return (gx + sub - 1) / sub * 8; }
+    return (gx * gy + 7) / 8 * 8;
+}
+template <int DT, int RT, bool SCALED>
+__global__ __launch_bounds__(256) void gemm_block_group_kernel(GemmGroup g) {
+    const int b = blockIdx.x;
+    int p = 0;
+    while (p + 1 < g.count && b >= g.first[p + 1]) ++p;
+    const GemmArgs a = g.a[p];
+    const int local = b - g.first[p];
+    const int gx = a.xcd_gx, gy = (a.T + 63) >> 6;
+    const int mode = group_mode(gy);
+    int bx, by;
+    if (mode == 0) {
+        const int slot = local >> 3;
+        by = (slot / gx) * 8 + (local & 7);
+        bx = slot % gx;
+    } else if (mode == 1) {
+        const int sub = 8 / gy, xcd = local & 7;
+        by = xcd % gy;
+        bx = (local >> 3) * sub + xcd / gy;
+    } else {
+        bx = local % gx;
+        by = local / gx;
+    }
+    if (bx >= gx || by >= gy) return;
+    block_tile<DT, 2, RT, kTileK, false, SCALED>(a, bx, by, 0);
+}
+
 // Scales, converts and stores the accumulated sums, and puts the accumulator back to zero: the scratch
 // is zero on entry of every GEMM call and zero again when the call has finished.
 template <int DT>
@@ -542,12 +586,58 @@ hipError_t gemm_onebit(int dtype, const void* x, const uint32_t* tiles, const vo
     return p.rt == 2 ? launch_gemm<1, 2, 2, 256>(a, p, stream) : launch_gemm<1, 2, 1, 256>(a, p, stream);
 }
 
-// Few-token GEMMs of several problems in one launch; every problem: K % 256 == 0, R % 32 == 0, tokens <=
-// kKwaveMaxTokens, and either all have input scales or none (checked by the caller).
+// More than kKwaveMaxTokens tokens: one launch of gemm_block_group_kernel.  Two row tiles per wavefront halve the
+// LDS reads per MFMA and are taken once that still leaves two workgroups for every CU.
+static hipError_t gemm_block_group(int dtype, int count, const void* const* x, const uint32_t* const* tiles,
+                                   const void* const* s_in, const void* const* s_out, const void* const* bias,
+                                   void* const* y, int T, const int* K, const int* R, hipStream_t stream) {
+    const int gy = (T + 63) / 64;
+    long wide = 0;
+    for (int p = 0; p < count; ++p) wide += (long)((R[p] + 255) / 256) * gy;
+    const int rt = wide >= 512 ? 2 : 1;
+    // Longest k first: the workgroups that run longest start first, the short ones fill in behind them.
+    int order[kGroupMax];
+    for (int p = 0; p < count; ++p) order[p] = p;
+    for (int i = 1; i < count; ++i)
+        for (int j = i; j > 0 && K[order[j]] > K[order[j - 1]]; --j) { const int t = order[j]; order[j] = order[j - 1]; order[j - 1] = t; }
+    GemmGroup g;
+    g.count = count;
+    int blocks = 0;
+    for (int p = 0; p < kGroupMax; ++p) {
+        const int q = order[p < count ? p : count - 1];
+        GemmArgs& a = g.a[p];
+        a.x = x[q]; a.tiles = (const uint4*)tiles[q];
+        a.s_in = (const uint16_t*)(s_in ? s_in[q] : nullptr); a.s_out = (const uint16_t*)(s_out ? s_out[q] : nullptr);
+        a.bias = (const uint16_t*)(bias ? bias[q] : nullptr);
+        a.y = y[q]; a.acc = nullptr;
+        a.T = T; a.K = K[q]; a.R = R[q];
+        a.ktiles = K[q] / kTileK; a.ktiles_per_split = a.ktiles;
+        a.xcd_gx = (R[q] + 128 * rt - 1) / (128 * rt);
+        g.first[p] = blocks;
+        if (p < count) blocks += group_blocks(a.xcd_gx, gy);
+    }
+    g.first[kGroupMax] = blocks;
+    for (int p = count; p < kGroupMax; ++p) g.first[p] = blocks;
+    const bool scaled = g.a[0].s_in != nullptr;
+    const size_t lds = ((size_t)64 * slab_pitch<kTileK>() + kTileK) * sizeof(uint16_t);
+    auto launch = [&](auto kern) -> hipError_t {
+        hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds, stream, g);
+        return hipGetLastError();
+    };
+#define NQ_BG(D, S) (rt == 1 ? launch(gemm_block_group_kernel<D, 1, S>) : launch(gemm_block_group_kernel<D, 2, S>))
+    if (dtype == 0) return scaled ? NQ_BG(0, true) : NQ_BG(0, false);
+    return scaled ? NQ_BG(1, true) : NQ_BG(1, false);
+#undef NQ_BG
+}
+
+// GEMMs of several problems on the same token count in one launch; every problem: K % 256 == 0, R % 32 == 0, and
+// either all have input scales or none (checked by the caller).  Up to kKwaveMaxTokens tokens the few-token
+// tiles, above them block tiles.
 hipError_t gemm_onebit_group(int dtype, int count, const void* const* x, const uint32_t* const* tiles,
                              const void* const* s_in, const void* const* s_out, const void* const* bias, void* const* y,
                              int T, const int* K, const int* R, hipStream_t stream) {
-    if (count < 1 || count > kGroupMax || T > kKwaveMaxTokens) return hipErrorInvalidValue;
+    if (count < 1 || count > kGroupMax) return hipErrorInvalidValue;
+    if (T > kKwaveMaxTokens) return gemm_block_group(dtype, count, x, tiles, s_in, s_out, bias, y, T, K, R, stream);
     const int gy = (T + 31) / 32;
     int rt = 4;                                  // widest row blocks that still leave two workgroups per CU
     for (; rt > 1; rt /= 2) {

@@ -58,7 +58,8 @@ size_t gemm_scratch_bytes(int T, int K, int R);
 hipError_t gemm_onebit(int dtype, const void* x, const uint32_t* tiles, const void* s_in, const void* s_out,
                        void* y, float* scratch, int T, int K, int R, hipStream_t stream, const void* bias = nullptr);
 
-// Up to gemm_group_max() GEMMs of at most gemm_group_max_tokens() tokens in one launch (s_in: all or none).
+// Up to gemm_group_max() GEMMs on the same token count in one launch (s_in: all or none); few-token tiles up to
+// gemm_group_max_tokens() tokens, block tiles above.
 int gemm_group_max();
 int gemm_group_max_tokens();
 hipError_t gemm_onebit_group(int dtype, int count, const void* const* x, const uint32_t* const* tiles,

@@ -27,10 +27,10 @@ def _term(dev, m, n, r, seed, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("tokens", [128, 77, 1, 200])
+@pytest.mark.parametrize("tokens", [128, 77, 1, 200, 320, 512])
 def test_group_on_shared_tokens(dev, tokens, dtype):
-    # q, k, v-like: one input, different widths and ranks (one rank padded by the packer); 200 tokens takes the
-    # one-by-one branch of the same entry point
+    # q, k, v-like: one input, different widths and ranks (one rank padded by the packer); above 128 tokens the
+    # group runs on block tiles (64 tokens; 200 leaves a ragged last block), every workgroup walking the whole k
     n = 1024
     shapes = [(1024, 512), (256, 100), (320, 256), (2048, 768)]
     terms = [_term(dev, m, n, r, 500 + i, dtype) for i, (m, r) in enumerate(shapes)]
