@@ -319,7 +319,7 @@ def main():
                                                "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
                 del g, x
             extra[f"prefill_{tokens}_tokens"] = gemm_lines
-        # ---- the 7 linears of the layer sharing their launches (two per group of <= 8 terms) ----
+        # ---- the 7 linears of the layer sharing their launches (two per group of <= 16 terms) ----
         from nanoquant_amd import ops as nq_ops
         by_mn = {(m, n): (packed, r) for (m, n, r), packed in packed_by_shape.items()}
         group = [by_mn[(m, n)] for (_, m, n) in LLAMA2_7B_LAYER]
@@ -374,6 +374,45 @@ def main():
             "us_per_layer": round(ms_q * 1e3, 3), "GBps": round(q_bytes / (ms_q * 1e-3) / 1e9, 2),
             "note": "14 terms in one launch, second terms add onto the fp32 output of the first inside the kernel"}
         del q_lists
+
+        # ---- cfg3 at 128 tokens: the 14 terms of the layer in shared launches, the two terms of a weight summed ----
+        q_packed = {}
+        for (_, m, n) in qwen:
+            if (m, n) in q_packed:
+                continue
+            pair = []
+            for r in mixture_ranks(m, n):
+                v = (torch.randint(0, 2, (n, r), device=dev, generator=gq, dtype=torch.int8) * 2 - 1)
+                u = (torch.randint(0, 2, (r, m), device=dev, generator=gq, dtype=torch.int8) * 2 - 1)
+                sc = lambda k: (torch.randn(k, device=dev, generator=gq).abs() * 0.02 + 1e-3).to(torch.float16)
+                pair.append(packing.marlin_nanoquant_packer(v, u, sc(n), sc(r), sc(m)))
+                del v, u
+            q_packed[(m, n)] = pair
+        xq128 = {n: torch.randn(128, n, device=dev, generator=gq).to(torch.float16) for n in (4096, 12288)}
+        q_terms = [t for (_, m, n) in qwen for t in q_packed[(m, n)]]
+        q_xs = [xq128[n] for (_, m, n) in qwen for _ in range(2)]
+        q_flops = sum(gemm_flops(m, n, r, 128) for (_, m, n) in qwen for r in mixture_ranks(m, n))
+
+        def qwen_prefill():
+            ys = nq_ops.gemm_group_forward(q_xs, q_terms)
+            return [ys[2 * i] + ys[2 * i + 1] for i in range(len(qwen))]
+
+        g = capture_rotation([qwen_prefill] * 5)
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(5):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / 25
+        tf = q_flops / (us * 1e-6) / 1e12
+        extra["cfg3_qwen3_8b_two_term_layer_128_tokens"] = {
+            "us_per_layer": round(us, 2), "TFLOPs": round(tf, 2), "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+            "note": "14 terms in two grouped launches (first GEMMs, second GEMMs) plus 7 adds of the term pairs; "
+                    "flops at the nominal ranks"}
+        del g, q_packed, q_terms
 
         # ---- cfg4: Llama-3-70B-shaped weight stream, 80 layers x 7 linears in one launch ----
         llama70 = (("q", 8192, 8192), ("k", 1024, 8192), ("v", 1024, 8192), ("o", 8192, 8192),

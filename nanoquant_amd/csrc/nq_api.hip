@@ -489,8 +489,11 @@ int nq_gemm_nanoquant_group(const nq_gemm_term* terms, int count, int tokens, in
         }
         return NQ_OK;
     }
-    const void* x[8]; const uint32_t* w[8]; const void* si[8]; const void* so[8]; const void* bs[8]; void* out[8];
-    int K[8], R[8];
+    constexpr int kMax = 16;                     // >= nq::gemm_group_max(), checked above
+    static_assert(kMax >= 16, "group arrays");
+    const void* x[kMax]; const uint32_t* w[kMax]; const void* si[kMax]; const void* so[kMax]; const void* bs[kMax]; void* out[kMax];
+    int K[kMax], R[kMax];
+    if (count > kMax) return NQ_ERR_SHAPE;
     for (int i = 0; i < count; ++i) {
         const nq_gemm_term& t = terms[i];
         x[i] = t.x; w[i] = t.vt_tiles; si[i] = t.s_in; so[i] = t.s_mid; bs[i] = nullptr; out[i] = t.h; K[i] = t.n; R[i] = t.r;

@@ -368,7 +368,7 @@ __global__ __launch_bounds__(256) void gemm_kwave_kernel(GemmArgs a) {
 // Several GEMMs of the few-token kind in one launch (the projections that share a layer's tokens): workgroup b
 // belongs to the problem p with first[p] <= b < first[p + 1]; inside a problem the row blocks run fastest, so
 // neighbours share an activation slab.  All problems have the same token count.
-constexpr int kGroupMax = 8;
+constexpr int kGroupMax = 16;   // 16 problems of 80 bytes: well inside the 4 KB of kernel arguments
 struct GemmGroup {
     GemmArgs a[kGroupMax];
     int first[kGroupMax + 1];

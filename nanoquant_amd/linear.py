@@ -300,23 +300,31 @@ class NanoQuantLinear(nn.Module):
         }
 
 
-def prefill_group(modules: Sequence[NanoQuantLinear], x) -> list:
+def prefill_group(modules: Sequence, x) -> list:
     """`[mod(x) for mod in modules]` for modules prepared with `_prepare_kernel("gemm")`, with the GEMMs of all
     modules sharing launches (`ops.gemm_group_forward`): the projections of a decoder block that read the same
     tokens (q/k/v, gate/up).  `x` is one tensor for all modules or a list of one tensor per module, 2-D or 3-D as
-    `forward` takes it (linear.py:106-141 of the reference launches each module by itself)."""
-    mods = list(modules)
-    if not mods:
+    `forward` takes it (linear.py:106-141 of the reference launches each module by itself).  A
+    `MixtureOfRankLinear` among the modules contributes all its terms to the shared launches; its output is the
+    sum of their outputs."""
+    entries = list(modules)
+    if not entries:
         return []
+    xs_in = [x] * len(entries) if isinstance(x, torch.Tensor) else list(x)
+    if len(xs_in) != len(entries):
+        raise ValueError("one input per module")
+    mods, xs, owner = [], [], []               # one entry per term; owner = index of the module it belongs to
+    for i, (entry, t) in enumerate(zip(entries, xs_in)):
+        for mod in (entry.terms if isinstance(entry, MixtureOfRankLinear) else (entry,)):
+            mods.append(mod)
+            xs.append(t)
+            owner.append(i)
     for mod in mods:
         if not getattr(mod, "do_kernel_inference", False) or mod.kernel_type != "gemm":
             raise ValueError("prefill_group needs modules prepared with _prepare_kernel('gemm', dtype)")
         if mod.dtype != mods[0].dtype:
             raise ValueError("all modules of a group must be prepared for the same dtype")
-    xs = [x] * len(mods) if isinstance(x, torch.Tensor) else list(x)
-    if len(xs) != len(mods):
-        raise ValueError("one input per module")
-    flat, shapes, cache = [], [], {}
+    flat, cache = [], {}
     for t in xs:
         if t.ndim not in (2, 3):
             raise ValueError(f"Expected 2D or 3D input tensor, got {t.ndim}D")
@@ -324,18 +332,20 @@ def prefill_group(modules: Sequence[NanoQuantLinear], x) -> list:
             v = t if t.dtype == mods[0].dtype else t.to(mods[0].dtype)
             cache[id(t)] = v.contiguous().view(-1, v.size(-1))
         flat.append(cache[id(t)])
-        shapes.append(t.shape)
     biases = []
     for mod in mods:
         b = mod.bias if (mod.kernel_path_bias and mod.bias is not None) else None
         biases.append(None if b is None else (b if b.dtype == mod.dtype else b.to(mod.dtype)))
     ys = ops.gemm_group_forward(flat, [(m.V_int8, m.U_int8, m.s1, m.s2, m.s3, m.workspace) for m in mods],
                                 biases if any(b is not None for b in biases) else None)
-    outs = []
-    for y, t, shape in zip(ys, xs, shapes):
-        if len(shape) == 3:
-            y = y.view(shape[0], shape[1], -1)
-        outs.append(y.to(t.dtype) if y.dtype != t.dtype else y)
+    outs = [None] * len(entries)
+    for y, i in zip(ys, owner):
+        outs[i] = y if outs[i] is None else outs[i] + y
+    for i, t in enumerate(xs_in):
+        y = outs[i]
+        if t.ndim == 3:
+            y = y.view(t.shape[0], t.shape[1], -1)
+        outs[i] = y.to(t.dtype) if y.dtype != t.dtype else y
     return outs
 
 
@@ -367,6 +377,8 @@ class MixtureOfRankLinear(nn.Module):
             y = ops.gemv_mixture_forward(
                 xk, [(t.scale_pre, t.V_int8, t.scale_mid, t.U_int8, t.scale_post) for t in self.terms])
             return y.to(orig_dtype) if y.dtype != orig_dtype else y
+        if self.kernel_type == "gemm":            # all terms in shared launches, summed afterwards
+            return prefill_group([self], x)[0]
         y = self.terms[0](x)
         for t in self.terms[1:]:
             y = y + t(x)

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import nanoquant_amd  # noqa: F401
-from nanoquant_amd import NanoQuantLinear, ops, packing, prefill_group
+from nanoquant_amd import MixtureOfRankLinear, NanoQuantLinear, ops, packing, prefill_group
 from oracle import nq_oracle as oracle
 
 pytestmark = pytest.mark.gpu
@@ -51,7 +51,7 @@ def test_group_on_shared_tokens(dev, tokens, dtype):
 def test_group_with_own_inputs_bias_and_more_terms_than_one_launch_takes(dev):
     dtype, tokens = torch.float16, 96
     rng = np.random.default_rng(4)
-    shapes = [(256 + 32 * (i % 3), 512 if i % 2 else 768, 64 + 32 * i) for i in range(11)]   # 11 > 8 terms per launch
+    shapes = [(256 + 32 * (i % 3), 512 if i % 2 else 768, 64 + 32 * i) for i in range(19)]   # 19 > 16 terms per launch
     terms, xs, biases = [], [], []
     for i, (m, n, r) in enumerate(shapes):
         terms.append(_term(dev, m, n, r, 600 + i, dtype))
@@ -103,3 +103,30 @@ def test_prefill_group_of_modules(dev, ndim):
     unprepared = NanoQuantLinear(256, 256, 64, dtype=dtype)
     with pytest.raises(ValueError):
         prefill_group([mods[0], unprepared], x)
+
+
+@pytest.mark.parametrize("tokens", [96, 200])
+def test_prefill_group_with_a_mixture_module(dev, tokens):
+    # a two-term weight and a plain linear on the same tokens: all three terms share the launches, the mixture's
+    # output is the sum of its terms (the dense definition of a sum of low-rank terms)
+    dtype, n = torch.float16, 768
+    f = lambda a: torch.from_numpy(a.astype(np.float32))
+    make = lambda m, r, seed: (oracle.synth_term(m, n, r, seed))
+    t0, t1, t2 = make(512, 192, 820), make(512, 64, 821), make(1024, 256, 822)
+    mods = [NanoQuantLinear.from_factors(*(f(a) for a in t), dtype=dtype).to(dev) for t in (t0, t1, t2)]
+    mix = MixtureOfRankLinear(mods[:2])
+    mix._prepare_kernel("gemm", dtype)
+    mods[2]._prepare_kernel("gemm", dtype)
+    x = oracle.synth_x(tokens, n, 13)
+    xt = _cast(x, dtype).to(dev)
+    print(f"group with mixture tokens={tokens}", flush=True)
+    y_mix, y_plain = prefill_group([mix, mods[2]], xt)
+    y_fwd = mix(xt)
+    torch.cuda.synchronize()
+    xf = xt.float().cpu().numpy()
+    ref_mix = oracle.mixture_forward(xf.astype(np.float64), [t0, t1], dtype=np.float64)
+    ref_plain = oracle.layer_forward(xf.astype(np.float64), *t2, dtype=np.float64)
+    assert y_mix.shape == (tokens, 512) and y_plain.shape == (tokens, 1024)
+    assert oracle.max_rel_err(y_mix.float().cpu().numpy(), ref_mix) < TOL[dtype]
+    assert oracle.max_rel_err(y_fwd.float().cpu().numpy(), ref_mix) < TOL[dtype]
+    assert oracle.max_rel_err(y_plain.float().cpu().numpy(), ref_plain) < TOL[dtype]
