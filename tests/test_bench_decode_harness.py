@@ -76,3 +76,14 @@ def test_tiny_sweep_writes_rows_and_aggregates(dev, tmp_path, kind):
         assert float(r["decode_tps_total"]) > 0 and r["quant_kernel_type"] == kind
         assert int(r["decode_tokens_total"]) in (4, 8, 16)
     assert float(rows[2]["prefill_time_s"]) > 0
+
+
+def test_prefill_harness_rank_and_gpu_requirement():
+    import torch
+    from nanoquant_amd import bench_prefill as bp
+    assert bp.prefill_rank(4096, 4096, 1.0) == 2048
+    assert bp.prefill_rank(11008, 4096, 1.0) == 2985
+    assert bp.prefill_rank(64, 64, 0.1) == 32
+    if not torch.cuda.is_available():
+        with pytest.raises(RuntimeError, match="needs a GPU"):
+            bp.run(["--model_shape", "tiny", "--tokens", "32"])

@@ -130,3 +130,11 @@ def test_prefill_group_with_a_mixture_module(dev, tokens):
     assert oracle.max_rel_err(y_mix.float().cpu().numpy(), ref_mix) < TOL[dtype]
     assert oracle.max_rel_err(y_fwd.float().cpu().numpy(), ref_mix) < TOL[dtype]
     assert oracle.max_rel_err(y_plain.float().cpu().numpy(), ref_plain) < TOL[dtype]
+
+
+def test_prefill_harness_on_a_tiny_layer(dev):
+    from nanoquant_amd import bench_prefill
+    rows = bench_prefill.run(["--model_shape", "tiny", "--tokens", "32,160", "--iters", "2", "--reps", "2"])
+    assert [r["tokens"] for r in rows] == [32, 160]
+    for r in rows:
+        assert r["one_by_one"]["us_per_layer"] > 0 and r["grouped"]["us_per_layer"] > 0
