@@ -323,7 +323,7 @@ def main():
         from nanoquant_amd import ops as nq_ops
         by_mn = {(m, n): (packed, r) for (m, n, r), packed in packed_by_shape.items()}
         group = [by_mn[(m, n)] for (_, m, n) in LLAMA2_7B_LAYER]
-        for tokens in (128, 512):
+        for tokens in (16, 128, 512):
             xs_t = {n: torch.randn(tokens, n, device=dev, generator=g2).to(torch.float16) for n in (4096, 11008)}
             group_x = [xs_t[n] for (_, _, n) in LLAMA2_7B_LAYER]
             group_flops = sum(gemm_flops(m, n, by_mn[(m, n)][1], tokens) for (_, m, n) in LLAMA2_7B_LAYER)
@@ -341,6 +341,10 @@ def main():
             extra[f"prefill_{tokens}_tokens_layer_grouped"] = {
                 "us_per_layer": round(us, 2), "TFLOPs": round(tf, 2), "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
                 "note": "7 linears of the layer in two launches (nq_gemm_nanoquant_group); q,k,v,o share one weight copy here"}
+            if tokens == 16:
+                extra[f"prefill_{tokens}_tokens_layer_grouped"]["note"] += (
+                    "; the same 16 rows as extra.batch16 on the prefill kernels (kernel_type='gemm' + prefill_group), "
+                    "weights warm in cache here, rotating copies there")
             del g, xs_t, group_x
         # ---- cfg3: Qwen3-8B-like layer, every weight a sum of two terms (ranks 3:1, ~0.55 bpw), batch 1 ----
         qwen = (("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
