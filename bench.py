@@ -341,11 +341,26 @@ def main():
             extra[f"prefill_{tokens}_tokens_layer_grouped"] = {
                 "us_per_layer": round(us, 2), "TFLOPs": round(tf, 2), "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
                 "note": "7 linears of the layer in two launches (nq_gemm_nanoquant_group); q,k,v,o share one weight copy here"}
+            del g
             if tokens == 16:
-                extra[f"prefill_{tokens}_tokens_layer_grouped"]["note"] += (
-                    "; the same 16 rows as extra.batch16 on the prefill kernels (kernel_type='gemm' + prefill_group), "
-                    "weights warm in cache here, rotating copies there")
-            del g, xs_t, group_x
+                # the same 16 rows as extra.batch16, on the prefill kernels and with cold weights as there: every
+                # linear of every rotation step reads its own copy of the packed tiles (args.copies x 7 clones)
+                cold = [[tuple(t.clone() for t in pk) for pk, _ in group] for _ in range(args.copies)]
+                g = capture_rotation([(lambda terms=terms: nq_ops.gemm_group_forward(group_x, terms)) for terms in cold])
+                g.replay()
+                torch.cuda.synchronize()
+                e0.record()
+                for _ in range(4):
+                    g.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                us_cold = e0.elapsed_time(e1) * 1e3 / (4 * args.copies)
+                extra["batch16_on_prefill_kernels"] = {
+                    "us_per_layer": round(us_cold, 2), "GBps": round(layer_bytes(16) / (us_cold * 1e-6) / 1e9, 2),
+                    "note": "16 rows through kernel_type='gemm' + grouped launches (two per layer), rotating weight copies "
+                            "as in the decode legs; GB/s counts the decode path's algorithmic bytes"}
+                del g, cold
+            del xs_t, group_x
         # ---- cfg3: Qwen3-8B-like layer, every weight a sum of two terms (ranks 3:1, ~0.55 bpw), batch 1 ----
         qwen = (("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
                 ("gate", 12288, 4096), ("up", 12288, 4096), ("down", 4096, 12288))
