@@ -136,7 +136,25 @@ __global__ __launch_bounds__(256) void gemv_stage_kernel(StageArgs a) {
 }
 
 // ---- host side --------------------------------------------------------------------------------
-static int pick_group_log2(int units) {
+static int pick_group_log2(int units, int rows, int batch) {
+    if (batch == 1) {
+        // One batch row is bound by how many bytes are in flight: a small lane group puts many rows into a workgroup
+        // and leaves few workgroups (rank 3008 x 11008 columns: 86 units, 8 lanes per row, 94 workgroups on 256 CUs,
+        // 14 us).  Take the lane group that maximises (share of lanes on real data) x (workgroups, up to what the
+        // device keeps resident), the smaller group on ties (Llama-2-7B layer: 80 -> 74 us; with more batch rows the
+        // arithmetic per workgroup weighs more and the rule below stays faster).
+        int best = 0;
+        double best_score = -1.0;
+        for (int gl = 0; gl <= 6; ++gl) {
+            const int G = 1 << gl;
+            const int passes = (units + G - 1) / G;
+            double grid = (double)rows / (4 * (kWave / G));
+            if (grid > 1536.0) grid = 1536.0;
+            const double score = (double)units / (double)(G * passes) * grid;
+            if (score > best_score * 1.001) { best_score = score; best = gl; }
+        }
+        return best;
+    }
     // Largest lane group whose last pass still keeps >= 90% of the lanes on real data.
     int best = 0;
     for (int gl = 6; gl >= 0; --gl) {
@@ -218,7 +236,7 @@ hipError_t gemv_stage(int dtype, bool first, const uint32_t* bits, const void* i
         cap = (cap - 1) & ~1;                                       // even, so that cap|1 <= budget
         if (cap > kXsumStride - 2) cap = kXsumStride - 2;
         a.chunk_units = a.units < cap ? a.units : cap;
-        a.group_log2 = pick_group_log2(a.chunk_units);
+        a.group_log2 = pick_group_log2(a.chunk_units, rows, piece);
         a.in = (const char*)in + (size_t)done * in_stride * in_elt;
         a.out = (char*)out + (size_t)done * out_stride * (out_f32 ? 4 : 2);
         a.addend = addend ? addend + (size_t)done * out_stride : nullptr;
