@@ -64,6 +64,7 @@ class SynthLinear:
         if self.rp > r:
             self.s_mid[r:] = 0
         self._tiled = None
+        self._scales_alt = None
 
     def runlist_words(self, keep_row_major=True):
         """(first-stage words, second-stage words) in the tile order that run lists read fastest: a fixed
@@ -78,10 +79,19 @@ class SynthLinear:
     def add_to(self, rl, x, keep_row_major=True, **kw):
         """Tile order for the HBM-bound small batches; batch >= 8 runs on 16-bit MFMA operands, is bound by its
         arithmetic and measures 3 % slower on tiled words, so it reads the row-major ones."""
+        s_in, s_mid, s_out = self.scales_as(x.dtype)
         if rl.batch > 4:
-            return rl.add(x, self.s_in, self.vt_bits, self.s_mid, self.u_bits, self.s_out, **kw)
+            return rl.add(x, s_in, self.vt_bits, s_mid, self.u_bits, s_out, **kw)
         vt, u = self.runlist_words(keep_row_major)
-        return rl.add(x, self.s_in, vt, self.s_mid, u, self.s_out, tiled=True, **kw)
+        return rl.add(x, s_in, vt, s_mid, u, s_out, tiled=True, **kw)
+
+    def scales_as(self, dtype):
+        """The scale vectors in the activation type (drawn as fp16; converted once for bf16 runs)."""
+        if dtype == self.s_in.dtype:
+            return self.s_in, self.s_mid, self.s_out
+        if self._scales_alt is None or self._scales_alt[0].dtype != dtype:
+            self._scales_alt = (self.s_in.to(dtype), self.s_mid.to(dtype), self.s_out.to(dtype))
+        return self._scales_alt
 
 
 def build_layers(torch, dev, shapes, copies, seed):
@@ -123,10 +133,10 @@ def main():
     gen = torch.Generator(device=dev)
     gen.manual_seed(1)
 
-    def make_io(batch):
-        xs = [torch.randn(batch, lin.n, device=dev, generator=gen).to(torch.float16) for lin in layers[0]]
+    def make_io(batch, dtype=torch.float16):
+        xs = [torch.randn(batch, lin.n, device=dev, generator=gen).to(dtype) for lin in layers[0]]
         hs = [torch.empty(batch, lin.rp, dtype=torch.float32, device=dev) for lin in layers[0]]
-        ys = [torch.empty(batch, lin.m, dtype=torch.float16, device=dev) for lin in layers[0]]
+        ys = [torch.empty(batch, lin.m, dtype=dtype, device=dev) for lin in layers[0]]
         return xs, hs, ys
 
     def layer_pass(layer, io, batch, stream):
@@ -144,7 +154,7 @@ def main():
         xs, _, ys = io
         lists = []
         for layer in layers:
-            rl = DecodeRunList(batch, torch.float16, dev)
+            rl = DecodeRunList(batch, xs[0].dtype, dev)
             for lin, x, y in zip(layer, xs, ys):
                 lin.add_to(rl, x, y=y)
             rl.build()
@@ -267,6 +277,12 @@ def main():
             extra[f"batch{b}"] = {"us_per_layer": round(msb * 1e3, 3),
                                   "GBps": round(layer_bytes(b) / (msb * 1e-3) / 1e9, 2)}
             del lists
+        # bf16 activations and scales (what the reference's module defaults to), same layer and launch shape
+        io_bf = make_io(1, torch.bfloat16)
+        lists = make_runlists(io_bf, 1)
+        ms_bf = timed([rl.run for rl in lists], max(args.steps // 4, args.copies), args.copies)
+        extra["batch1_bf16"] = {"us_per_layer": round(ms_bf * 1e3, 3), "GBps": round(bytes1 / (ms_bf * 1e-3) / 1e9, 2)}
+        del lists, io_bf
         # all weight copies in ONE run list (= one launch over copies x 7 linears): the per-launch latencies
         # (descriptor fetch, two dependency phases, drain) are paid once for the whole stack
         from nanoquant_amd import DecodeRunList
