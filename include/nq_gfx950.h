@@ -170,7 +170,7 @@ int nq_gemm_nanoquant_bias(const void* x, const uint32_t* vt_tiles, const uint32
 /* Several terms with the same token count in two launches instead of two per term: the first GEMMs of all
  * terms, then the second ones (the projections of a decoder block that read the same tokens: q/k/v, gate/up, or
  * independent linears of a layer).  Up to 128 tokens a single term cannot fill the device and is bound by launch
- * and load latencies; grouped, the same launches carry several times the work.  Above 128 tokens the group runs
+ * and load latencies; grouped, the same launches carry several times the work.  Above 160 tokens the group runs
  * on 64-token block tiles whose workgroups walk the whole k of their term (no k-split, no scratch): together the
  * terms fill the device where one term needs a k-split and a finish launch to do so.  Only when some terms have
  * s_in and others do not does the call run the terms one after another (nq_gemm_nanoquant_bias); it then needs

@@ -386,7 +386,7 @@ __global__ __launch_bounds__(256) void gemm_kwave_group_kernel(GemmGroup g) {
     kwave_tile<DT, SCALED, RT>(a, local % gx, local / gx);
 }
 
-// The same for more than 128 tokens: block tiles of 64 tokens x 128*RT rows, every workgroup walks the whole k of
+// The same for more tokens (above kKwaveGroupMaxTokens): block tiles of 64 tokens x 128*RT rows, every workgroup walks the whole k of
 // its problem (no k-split, no scratch).  Workgroups go to the 8 XCDs round-robin by id and first[p] is a multiple
 // of 8, so (id - first[p]) mod 8 is the XCD; the mapping keeps the workgroups that share an activation slab on one
 // XCD (one L2) where the number of token blocks gy allows it: gy a multiple of 8 (or large): XCD = token block
@@ -463,6 +463,9 @@ struct GemmPlan {
 };
 
 constexpr int kKwaveMaxTokens = 128;
+// In a group the few-token tiles stay ahead a little longer (Llama-2-7B layer, share of the fp16 peak, few-token vs
+// block tiles: 144 tokens 22.5 vs 19.6 %, 160 tokens 27.1 vs 22.3 %, 192 tokens 25.8 vs 26.1 %, 256 tokens 28.1 vs 30.8 %).
+constexpr int kKwaveGroupMaxTokens = 160;
 
 static GemmPlan plan_gemm(int T, int K, int R) {
     GemmPlan p;
@@ -586,7 +589,7 @@ hipError_t gemm_onebit(int dtype, const void* x, const uint32_t* tiles, const vo
     return p.rt == 2 ? launch_gemm<1, 2, 2, 256>(a, p, stream) : launch_gemm<1, 2, 1, 256>(a, p, stream);
 }
 
-// More than kKwaveMaxTokens tokens: one launch of gemm_block_group_kernel.  Two row tiles per wavefront halve the
+// More than kKwaveGroupMaxTokens tokens: one launch of gemm_block_group_kernel.  Two row tiles per wavefront halve the
 // LDS reads per MFMA and are taken once that still leaves two workgroups for every CU.
 static hipError_t gemm_block_group(int dtype, int count, const void* const* x, const uint32_t* const* tiles,
                                    const void* const* s_in, const void* const* s_out, const void* const* bias,
@@ -631,13 +634,13 @@ static hipError_t gemm_block_group(int dtype, int count, const void* const* x, c
 }
 
 // GEMMs of several problems on the same token count in one launch; every problem: K % 256 == 0, R % 32 == 0, and
-// either all have input scales or none (checked by the caller).  Up to kKwaveMaxTokens tokens the few-token
+// either all have input scales or none (checked by the caller).  Up to kKwaveGroupMaxTokens tokens the few-token
 // tiles, above them block tiles.
 hipError_t gemm_onebit_group(int dtype, int count, const void* const* x, const uint32_t* const* tiles,
                              const void* const* s_in, const void* const* s_out, const void* const* bias, void* const* y,
                              int T, const int* K, const int* R, hipStream_t stream) {
     if (count < 1 || count > kGroupMax) return hipErrorInvalidValue;
-    if (T > kKwaveMaxTokens) return gemm_block_group(dtype, count, x, tiles, s_in, s_out, bias, y, T, K, R, stream);
+    if (T > kKwaveGroupMaxTokens) return gemm_block_group(dtype, count, x, tiles, s_in, s_out, bias, y, T, K, R, stream);
     const int gy = (T + 31) / 32;
     int rt = 4;                                  // widest row blocks that still leave two workgroups per CU
     for (; rt > 1; rt /= 2) {
@@ -682,6 +685,6 @@ hipError_t gemm_onebit_group(int dtype, int count, const void* const* x, const u
 }
 
 int gemm_group_max() { return kGroupMax; }
-int gemm_group_max_tokens() { return kKwaveMaxTokens; }
+int gemm_group_max_tokens() { return kKwaveGroupMaxTokens; }
 
 }  // namespace nq

@@ -313,7 +313,7 @@ def gemm_group_forward(xs, terms, biases=None):
     call: `terms` is a list of argument tuples (weight_u, weight_v, scale_g, scale_l, scale_h, workspace) as that
     op takes them after x; `xs` is one tensor [tokens, n] read by every term or a list of one tensor per term;
     `biases` an optional list of [m] tensors / None.  Returns the list of outputs.  The terms share
-    launches (a single linear leaves most of the device idle up to some hundred tokens): few-token tiles up to 128
+    launches (a single linear leaves most of the device idle up to some hundred tokens): few-token tiles up to 160
     tokens, 64-token block tiles without k-split above.  The
     reference launches every linear by itself (modules/linear.py:131-133)."""
     lib = _lib.lib()

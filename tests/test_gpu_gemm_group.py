@@ -27,7 +27,7 @@ def _term(dev, m, n, r, seed, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("tokens", [128, 77, 1, 200, 320, 512])
+@pytest.mark.parametrize("tokens", [128, 77, 1, 150, 200, 320, 512])
 def test_group_on_shared_tokens(dev, tokens, dtype):
     # q, k, v-like: one input, different widths and ranks (one rank padded by the packer); above 128 tokens the
     # group runs on block tiles (64 tokens; 200 leaves a ragged last block), every workgroup walking the whole k
