@@ -339,7 +339,7 @@ def main():
         from nanoquant_amd import ops as nq_ops
         by_mn = {(m, n): (packed, r) for (m, n, r), packed in packed_by_shape.items()}
         group = [by_mn[(m, n)] for (_, m, n) in LLAMA2_7B_LAYER]
-        for tokens in (16, 128, 512):
+        for tokens in (16, 128, 512, 4096):
             xs_t = {n: torch.randn(tokens, n, device=dev, generator=g2).to(torch.float16) for n in (4096, 11008)}
             group_x = [xs_t[n] for (_, _, n) in LLAMA2_7B_LAYER]
             group_flops = sum(gemm_flops(m, n, by_mn[(m, n)][1], tokens) for (_, m, n) in LLAMA2_7B_LAYER)
