@@ -336,11 +336,16 @@ def prefill_group(modules: Sequence, x) -> list:
     for mod in mods:
         b = mod.bias if (mod.kernel_path_bias and mod.bias is not None) else None
         biases.append(None if b is None else (b if b.dtype == mod.dtype else b.to(mod.dtype)))
-    ys = ops.gemm_group_forward(flat, [(m.V_int8, m.U_int8, m.s1, m.s2, m.s3, m.workspace) for m in mods],
-                                biases if any(b is not None for b in biases) else None)
-    outs = [None] * len(entries)
-    for y, i in zip(ys, owner):
-        outs[i] = y if outs[i] is None else outs[i] + y
+    pack = lambda m: (m.V_int8, m.U_int8, m.s1, m.s2, m.s3, m.workspace)
+    if len(mods) == len(entries):              # no mixtures: one output per module
+        outs = ops.gemm_group_forward(flat, [pack(m) for m in mods], biases if any(b is not None for b in biases) else None)
+    else:                                      # the terms of a mixture are summed (one add per extra term index)
+        groups, bias_groups, group_x = [[] for _ in entries], [[] for _ in entries], [None] * len(entries)
+        for mod, xf, b, i in zip(mods, flat, biases, owner):
+            groups[i].append(pack(mod))
+            bias_groups[i].append(b)
+            group_x[i] = xf
+        outs = ops.gemm_group_sum_forward(group_x, groups, bias_groups if any(b is not None for b in biases) else None)
     for i, t in enumerate(xs_in):
         y = outs[i]
         if t.ndim == 3:

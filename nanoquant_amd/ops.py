@@ -308,11 +308,12 @@ class NqGemmTerm(ctypes.Structure):
                 ("n", ctypes.c_int), ("r", ctypes.c_int), ("m", ctypes.c_int)]
 
 
-def gemm_group_forward(xs, terms, biases=None):
+def gemm_group_forward(xs, terms, biases=None, outs=None):
     """Several `marlin_nanoquant_forward` calls on the same number of tokens in two launches instead of two per
     call: `terms` is a list of argument tuples (weight_u, weight_v, scale_g, scale_l, scale_h, workspace) as that
     op takes them after x; `xs` is one tensor [tokens, n] read by every term or a list of one tensor per term;
-    `biases` an optional list of [m] tensors / None.  Returns the list of outputs.  The terms share
+    `biases` an optional list of [m] tensors / None; `outs` an optional list of contiguous [tokens, m] tensors of
+    the activation type to write into (allocated here when absent).  Returns the list of outputs.  The terms share
     launches (a single linear leaves most of the device idle up to some hundred tokens): few-token tiles up to 160
     tokens, 64-token block tiles without k-split above.  The
     reference launches every linear by itself (modules/linear.py:131-133)."""
@@ -322,10 +323,10 @@ def gemm_group_forward(xs, terms, biases=None):
         return []
     if isinstance(xs, torch.Tensor):
         xs = [xs] * count
-    if len(xs) != count or (biases is not None and len(biases) != count):
-        raise RuntimeError("one x (and one bias entry) per term")
+    if len(xs) != count or (biases is not None and len(biases) != count) or (outs is not None and len(outs) != count):
+        raise RuntimeError("one x (and one bias / output entry) per term")
     dt = _gemm_dtype(xs[0])
-    outs, keep, arr_items, nbytes = [], [], [], 0
+    given, outs, keep, arr_items, nbytes = outs, [], [], [], 0
     for i, (x, term) in enumerate(zip(xs, terms)):
         weight_u, weight_v, scale_g, scale_l, scale_h, workspace = term
         bias = None if biases is None else biases[i]
@@ -340,7 +341,13 @@ def gemm_group_forward(xs, terms, biases=None):
         imm = torch.empty((t, r), dtype=x.dtype, device=x.device)
         _, m, _ = _onebit_check(imm, weight_v, None, scale_h, workspace)
         _check_bias(bias, m, x)
-        out = torch.empty((t, m), dtype=x.dtype, device=x.device)
+        if given is None:
+            out = torch.empty((t, m), dtype=x.dtype, device=x.device)
+        else:
+            out = given[i]
+            if (tuple(out.shape) != (t, m) or out.dtype != x.dtype or out.device != x.device or not out.is_contiguous()
+                    or out.data_ptr() % 16 != 0):
+                raise RuntimeError(f"outs[{i}] must be a contiguous, 16-byte aligned [{t}, {m}] tensor of {x.dtype} on {x.device}")
         outs.append(out)
         keep.append(imm)
         nbytes = max(nbytes, int(lib.nq_gemm_scratch_bytes(t, n, r)), int(lib.nq_gemm_scratch_bytes(t, r, m)))
@@ -359,6 +366,50 @@ def gemm_group_forward(xs, terms, biases=None):
             arr = (NqGemmTerm * len(part))(*part)
             _lib.check(lib.nq_gemm_nanoquant_group(arr, len(part), tokens, dt, _ptr(scratch), nbytes, _stream(device)))
     return outs
+
+
+def gemm_group_sum_forward(xs, term_groups, bias_groups=None):
+    """`[sum_t marlin_nanoquant_forward(x_i, *term_groups[i][t]) for i]`: weights that are sums of several binary
+    low-rank terms (mixture of ranks) on the grouped prefill launches.  All terms of all weights share the two
+    launches of `gemm_group_forward`; the t-th terms of all weights write into one flat buffer per t, weights with
+    more terms first, so that the sums over the terms are one in-place add per extra term index instead of one
+    per weight.  `xs`: one tensor or one per weight; `bias_groups`: optional list (per weight) of lists (per term) of
+    bias tensors / None.  Returns one [tokens, m] tensor per weight (views of one buffer)."""
+    nw = len(term_groups)
+    if nw == 0:
+        return []
+    if isinstance(xs, torch.Tensor):
+        xs = [xs] * nw
+    if len(xs) != nw or any(len(g) == 0 for g in term_groups):
+        raise RuntimeError("one x and at least one term per weight")
+    tokens, dtype, device = xs[0].size(0), xs[0].dtype, xs[0].device
+    ms = [g[0][1].size(1) * 2 for g in term_groups]                  # weight_v [r / 16, m / 2]
+    order = sorted(range(nw), key=lambda i: -len(term_groups[i]))      # stable: more terms first
+    depth = len(term_groups[order[0]])
+    sizes = [sum(tokens * ms[i] for i in order if len(term_groups[i]) > t) for t in range(depth)]
+    bufs = [torch.empty(n, dtype=dtype, device=device) for n in sizes]
+    flat_x, flat_terms, flat_bias, flat_out = [], [], [], []
+    results = [None] * nw
+    for t in range(depth):
+        off = 0
+        for i in order:
+            if len(term_groups[i]) <= t:
+                break
+            m = ms[i]
+            if (off * bufs[t].element_size()) % 16 != 0:
+                raise RuntimeError("tokens * out_features must keep the outputs 16-byte aligned")
+            view = bufs[t][off:off + tokens * m].view(tokens, m)
+            off += tokens * m
+            if t == 0:
+                results[i] = view
+            flat_x.append(xs[i])
+            flat_terms.append(term_groups[i][t])
+            flat_bias.append(None if bias_groups is None or bias_groups[i] is None else bias_groups[i][t])
+            flat_out.append(view)
+    gemm_group_forward(flat_x, flat_terms, flat_bias if any(b is not None for b in flat_bias) else None, outs=flat_out)
+    for t in range(1, depth):
+        bufs[0][:sizes[t]].add_(bufs[t])
+    return results
 
 
 def gemv_mixture_forward(x, terms):

@@ -138,3 +138,36 @@ def test_prefill_harness_on_a_tiny_layer(dev):
     assert [r["tokens"] for r in rows] == [32, 160]
     for r in rows:
         assert r["one_by_one"]["us_per_layer"] > 0 and r["grouped"]["us_per_layer"] > 0
+
+
+def test_group_sum_with_uneven_term_counts_and_bias(dev):
+    # three weights with 2, 1 and 3 terms: the flat output buffers put weights with more terms first; every weight
+    # must still come back in its own position and equal the sum of its terms (dense definition, fp64)
+    dtype, tokens, n = torch.float16, 100, 512
+    spec = [(256, [64, 32]), (512, [128]), (320, [96, 64, 32])]
+    rng = np.random.default_rng(8)
+    groups, refs, bias_groups = [], [], []
+    x = _cast(oracle.synth_x(tokens, n, 21), dtype)
+    for w, (m, ranks) in enumerate(spec):
+        terms, ref, biases = [], 0.0, []
+        for t, r in enumerate(ranks):
+            packed, f = _term(dev, m, n, r, 900 + 10 * w + t, dtype)
+            terms.append(packed)
+            ref = ref + f(x.float().numpy().astype(np.float64))
+            if w == 2 and t == 1:
+                b = _cast(rng.normal(0, 0.05, m), dtype)
+                biases.append(b.to(dev))
+                ref = ref + b.float().numpy()[None, :]
+            else:
+                biases.append(None)
+        groups.append(terms)
+        refs.append(ref)
+        bias_groups.append(biases)
+    print("group sum 2/1/3 terms", flush=True)
+    ys = ops.gemm_group_sum_forward(x.to(dev), groups, bias_groups)
+    torch.cuda.synchronize()
+    for (m, _), y, ref in zip(spec, ys, refs):
+        assert y.shape == (tokens, m) and y.dtype == dtype
+        assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < TOL[dtype]
+    with pytest.raises(RuntimeError):
+        ops.gemm_group_sum_forward(x.to(dev), [groups[0], []])
