@@ -171,3 +171,38 @@ def test_group_sum_with_uneven_term_counts_and_bias(dev):
         assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < TOL[dtype]
     with pytest.raises(RuntimeError):
         ops.gemm_group_sum_forward(x.to(dev), [groups[0], []])
+
+
+@pytest.mark.parametrize("tokens", [64, 300])
+def test_group_through_the_c_abi_without_scratch(dev, tokens):
+    # nq_gemm_nanoquant_group called directly with raw pointers and scratch = NULL: groups whose terms all have input
+    # scales need no scratch at any token count; null pointers, duplicate outputs and oversized groups are refused
+    import ctypes
+    from nanoquant_amd import _lib
+    lib = _lib.lib()
+    dtype, n = torch.float16, 512
+    shapes = [(256, 64), (512, 128)]
+    x = _cast(oracle.synth_x(tokens, n, 31), dtype).to(dev)
+    items, keep, refs = [], [], []
+    for i, (m, r) in enumerate(shapes):
+        packed, ref = _term(dev, m, n, r, 950 + i, dtype)
+        wu, wv, sg, sl, sh, _ = packed
+        rp = wu.size(1) * 2                                   # rank as padded by the packer
+        h = torch.empty(tokens, rp, dtype=dtype, device=dev)
+        y = torch.empty(tokens, m, dtype=dtype, device=dev)
+        keep += [packed, h, y]
+        refs.append((y, ref))
+        items.append(ops.NqGemmTerm(x.data_ptr(), wu.data_ptr(), wv.data_ptr(), sg.data_ptr(), sl.data_ptr(), sh.data_ptr(),
+                                    None, h.data_ptr(), y.data_ptr(), n, rp, m))
+    arr = (ops.NqGemmTerm * len(items))(*items)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    print(f"group via C ABI tokens={tokens}", flush=True)
+    assert lib.nq_gemm_nanoquant_group(arr, len(items), tokens, _lib.NQ_F16, None, 0, stream) == 0
+    torch.cuda.synchronize()
+    for y, ref in refs:
+        assert oracle.max_rel_err(y.float().cpu().numpy(), ref(x.float().cpu().numpy())) < TOL[dtype]
+    dup = (ops.NqGemmTerm * 2)(items[0], items[0])            # same h / y twice
+    assert lib.nq_gemm_nanoquant_group(dup, 2, tokens, _lib.NQ_F16, None, 0, stream) != 0
+    assert lib.nq_gemm_nanoquant_group(None, 2, tokens, _lib.NQ_F16, None, 0, stream) != 0
+    assert lib.nq_gemm_nanoquant_group(arr, int(lib.nq_gemm_group_max()) + 1, tokens, _lib.NQ_F16, None, 0, stream) != 0
+    assert lib.nq_gemm_nanoquant_group(arr, 0, tokens, _lib.NQ_F16, None, 0, stream) == 0
