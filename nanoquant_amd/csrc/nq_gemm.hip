@@ -462,7 +462,7 @@ struct GemmPlan {
     bool kwave;   // few tokens: gemm_kwave_kernel (32x32 output tiles, wavefronts split k)
 };
 
-constexpr int kKwaveMaxTokens = 128;
+constexpr int kKwaveMaxTokens = 256;
 // In a group the few-token tiles stay ahead a little longer (Llama-2-7B layer, share of the fp16 peak, few-token vs
 // block tiles: 144 tokens 22.5 vs 19.6 %, 160 tokens 27.1 vs 22.3 %, 192 tokens 25.8 vs 26.1 %, 256 tokens 28.1 vs 30.8 %).
 constexpr int kKwaveGroupMaxTokens = 160;
@@ -472,7 +472,9 @@ static GemmPlan plan_gemm(int T, int K, int R) {
     p.kwave = false;
     if (T <= kKwaveMaxTokens) {
         // 32x32 output tiles, wavefronts split k: no k-split scratch, one launch (4096x4096 at 128 tokens:
-        // 16.8 vs 22.7 us per linear with the block kernel; no gain above 128 tokens)
+        // 16.8 vs 22.7 us per linear with the block kernel).  The 7 linears of a Llama-2-7B layer one after the other,
+        // few-token vs block tiles: 144 tokens 191 vs 224 us, 160: 193 vs 231, 192: 220 vs 246, 256: 236 vs 252,
+        // 288: 287 vs 268, 384: 313 vs 300, 448: 349 vs 314.
         p.kwave = true;
         p.tt = 1; p.gy = (T + 31) / 32;
         // every 32-row tile re-reads the 32-token activation slab: wider workgroups once there are enough of them
