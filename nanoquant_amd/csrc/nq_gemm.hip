@@ -491,10 +491,12 @@ static GemmPlan plan_gemm(int T, int K, int R) {
     p.tt = 2;
     {
         // Few tokens: 32-token blocks give twice the workgroups, which can spare the k-split and with it
-        // the atomics and the finish launch (4096x4096 at 256 tokens: 44 -> 27 us per linear).  Only when
+        // the atomics and the finish launch (4096x4096 at 256 tokens: 44 -> 27 us per linear; with the bound on
+        // 64-token workgroups raised from 256 to 512: 4096x4096 at 512 tokens 45.5 -> 33.6 us, at 1024 tokens
+        // 59.3 -> 49.5 us, 4096x11008 at 512 tokens 80.2 -> 71.0 us, the other shapes within 5 %).  Only when
         // k is short enough for one workgroup to walk it (<= 16 tiles).
         const int gx1 = (R + 127) / 128, gy1 = (T + 31) / 32;
-        if (gx1 * ((T + 63) / 64) < 256 && gx1 * gy1 >= 128 && K / kTileK <= 16) {
+        if (gx1 * ((T + 63) / 64) < 512 && gx1 * gy1 >= 128 && K / kTileK <= 16) {
             p.tt = 1; p.rt = 1; p.gx = gx1; p.gy = gy1;
             p.ktiles_per_split = K / kTileK; p.ksplit = 1; p.xcd = false;
             return p;
