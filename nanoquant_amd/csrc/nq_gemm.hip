@@ -477,10 +477,22 @@ static GemmPlan plan_gemm(int T, int K, int R) {
         // 288: 287 vs 268, 384: 313 vs 300, 448: 349 vs 314.
         p.kwave = true;
         p.tt = 1; p.gy = (T + 31) / 32;
-        // every 32-row tile re-reads the 32-token activation slab: wider workgroups once there are enough of them
-        // (two per CU; 11008 rows at 128 tokens: 36.4 -> 31.5 us per linear with two row tiles per workgroup)
-        p.rt = 1;
-        while (p.rt < 4 && (R / 32 / (2 * p.rt)) * p.gy >= 512) p.rt *= 2;
+        // Every 32-row tile re-reads the 32-token activation slab, so wider workgroups save L2 traffic, and a launch
+        // lasts about (workgroups per CU, rounded up) x (row tiles per workgroup): take the width that minimises
+        // that product, the wider one on ties.  Measured at 128 tokens (us per GEMM, 1 / 2 / 4 row tiles): 2048 rows
+        // k 4096: 8.3 / 9.8 / 13.6; 3072 rows k 4096: 10.9 / 9.9 / 13.5; 3072 rows k 11008: 23.3 / 20.1 / 27.5;
+        // 4096 rows k 3072: 8.9 / 8.7 / 11.9; 11008 rows k 3072: 21.8 / 18.5 / 18.9.
+        // With two or more workgroups per CU left, wider is better outright (11008 rows at 256 tokens: 4 row tiles).
+        constexpr int kCUs = 256;
+        auto wgs = [&](int rt) { return (long)((R / 32 + rt - 1) / rt) * p.gy; };
+        int rt0 = 1;
+        while (rt0 < 4 && wgs(2 * rt0) >= 2 * kCUs) rt0 *= 2;
+        p.rt = rt0;
+        long best_cost = -1;
+        for (int rt = rt0; rt <= 4; rt *= 2) {
+            const long cost = ((wgs(rt) + kCUs - 1) / kCUs) * rt;
+            if (best_cost < 0 || cost <= best_cost) { best_cost = cost; p.rt = rt; }
+        }
         p.gx = (R / 32 + p.rt - 1) / p.rt;
         p.ktiles_per_split = K / kTileK; p.ksplit = 1; p.xcd = false;
         return p;
