@@ -470,29 +470,28 @@ constexpr int kKwaveGroupMaxTokens = 160;
 static GemmPlan plan_gemm(int T, int K, int R) {
     GemmPlan p;
     p.kwave = false;
-    if (T <= kKwaveMaxTokens) {
+    // A long k (more than 16 tiles) needs a k-split with atomics and a finish launch on block tiles, while the
+    // wavefronts of a few-token tile split k for free: those GEMMs stay on few-token tiles up to 1024 tokens
+    // (k 11008 -> 3072 rows: 512 tokens 51.3 vs 55.5 us, 1024 tokens 79.3 vs 94.7, 2048 tokens 148.8 vs 147.0).
+    if (T <= kKwaveMaxTokens || (K / kTileK > 16 && T <= 1024)) {
         // 32x32 output tiles, wavefronts split k: no k-split scratch, one launch (4096x4096 at 128 tokens:
         // 16.8 vs 22.7 us per linear with the block kernel).  The 7 linears of a Llama-2-7B layer one after the other,
         // few-token vs block tiles: 144 tokens 191 vs 224 us, 160: 193 vs 231, 192: 220 vs 246, 256: 236 vs 252,
         // 288: 287 vs 268, 384: 313 vs 300, 448: 349 vs 314.
         p.kwave = true;
         p.tt = 1; p.gy = (T + 31) / 32;
-        // Every 32-row tile re-reads the 32-token activation slab, so wider workgroups save L2 traffic, and a launch
-        // lasts about (workgroups per CU, rounded up) x (row tiles per workgroup): take the width that minimises
-        // that product, the wider one on ties.  Measured at 128 tokens (us per GEMM, 1 / 2 / 4 row tiles): 2048 rows
-        // k 4096: 8.3 / 9.8 / 13.6; 3072 rows k 4096: 10.9 / 9.9 / 13.5; 3072 rows k 11008: 23.3 / 20.1 / 27.5;
-        // 4096 rows k 3072: 8.9 / 8.7 / 11.9; 11008 rows k 3072: 21.8 / 18.5 / 18.9.
-        // With two or more workgroups per CU left, wider is better outright (11008 rows at 256 tokens: 4 row tiles).
-        constexpr int kCUs = 256;
-        auto wgs = [&](int rt) { return (long)((R / 32 + rt - 1) / rt) * p.gy; };
-        int rt0 = 1;
-        while (rt0 < 4 && wgs(2 * rt0) >= 2 * kCUs) rt0 *= 2;
-        p.rt = rt0;
-        long best_cost = -1;
-        for (int rt = rt0; rt <= 4; rt *= 2) {
-            const long cost = ((wgs(rt) + kCUs - 1) / kCUs) * rt;
-            if (best_cost < 0 || cost <= best_cost) { best_cost = cost; p.rt = rt; }
-        }
+        // Every 32-row tile re-reads the 32-token activation slab, so wider workgroups save L2 traffic: with a
+        // long k the widest that still leaves workgroups for three quarters of the CUs.  Measured (us per GEMM, 1 / 2 / 4 row tiles):
+        // 128 tokens: 2048 rows k 4096: 8.3 / 9.8 / 13.6; 3072 rows k 4096: 10.9 / 9.9 / 13.5; 3072 rows k 11008:
+        // 23.3 / 20.1 / 27.5; 4096 rows k 3072: 8.9 / 8.7 / 11.9; 11008 rows k 3072: 21.8 / 18.5 / 18.9;
+        // 256 tokens: 2048 rows k 4096: 10.8 / 10.9 / 14.2; 3072 rows k 4096: 16.5 / 14.3 / 14.1; 3072 rows k 11008:
+        // 36.5 / 34.3 / 31.5; 4096 rows k 3072: 12.2 / 11.9 / 12.2.
+        // With a short k a workgroup is gone before its neighbours have started, and more of them do better: two
+        // per CU there (11008 rows k 3072 at 128 tokens: 688 workgroups of two row tiles, 2 us per linear faster than 344 of four).
+        const int min_workgroups = K / kTileK >= 16 ? 192 : 512;
+        p.rt = 1;
+        for (int rt = 2; rt <= 4; rt *= 2)
+            if ((long)((R / 32 + rt - 1) / rt) * p.gy >= min_workgroups) p.rt = rt;
         p.gx = (R / 32 + p.rt - 1) / p.rt;
         p.ktiles_per_split = K / kTileK; p.ksplit = 1; p.xcd = false;
         return p;
