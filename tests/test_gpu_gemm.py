@@ -49,6 +49,9 @@ def test_config0_shape(dev, dtype, tokens):
     (256, 256, 32, 1),          # a single token, rank padded 32 -> 256
     (320, 512, 100, 77),        # ragged tokens, rows not a multiple of 128
     (128, 768, 256, 200),
+    (256, 4352, 256, 300),      # k of 17 tiles: few-token tiles beyond 256 tokens (wavefronts split k, no scratch)
+    (256, 4352, 256, 1100),     # the same above 1024 tokens: block tiles with a k-split
+    (384, 512, 1024, 640),      # 32-token blocks without k-split (few 64-token workgroups, short k)
 ])
 def test_shapes_fp16(dev, m, n, r, tokens):
     err = _run_fused(dev, m, n, r, tokens, torch.float16, seed=m + r + tokens)
