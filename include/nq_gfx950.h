@@ -35,6 +35,7 @@ typedef enum nq_status {
     NQ_ERR_WORKSPACE = -6,    /* "workspace too small" (kernel/cuda/gemm.cpp:52) */
     NQ_ERR_ORDER = -7,        /* unknown word order id */
     NQ_ERR_ALIGN = -8,        /* a prefill operand is not 16-byte aligned */
+    NQ_ERR_SCRATCH_LIMIT = -9, /* nq_gemv_forward_noalloc: batch * r above NQ_NOALLOC_MAX_H_FLOATS */
     NQ_ERR_HIP = -100         /* a HIP call failed; see nq_last_hip_error() */
 } nq_status;
 
@@ -63,6 +64,19 @@ int nq_gemv_forward_bias(const void* x, const void* s_in, const uint32_t* vt_bit
                          const uint32_t* u_bits, const void* s_out, const void* bias, float* h_scratch, void* y,
                          int batch, int n, int r, int m, int dtype, void* stream);
 
+/* nq_gemv_forward_bias for callers that cannot allocate device memory or hand over a workspace: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference (whose
+ * wrapper allocates `interm` with torch::empty on every call, kernel/cuda/gemv_kernel.cu:345).  The fp32
+ * intermediate h lives in a device array inside the library, NQ_NOALLOC_MAX_H_FLOATS floats (1 MiB) per GPU, held
+ * until the process ends: batch * r above that returns NQ_ERR_SCRATCH_LIMIT.  The call allocates and frees nothing.
+ * All calls on one GPU share that array: calls that overlap in time on one GPU (two streams, two threads) race on
+ * it; h is fully rewritten by every call, nothing needs clearing between calls.  The first call on each device
+ * looks up the array's address and should be made outside graph capture. */
+#define NQ_NOALLOC_MAX_H_FLOATS (256 * 1024)
+int nq_gemv_forward_noalloc(const void* x, const void* s_in, const uint32_t* vt_bits, const void* s_mid,
+                            const uint32_t* u_bits, const void* s_out, const void* bias, void* y,
+                            int batch, int n, int r, int m, int dtype, void* stream);
+
 /* Decode path, sum of `nterms` terms that share x (the mixture-of-rank layer; no counterpart in the
  * reference's code, defined as the sum of single-term layers).  Arrays hold one pointer / rank per
  * term; s_mid[t] may be NULL.  h_scratch: fp32 [batch, max r]; y_scratch: fp32 [batch, m]. */
@@ -90,10 +104,13 @@ int nq_gemv_mixture(const void* x, const void* const* s_in, const uint32_t* cons
  * stability; the phase schedule does not need it.
  * nq_runlist_run enqueues the single launch; it allocates nothing and can be graph-captured.  Runs of
  * the same workspace must not overlap in time.  batch must be 1, 2, 4, 8 or 16.
- * Inside the launch a stage waits for the stages it depends on through device-scope counters; the
- * waits are bounded.
- * nq_runlist_status copies the error word back (synchronises): 0 ok, 1 = a bounded dependency wait
- * expired (the results of that run are invalid; call nq_runlist_build again before reuse). */
+ * Inside the launch a stage waits for the stages it depends on through device-scope counters, which needs every
+ * workgroup of the grid resident at once.  The grid is sized to what the device keeps resident when it has the
+ * device to itself: a run list must not share the GPU with other kernels (another stream, another process) while
+ * it runs.  The waits are bounded: if producers cannot become resident, waiting workgroups give up, set the status
+ * word and the grid drains; the outputs of that launch are then invalid.
+ * nq_runlist_status copies the status word back (synchronises) and clears it: 0 ok, 1 = a bounded dependency wait
+ * expired in some launch since the last call (results invalid; the list itself stays usable). */
 typedef struct nq_linear {
     const void* x;          /* NULL: bound at run time (nq_runlist_run_bound) */
     const void* s_in;
@@ -197,6 +214,16 @@ int nq_gemm_nanoquant_group(const nq_gemm_term* terms, int count, int tokens, in
  * ("lsb_first", modules/linear.py:298) to the kernel format ("half2", modules/linear.py:171-172)
  * without the dense round trip of utils/load_utils.py:269-293.  order ids: nq_word_order. */
 int nq_repack_words(const uint32_t* src, uint32_t* dst, size_t nwords, int src_order, int dst_order, void* stream);
+
+/* Row-major packed words of a factor (either word order) -> the 32-row x 256-k tile layout that the prefill
+ * entry points read, on the device and without a dense matrix: the second half of serving a checkpoint
+ * (modules/linear.py:288-321 writes `lsb_first` words [rows, ceil(cols/32)]; utils/load_utils.py:269-293 unpacks
+ * them to dense +-1 before kernel/utils.py:217-284 packs them again).  words [rows, words_per_row]; tiles receives
+ * rows_padded * k_padded / 32 words; rows_padded % 32 == 0, k_padded % 256 == 0, rows_padded >= rows,
+ * k_padded >= 32 * words_per_row.  Rows and columns beyond the source are +1 signs (zero bits): the rank padding
+ * of the two-stage packer (kernel/utils.py:262-271), to be paired with a zero mid scale.  src != dst. */
+int nq_pack_gemm_tiles(const uint32_t* words, uint32_t* tiles, int rows, int words_per_row, int rows_padded,
+                       int k_padded, int src_order, void* stream);
 
 /* Tile order of the packed words for run lists (no counterpart in the reference, whose kernels read the row-major
  * words of kernel/utils.py:51-113 directly): 16-byte units indexed [row/32][unit/4][(row/16)&1][unit&3][row&15],

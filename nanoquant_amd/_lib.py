@@ -24,6 +24,7 @@ _SIGNATURES = {
     "nq_device_query": (_i, [_i, ctypes.POINTER(_i)]),
     "nq_gemv_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "nq_gemv_forward_bias": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "nq_gemv_forward_noalloc": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "nq_gemv_mixture": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "nq_runlist_workspace_bytes": (_sz, [_vp, _i]),
     "nq_runlist_build": (_i, [_vp, _i, _i, _i, _i, _vp, _sz, _vp, _vp]),
@@ -39,6 +40,7 @@ _SIGNATURES = {
     "nq_repack_words": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
     "nq_gemm_group_max": (_i, []),
     "nq_gemm_nanoquant_group": (_i, [_vp, _i, _i, _i, _vp, _sz, _vp]),
+    "nq_pack_gemm_tiles": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "nq_tiled_words": (_sz, [_i, _i]),
     "nq_tile_words": (_i, [_vp, _vp, _i, _i, _i, _vp]),
     "nq_stream_copy": (_i, [_vp, _vp, _sz, _vp]),

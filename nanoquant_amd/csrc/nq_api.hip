@@ -4,6 +4,7 @@
 #include "nq_kernels.h"
 
 #include <algorithm>
+#include <mutex>
 #include <vector>
 
 namespace {
@@ -32,6 +33,7 @@ const char* nq_status_string(int status) {
         case NQ_ERR_WORKSPACE: return "workspace too small";
         case NQ_ERR_ORDER: return "unknown word order";
         case NQ_ERR_ALIGN: return "prefill operands must be 16-byte aligned";
+        case NQ_ERR_SCRATCH_LIMIT: return "batch * r exceeds the built-in scratch of the allocation-free entry point";
         case NQ_ERR_HIP: return "HIP runtime error";
         default: return "unknown status";
     }
@@ -39,7 +41,7 @@ const char* nq_status_string(int status) {
 
 int nq_last_hip_error(void) { return g_last_hip_error; }
 
-int nq_abi_version(void) { return 4; }
+int nq_abi_version(void) { return 5; }
 
 int nq_device_query(int attr, int* value) {
     if (!value) return NQ_ERR_NULL;
@@ -76,6 +78,47 @@ int nq_gemv_forward_bias(const void* x, const void* s_in, const uint32_t* vt_bit
     e = nq::gemv_stage(dtype, false, u_bits, h_scratch, nullptr, s_out, nullptr, y, false, batch, m,
                        words_of(r), r, r, m, st, bias);
     return hip_status(e);
+}
+
+// ---- the allocation-free variant of nq_gemv_forward_bias ---------------------------------------------
+// The fp32 intermediate h lives in a file-scope device array instead of a caller's buffer.  In host code the
+// array's name is only a handle: its device address is asked for once per device (each device holds its own copy)
+// and only that address is ever handed to a kernel.
+constexpr size_t kScratchFloats = NQ_NOALLOC_MAX_H_FLOATS;
+static __device__ __align__(256) float scratch[kScratchFloats];
+constexpr int kScratchMaxDevices = 64;
+static float* g_scratch_ptr[kScratchMaxDevices];
+static std::mutex g_scratch_mutex;
+
+static int scratch_address(float** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_status(e);
+    if (dev < 0 || dev >= kScratchMaxDevices) return NQ_ERR_SHAPE;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        float* p = nullptr;
+        e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_status(e);
+        if (!p) return NQ_ERR_NULL;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return NQ_OK;
+}
+
+int nq_gemv_forward_noalloc(const void* x, const void* s_in, const uint32_t* vt_bits, const void* s_mid,
+                            const uint32_t* u_bits, const void* s_out, const void* bias, void* y,
+                            int batch, int n, int r, int m, int dtype, void* stream) {
+    if (dtype != NQ_F16 && dtype != NQ_BF16) return NQ_ERR_DTYPE;
+    if (batch < 0 || n < 0 || r < 0 || m < 0) return NQ_ERR_SHAPE;
+    if ((unsigned long long)batch * (unsigned long long)r > kScratchFloats) return NQ_ERR_SCRATCH_LIMIT;
+    if (batch == 0 || m == 0) return NQ_OK;
+    if (!x || !s_in || !vt_bits || !u_bits || !s_out || !y) return NQ_ERR_NULL;
+    float* h = nullptr;
+    const int st = scratch_address(&h);
+    if (st != NQ_OK) return st;
+    return nq_gemv_forward_bias(x, s_in, vt_bits, s_mid, u_bits, s_out, bias, h, y, batch, n, r, m, dtype, stream);
 }
 
 int nq_gemv_mixture(const void* x, const void* const* s_in, const uint32_t* const* vt_bits,
@@ -159,6 +202,16 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         if (l.x_from >= 0 && !linears[l.x_from].y) return NQ_ERR_SHAPE;   // a bound output cannot feed another entry
         if (l.y_from >= 0 && !linears[l.y_from].y) return NQ_ERR_SHAPE;
         if (l.y_from >= 0 && !linears[l.y_from].out_f32) return NQ_ERR_SHAPE;   // addends are fp32 results
+        // a link must name the buffer, width and type that the earlier entry really produces: the kernel reads
+        // x as [batch, n] of the 16-bit type and the addend as fp32 [batch, m]
+        if (l.x_from >= 0) {
+            const nq_linear& p = linears[l.x_from];
+            if (l.x != p.y || l.n != p.m || p.out_f32) return NQ_ERR_SHAPE;
+        }
+        if (l.y_from >= 0) {
+            const nq_linear& p = linears[l.y_from];
+            if (l.addend != (const float*)p.y || l.m != p.m) return NQ_ERR_SHAPE;
+        }
         // two linears writing the same h would race inside a phase
         for (int j = 0; j < i; ++j)
             if (linears[j].h == l.h) return NQ_ERR_SHAPE;
@@ -416,6 +469,10 @@ int nq_runlist_status(const void* workspace, int* status_out, void* stream) {
     if (e != hipSuccess) return hip_status(e);
     e = hipStreamSynchronize((hipStream_t)stream);
     *status_out = (int)v;
+    if (e == hipSuccess && v != 0) {                 // read and clear: the next launch starts with a clean word
+        e = hipMemsetAsync(const_cast<void*>(workspace), 0, sizeof(v), (hipStream_t)stream);
+        if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
+    }
     return hip_status(e);
 }
 
@@ -526,6 +583,18 @@ int nq_repack_words(const uint32_t* src, uint32_t* dst, size_t nwords, int src_o
     if (nwords == 0) return NQ_OK;
     if (!src || !dst) return NQ_ERR_NULL;
     return hip_status(nq::repack_words(src, dst, nwords, src_order, dst_order, (hipStream_t)stream));
+}
+
+int nq_pack_gemm_tiles(const uint32_t* words, uint32_t* tiles, int rows, int words_per_row, int rows_padded,
+                       int k_padded, int src_order, void* stream) {
+    if (src_order != 0 && src_order != 1) return NQ_ERR_ORDER;
+    if (rows < 0 || words_per_row < 0 || rows_padded < rows || (long long)k_padded < 32ll * words_per_row) return NQ_ERR_SHAPE;
+    if (rows_padded % 32 != 0 || k_padded % 256 != 0) return NQ_ERR_PROB_SHAPE;
+    if (rows_padded == 0 || k_padded == 0) return NQ_OK;
+    if (!tiles || (!words && rows > 0 && words_per_row > 0)) return NQ_ERR_NULL;
+    if (words == tiles) return NQ_ERR_SHAPE;         // a permutation across words: not in place
+    return hip_status(nq::words_to_tiles(words, tiles, rows, words_per_row, rows_padded, k_padded, src_order,
+                                         (hipStream_t)stream));
 }
 
 int nq_stream_copy(void* dst, const void* src, size_t bytes, void* stream) {

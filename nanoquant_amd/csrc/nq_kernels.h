@@ -70,6 +70,8 @@ hipError_t gemm_onebit_group(int dtype, int count, const void* const* x, const u
 hipError_t stream_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);
 hipError_t repack_words(const uint32_t* src, uint32_t* dst, size_t nwords, int src_order, int dst_order,
                         hipStream_t stream);
+hipError_t words_to_tiles(const uint32_t* src, uint32_t* dst, int rows, int words, int rows_padded, int k_padded,
+                          int src_order, hipStream_t stream);
 size_t tiled_word_count(int rows, int words);
 hipError_t tile_words(const uint32_t* src, uint32_t* dst, int rows, int words, int inverse, hipStream_t stream);
 

@@ -22,17 +22,6 @@
 #include "nq_decode.h"
 #include "nq_kernels.h"
 
-// Development aid, never defined in the product build: per-workgroup timestamps.
-#ifdef NQ_TRACE
-#include <stdio.h>
-#include <stdlib.h>
-#include <vector>
-__device__ unsigned long long* g_nq_trace = nullptr;
-#define NQ_MARK(k) do { if (g_nq_trace && threadIdx.x == 0) g_nq_trace[(size_t)blockIdx.x * 16 + (k)] = __builtin_amdgcn_s_memtime(); } while (0)
-#else
-#define NQ_MARK(k) do { } while (0)
-#endif
-
 namespace nq {
 
 // Rows whose sums a workgroup keeps in LDS at a time (then: barrier, scale, store, barrier).  Few large
@@ -141,7 +130,6 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
     const int tid = threadIdx.x;
     const int wg = blockIdx.x;
     if (tid == 0) s_flag = 0;
-    NQ_MARK(0);
 
     // Which launch of this run list is this?  Needed only by waiting slices; the load is issued now and
     // its latency is hidden behind phase 0.
@@ -243,7 +231,6 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
             }
             lds_barrier();                                       // s_flag; previous slice is done with xs / racc
             aborted = aborted || (s_flag != 0);
-            if (sg == seg_begin && ph < 3) NQ_MARK(1 + 4 * ph);
 
             if (!aborted) {
                 bool staged = false;
@@ -268,7 +255,6 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                             staged = true;
                         }
                         lds_barrier();                           // xs / xsum / zeroed racc visible
-                        if (sg == seg_begin && ph < 3 && rb == seg.row_begin && c0 == 0) NQ_MARK(2 + 4 * ph);
                         if constexpr (kQ8) {
                             // Items = (pair of 16-row groups, 4-unit group), unit group fastest: one read of the input
                             // operand (eight 16-byte LDS reads per lane) serves two row groups, and a wavefront takes a
@@ -340,7 +326,6 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                             if (it < it_end) step(wa0, wb0);
                             if (it + 1 < it_end) step(wa1, wb1);
                             if (it_begin < it_end) flush();              // + sum of x at the end
-                            if (ph == 0 && sg == seg_begin) NQ_MARK(14);
                         } else {
                             // Items = (16-row group, 4-unit group), unit group fastest; every wavefront takes a
                             // contiguous run of items, so it mostly stays on one row group and adds its
@@ -392,7 +377,6 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                         }
                         }
                     lds_barrier();                               // row sums complete
-                    if (ph < 3) NQ_MARK(3 + 4 * ph);
                     for (int i = tid; i < nr * BATCH; i += kStreamThreads) {
                         const int row = rb + i / BATCH, b = i % BATCH;
                         float v = racc[i];
@@ -422,7 +406,10 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
             }
 
             if (st.signal) {
-                // Workgroup-scope release + barrier: every lane's stores above have been acknowledged.
+                // Every wavefront waits until its own stores above have been acknowledged by the memory side (a
+                // workgroup-scope fence emits no such wait on this target, and nothing orders the stores of one
+                // wavefront against the counter add of another), then the barrier collects all of them.
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                 __syncthreads();
                 if (tid == 0) {
@@ -433,7 +420,6 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                 }
             }
         }
-        if (ph < 3) NQ_MARK(4 + 4 * ph);
     }
 
     if (tid == 0 && !SINGLE) {
@@ -530,32 +516,9 @@ static hipError_t launch_stream(const RunStage* stages, int nstages, int nphases
     stream_lds_plan(BATCH, StreamKernel<DT, BATCH>::kArith, max_units, &chunk_cap, &lds);
     hipError_t e = prepare_kernel<DT, BATCH>(lds);
     if (e != hipSuccess) return e;
-#ifdef NQ_TRACE
-    static unsigned long long* tbuf = nullptr;
-    static int calls = 0;
-    if (getenv("NQ_TS") && !tbuf) {
-        (void)hipMalloc(&tbuf, (size_t)nwg * 128);
-        (void)hipMemset(tbuf, 0, (size_t)nwg * 128);
-        (void)hipMemcpyToSymbol(HIP_SYMBOL(g_nq_trace), &tbuf, sizeof(tbuf));
-    }
-#endif
     using SK = StreamKernel<DT, BATCH>;
     hipLaunchKernelGGL((SK::fn), dim3(nwg), dim3(SK::kThreads), lds, stream, stages, nstages,
                        nphases, seg_index, segs, counters, status, (unsigned)(1u << 21), chunk_cap, RunStage{}, 0, ext_in, ext_out);
-#ifdef NQ_TRACE
-    if (tbuf && ++calls == 40) {
-        (void)hipStreamSynchronize(stream);
-        std::vector<unsigned long long> h((size_t)nwg * 16);
-        (void)hipMemcpy(h.data(), tbuf, h.size() * 8, hipMemcpyDeviceToHost);
-        FILE* f = fopen(getenv("NQ_TS"), "w");
-        for (int i = 0; i < nwg; ++i) {
-            fprintf(f, "%d", i);
-            for (int k = 0; k < 16; ++k) fprintf(f, " %llu", h[(size_t)i * 16 + k]);
-            fprintf(f, "\n");
-        }
-        fclose(f);
-    }
-#endif
     return hipGetLastError();
 }
 

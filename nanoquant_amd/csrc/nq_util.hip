@@ -45,6 +45,48 @@ hipError_t repack_words(const uint32_t* src, uint32_t* dst, size_t nwords, int s
     return hipGetLastError();
 }
 
+// Row-major words (either order) -> the 32-row x 256-k tiles of the prefill kernels, no dense matrix in between.
+// Tile (rt, kt) is 64 lanes x 4 words; lane l owns row 32 rt + (l & 31), its word q holds, at in-word element
+// j = 8 t + e (t = 0..3, e = 0..7; "half2" bit position), the column k = 256 kt + 64 q + 16 t + 8 (l >> 5) + e.
+// So an output word draws 16 elements from each of the source words 8 kt + 2 q and 8 kt + 2 q + 1 of its row.
+// Rows beyond `rows` and words beyond `words` read as zero words (= +1 signs), which is the rank padding of the
+// two-stage packer.  One thread per output word.
+__global__ __launch_bounds__(256) void words_to_tiles_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst,
+                                                             int rows, int words, int ktiles, int src_order, size_t nout) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nout; i += stride) {
+        const int q = (int)(i & 3), l = (int)((i >> 2) & 63);
+        const size_t tile = i >> 8;
+        const int kt = (int)(tile % (size_t)ktiles), rt = (int)(tile / (size_t)ktiles);
+        const int row = 32 * rt + (l & 31), half = l >> 5;
+        const int w0 = 8 * kt + 2 * q;
+        uint32_t s[2] = {0u, 0u};
+        if (row < rows) {
+            if (w0 < words) s[0] = src[(size_t)row * words + w0];
+            if (w0 + 1 < words) s[1] = src[(size_t)row * words + w0 + 1];
+        }
+        uint32_t o = 0;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            const int t = j >> 3, e = j & 7;
+            const int elem = 16 * (t & 1) + 8 * half + e;          // element of source word t >> 1
+            o |= ((s[t >> 1] >> word_bit(elem, src_order)) & 1u) << word_bit(j, 1);
+        }
+        dst[i] = o;
+    }
+}
+
+hipError_t words_to_tiles(const uint32_t* src, uint32_t* dst, int rows, int words, int rows_padded, int k_padded,
+                          int src_order, hipStream_t stream) {
+    const size_t nout = (size_t)rows_padded * k_padded / 32;
+    if (nout == 0) return hipSuccess;
+    size_t blocks = (nout + 255) / 256;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    hipLaunchKernelGGL(words_to_tiles_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, src, dst, rows, words,
+                       k_padded / 256, src_order, nout);
+    return hipGetLastError();
+}
+
 // Tile order of the run-list kernel: 16-byte units (4 words) indexed [row / 32][unit / 4][(row / 16) & 1][unit & 3]
 // [row & 15], rows padded to a multiple of 32 and units to a multiple of 4 with zero words.  The 64 units that
 // one wavefront fetches for an MFMA operand (16 rows x 4 units) are 1 KiB contiguous, the two row groups of a

@@ -21,7 +21,7 @@ import torch.nn.functional as F
 
 from . import ops
 from .runlist import DecodeRunList
-from .packing import (binary_packer, binary_unpacker, marlin_nanoquant_packer, repack_words)
+from .packing import (binary_packer, marlin_nanoquant_packer, pack_binary_marlin_fused_from_words, repack_words)
 
 
 def _sign_pm1(x: torch.Tensor) -> torch.Tensor:
@@ -178,9 +178,26 @@ class NanoQuantLinear(nn.Module):
             rl.add(None, self.scale_pre, V, scale_mid, U, self.scale_post, bias=bias, tiled=tiled, bind_y=True)
             rl.build()
             self._fused_lists[key] = rl
+            # The first launch of a new list is checked (one synchronisation per list): the kernel needs its whole
+            # grid resident at once, and a device shared with other work makes its bounded waits expire.
+            y = torch.empty((rows, self.scale_post.numel()), dtype=self.dtype, device=x.device)
+            rl.run(x=x, y=y)
+            if rl.status() != 0:
+                del self._fused_lists[key]
+                raise RuntimeError("the fused decode launch could not keep its grid resident (is the GPU shared with "
+                                   "other kernels?); set fused_launch = False to use the two-launch operator")
+            return y
         y = torch.empty((rows, self.scale_post.numel()), dtype=self.dtype, device=x.device)
         rl.run(x=x, y=y)
         return y
+
+    def fused_status(self) -> int:
+        """Synchronises.  0 when no fused launch of this module has run into its bounded dependency wait since the
+        last call; 1 otherwise (the outputs of such a launch are invalid).  Reading clears the flag."""
+        worst = 0
+        for rl in self._fused_lists.values():
+            worst = max(worst, rl.status())
+        return worst
 
     def _compute_forward(self, x, V, U, scale_pre, scale_mid, scale_post):
         """Dense definition of the layer (reference: linear.py:248-257)."""
@@ -255,9 +272,10 @@ class NanoQuantLinear(nn.Module):
 
     def load_packed(self, state: dict, prefix: str = "", kernel_type: str = "gemv",
                     dtype: torch.dtype = torch.float16) -> None:
-        """Load a packed checkpoint entry.  For the decode path the `lsb_first` words are permuted to the
-        kernel's `half2` order word by word -- the dense +-1 matrices of the reference's loader
-        (src/nanoquant/utils/load_utils.py:269-293) are never materialised."""
+        """Load a packed checkpoint entry.  The dense +-1 matrices of the reference's loader
+        (src/nanoquant/utils/load_utils.py:269-293) are never materialised: for the decode path the `lsb_first`
+        words are permuted to the kernel's `half2` order word by word, for the prefill path they go to the 32 x 256
+        tiles in one pass over the words (with the rank padding of the reference's packer, kernel/utils.py:262-271)."""
         dev = self.scale_pre.device
         v_shape = tuple(int(v) for v in state[prefix + "V_shape"])
         u_shape = tuple(int(v) for v in state[prefix + "U_shape"])
@@ -270,17 +288,30 @@ class NanoQuantLinear(nn.Module):
                 delattr(self, "scale_mid")
         v_words = state[prefix + "V_packed"].to(dev)
         u_words = state[prefix + "U_packed"].to(dev)
+        if kernel_type not in ("gemv", "gemm"):
+            raise ValueError("kernel_type must be one of ['gemv', 'gemm'].")
+        if u_shape[1] != v_shape[0] or tuple(v_words.shape) != (v_shape[0], (v_shape[1] + 31) // 32) or \
+                tuple(u_words.shape) != (u_shape[0], (u_shape[1] + 31) // 32):
+            raise ValueError("packed factor shapes do not match V_shape / U_shape")
+        for name in ("V", "U"):
+            if hasattr(self, name):
+                delattr(self, name)
+        self.in_features, self.out_features = v_shape[1], u_shape[0]
+        self._fused_lists, self._fused_tiled, self._fused_bias = {}, None, None   # built on the previous words
+        self._prepare_scales_only(dtype)
         if kernel_type == "gemv":
-            for name in ("V", "U"):
-                if hasattr(self, name):
-                    delattr(self, name)
-            self._prepare_scales_only(dtype)
             self.V_int8 = repack_words(v_words, "lsb_first", "half2")
             self.U_int8 = repack_words(u_words, "lsb_first", "half2")
         else:
-            self.V = nn.Parameter(binary_unpacker(v_words, v_shape).to(self.dtype), requires_grad=False)
-            self.U = nn.Parameter(binary_unpacker(u_words, u_shape).to(self.dtype), requires_grad=False)
-            self._prepare_kernel(kernel_type, dtype)
+            if v_shape[1] % 256 != 0 or u_shape[0] % 32 != 0:
+                raise ValueError("the prefill path needs in_features % 256 == 0 and out_features % 32 == 0")
+            self.kernel_type = "gemm"
+            (self.V_int8, self.U_int8, self.s1, self.s2, self.s3, self.workspace) = pack_binary_marlin_fused_from_words(
+                v_words, u_words, self.rank, self.scale_pre.data, None if self.scale_mid is None else self.scale_mid.data,
+                self.scale_post.data, "lsb_first")
+            for key in ["scale_pre", "scale_mid", "scale_post", "kernel_kwargs"]:
+                delattr(self, key)
+            self.kernel_forward = torch.ops.binary_kernels.marlin_nanoquant_forward
 
     def _prepare_scales_only(self, dtype: torch.dtype) -> None:
         self.do_kernel_inference = True

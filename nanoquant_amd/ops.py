@@ -462,6 +462,47 @@ def repack_words_device(packed: torch.Tensor, src: str, dst: str) -> torch.Tenso
     return out
 
 
+def pack_gemm_tiles_device(words: torch.Tensor, rows_padded: int, k_padded: int, method: str) -> torch.Tensor:
+    """Device pass of packing.pack_gemm_tiles_from_words."""
+    rows, nwords = words.shape
+    out = torch.empty(rows_padded * k_padded // 32, dtype=torch.int32, device=words.device)
+    with torch.cuda.device(words.device):
+        _lib.check(_lib.lib().nq_pack_gemm_tiles(_ptr(words), _ptr(out), rows, nwords, rows_padded, k_padded,
+                                                 _lib.ORDER_IDS[method], _stream(words.device)))
+    return out
+
+
+def gemv_stage_forward(inp: torch.Tensor, s_col: Optional[torch.Tensor], bits: torch.Tensor,
+                       s_row: Optional[torch.Tensor]) -> torch.Tensor:
+    """One matmul-free stage on its own: out[b, row] = s_row[row] * sum_c sgn(bits[row, c]) * inp[b, c] * s_col[c]
+    (what one of the reference's two launches computes, kernel/cuda/gemv_kernel.cu:283-301).  `bits` [rows,
+    ceil(cols/32)] in the "half2" order; the result has inp's dtype."""
+    if inp.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("Support only Half or BFloat16")
+    what = _FLOAT_WHAT[inp.dtype]
+    _check_dev_cont(inp, "in", inp.dtype, what)
+    _check_dev_cont(bits, "bits", torch.int32, "tensor dtype must be int32")
+    for name, t in (("s_col", s_col), ("s_row", s_row)):
+        if t is not None:
+            _check_dev_cont(t, name, inp.dtype, what)
+    cols = inp.size(-1)
+    if bits.dim() != 2 or bits.size(1) != (cols + 31) // 32:
+        raise RuntimeError(f"bits must be [rows, {(cols + 31) // 32}] for {cols} input columns")
+    rows = bits.size(0)
+    if (s_col is not None and s_col.numel() != cols) or (s_row is not None and s_row.numel() != rows):
+        raise RuntimeError("scale size mismatch")
+    lead = inp.shape[:-1]
+    batch = 1
+    for d in lead:
+        batch *= d
+    out = torch.empty((batch, rows), dtype=inp.dtype, device=inp.device)
+    if batch > 0 and rows > 0:
+        with torch.cuda.device(inp.device):
+            _lib.check(_lib.lib().nq_gemv_stage(_ptr(inp), _ptr(s_col), _ptr(bits), _ptr(s_row), _ptr(out), batch, cols,
+                                                rows, _dtype_id(inp), _stream(inp.device)))
+    return out.reshape(*lead, rows)
+
+
 def tile_words_device(packed: torch.Tensor, inverse: bool, shape=None) -> torch.Tensor:
     """Device pass of packing.tile_words / untile_words."""
     lib = _lib.lib()

@@ -170,6 +170,31 @@ def pack_gemm_tiles(weight: torch.Tensor) -> torch.Tensor:
     return _bits_to_words(by_position).contiguous()
 
 
+def pack_gemm_tiles_from_words(words: torch.Tensor, rows_padded: int, k_padded: int, method: str = "lsb_first") -> torch.Tensor:
+    """Row-major packed words [rows, ceil(cols/32)] (either word order) -> the "tile32x256" buffer of
+    pack_gemm_tiles for the matrix padded with +1 signs to [rows_padded, k_padded], without a dense +-1 matrix
+    on the device: one pass of `nq_pack_gemm_tiles` over the words (on CPU tensors a bit gather in torch).
+    This is what lets a packed checkpoint (`lsb_first` words, modules/linear.py:288-321 of the reference) be
+    served by the prefill kernels directly; the reference's loader unpacks to dense first
+    (utils/load_utils.py:269-293)."""
+    if words.dtype != torch.int32 or words.dim() != 2:
+        raise TypeError("packed words must be a 2-D int32 tensor")
+    rows, nwords = words.shape
+    if rows_padded % GEMM_TILE_ROWS != 0 or k_padded % GEMM_TILE_K != 0 or rows_padded < rows or k_padded < 32 * nwords:
+        raise ValueError(f"prefill packing needs rows_padded % {GEMM_TILE_ROWS} == 0, k_padded % {GEMM_TILE_K} == 0 and "
+                         f"both at least the source's size, got {rows_padded} x {k_padded} for {rows} x {32 * nwords}")
+    pos = _bit_positions(method, words.device)      # also validates the method name
+    if words.is_cuda:
+        from . import ops
+        return ops.pack_gemm_tiles_device(words.contiguous(), rows_padded, k_padded, method)
+    neg = torch.zeros((rows_padded, k_padded), dtype=torch.uint8)
+    neg[:rows, :32 * nwords] = _words_to_bits(words)[..., pos].reshape(rows, 32 * nwords)
+    neg = neg.view(rows_padded // 32, 32, k_padded // 256, 4, 4, 2, 8).permute(0, 2, 5, 1, 3, 4, 6).reshape(-1, 32)
+    by_position = torch.empty_like(neg)
+    by_position[..., _bit_positions("half2", words.device)] = neg
+    return _bits_to_words(by_position).contiguous()
+
+
 def unpack_gemm_tiles(packed: torch.Tensor, out: int, k: int) -> torch.Tensor:
     """Inverse of pack_gemm_tiles -> int8 {-1,+1} [out, k]."""
     pos = _bit_positions("half2", packed.device)
@@ -213,6 +238,28 @@ def pack_binary_marlin_fused(V_sign: torch.Tensor, U_sign: torch.Tensor, scale_g
     U_bits, _, s_h, ws_u = pack_binary_marlin(U_sign.T.contiguous(), scale_l, scale_h)
     workspace = torch.zeros(max(ws_v, ws_u), device=dev, dtype=torch.int32)
     return V_bits.contiguous(), U_bits.contiguous(), s_g, s_l, s_h, workspace
+
+
+def pack_binary_marlin_fused_from_words(V_words: torch.Tensor, U_words: torch.Tensor, rank: int, scale_g: torch.Tensor,
+                                        scale_l: Optional[torch.Tensor], scale_h: torch.Tensor, method: str = "lsb_first"):
+    """pack_binary_marlin_fused for factors that are already packed row-major words, as a checkpoint holds them
+    (modules/linear.py:288-321): V_words [rank, in/32] (module V, the first stage), U_words [out, ceil(rank/32)]
+    (module U, the second stage).  Same 6-tuple, same rank padding (+1 signs, zero mid scale), bit-identical to
+    packing the unpacked factors -- but the dense +-1 matrices are never formed."""
+    dev = V_words.device
+    n, m = 32 * V_words.shape[1], U_words.shape[0]
+    if V_words.shape[0] != rank or U_words.shape[1] != (rank + 31) // 32:
+        raise ValueError("packed factor shapes do not match the rank")
+    if scale_l is None:
+        scale_l = torch.ones(rank, device=dev, dtype=scale_g.dtype)
+    rank_p = (rank + RANK_MULTIPLE_GEMM - 1) // RANK_MULTIPLE_GEMM * RANK_MULTIPLE_GEMM
+    if rank_p > rank:
+        scale_l = torch.cat([scale_l, torch.zeros(rank_p - rank, device=dev, dtype=scale_l.dtype)], dim=0)
+    V_bits = pack_gemm_tiles_from_words(V_words, rank_p, n, method).view(n // 16, rank_p // 2)
+    U_bits = pack_gemm_tiles_from_words(U_words, m, rank_p, method).view(rank_p // 16, m // 2)
+    workspace = torch.zeros(max(rank_p, m) // 128 * MARLIN_MIN_MAX_PAR, device=dev, dtype=torch.int32)
+    return (V_bits.contiguous(), U_bits.contiguous(), scale_g.reshape(-1).contiguous(), scale_l.reshape(-1).contiguous(),
+            scale_h.reshape(-1).contiguous(), workspace)
 
 
 # aliases used by the reference's callers (utils.py:503-507)

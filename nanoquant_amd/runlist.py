@@ -159,7 +159,8 @@ class DecodeRunList:
         return self.outputs
 
     def status(self) -> int:
-        """Synchronises.  0 = ok; 1 = a dependency wait ran into its bound (results invalid)."""
+        """Synchronises.  0 = ok; 1 = a dependency wait ran into its bound in some launch since the last call (the
+        results of that launch are invalid: the kernel needs the GPU to itself).  Reading clears the flag."""
         out = ctypes.c_int(0)
         with torch.cuda.device(self.device):
             stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
