@@ -7,6 +7,8 @@ which one ran is printed."""
 import numpy as np
 import pytest
 import torch
+import torch._dynamo
+import torch._inductor.config as inductor_config
 
 import nanoquant_amd  # noqa: F401
 from nanoquant_amd.linear import NanoQuantLinear
@@ -27,7 +29,7 @@ class _Stack(torch.nn.Module):
 
 
 def _stack(dev, kernel_type, dtype):
-    dims = [(384, 256, 96), (512, 384, 128), (256, 512, 160)]          # (out, in, rank), chained
+    dims = [(512, 256, 96), (768, 512, 128), (256, 768, 160)]          # (out, in, rank), chained
     mods, terms = [], []
     for i, (m, n, r) in enumerate(dims):
         vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, 2000 + i)
@@ -67,8 +69,6 @@ def test_compiled_stack_matches_the_oracle(dev, kernel_type, rows):
                 torch.cuda.synchronize()
         return outs
 
-    import torch._dynamo
-    import torch._inductor.config as inductor_config
     inductor_config.compile_threads = 1                                # no pool of compile workers beside the GPU process
     torch._dynamo.reset()
     how = "inductor, mode=reduce-overhead"
