@@ -132,7 +132,8 @@ typedef struct nq_linear {
 /* Launch geometry of a built run list; filled by nq_runlist_build, passed back to nq_runlist_run. */
 typedef struct nq_runlist_plan {
     int nlinears, nstages, nphases, workgroups, max_units, batch, dtype, index_words;
-    int bound;              /* bit 0: some x was NULL, bit 1: some y was NULL (nq_runlist_run_bound must supply them) */
+    int bound;              /* bit 0: some x was NULL, bit 1: some y was NULL (nq_runlist_run_bound must supply them);
+                               bit 2: the linears are in tile order (up to batch 4 all linears of a list must agree) */
 } nq_runlist_plan;
 
 size_t nq_runlist_workspace_bytes(const nq_linear* linears, int nlinears);

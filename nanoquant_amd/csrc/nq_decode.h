@@ -464,34 +464,48 @@ __device__ __forceinline__ float4_t pow2_combine(const float4_t (&acc)[kPow2Clas
 }
 
 // ---- one-bit fp4 weights x fp8 pieces of the input (batch 1..4, fp16 and bf16 alike) ---------------
-// v_mfma_f32_16x16x128_f8f6f4 takes an fp4 (e2m1) A operand and an fp8 (e4m3) B operand.  A 4-bit pattern
-// with a single bit set is a valid e2m1 number (0.5, 1, 2 for bit 0, 1, 2; bit 3 is the sign of zero), so
-// `word & 0x11111111 << p` IS the weight operand "c_p * b" of the eight sign bits at position p of the
-// eight nibbles of a packed word: one AND per 32 bits and class (bit 3 goes through a one-bit shift), and
-// one MFMA multiplies 16 rows x 512 columns of signs.  The input is staged as kQ8Pieces fp8 numbers per
-// element, u = x * s * S ~ q0 + q1 + q2 with q_k = fp8(u - q_0 - .. - q_{k-1}) and S a power of two that brings
-// the largest |u| of the staged slice into [128, 256): every piece carries 4 significant bits, three of them
-// reproduce u to 2^-12 relative or 2^-17 of the slice maximum, whichever is larger (fp16 staging keeps 2^-11
-// relative); products are exact and accumulators fp32, but the instruction's internal 128-term sum keeps 13 bits
-// below its largest product (measured), which cuts elements far below the largest of their group at 2^-14 of it.  Pieces and batch rows
+// v_mfma_scale_f32_16x16x128_f8f6f4 takes an fp4 (e2m1) A operand, an fp8 (e4m3) B operand and one power-of-two
+// scale per operand and block of 32 contraction indices.  The eight nibbles of a packed word are eight fp4 numbers,
+// so the sign bits at position p of every nibble ("class" p, eight signs per word) become a weight operand with ONE
+// lane operation:
+//   p = 0, 1, 2:  w & (0x11111111 << p)            nibble = one-hot bit p = 0.5, 1, 2 times the packed bit b
+//   p = 3:        (w & 0x88888888) | 0x22222222     nibble = sign bit b on the number 1.0 = +-1, i.e. 1 - 2 b
+// Four lane operations per 32 signs, and one MFMA multiplies 16 rows x 512 columns of signs.  The signed sum over
+// the columns of the classes 0..2 is (sum of u) - 2 (sum of b u): their input pieces are staged NEGATED and the
+// block scale of the B operand carries the factors 4, 2, 1 that make every class contribute -2 b u, so that all four
+// classes add into one accumulator; (sum of u) over the columns of classes 0..2 is taken once while staging (xtot).
+//
+// The input is staged as kQ8Pieces fp8 numbers per element, u = x * s * S ~ q0 + q1 + q2 with
+// q_k = fp8(u - q_0 - .. - q_{k-1}) (round to nearest, residuals exact in fp32) and S the power of two that brings
+// the largest |u| of the element's UNIT (128 consecutive columns) into [128, 256): one scale per unit and batch
+// row, handed to the MFMA as its block scale, so an outlier lowers the resolution of its own 127 neighbours only.
+// Every piece carries 4 significant bits; three reproduce u to 2^-12 relative or 2^-17 of the unit's maximum,
+// whichever is larger (fp16 staging keeps 2^-11 relative).  Products are exact, accumulators fp32; the
+// instruction's internal 128-term sum keeps 13 bits below its largest product (measured).  Pieces and batch rows
 // are columns of the B operand: column j = b * kQ8Pieces + piece, at most 16.
 //
 // Operand geometry (measured on gfx950 with one-hot operands): lane (i = l & 15, g = l >> 4) supplies
 //   A (fp4, 4 dwords): row i, k = 32 g + idx, idx = 8 t + e for nibble e of dword t;
-//   B (fp8, 8 dwords): column i, k = 64 (idx >> 4) + 16 g + (idx & 15) for byte idx of the 32.
+//   B (fp8, 8 dwords): column i, k = 64 (idx >> 4) + 16 g + (idx & 15) for byte idx of the 32;
+//   B block scale: byte `opsel` of the lane's scale register applies to column i, k = 32 g .. 32 g + 31.
 // With A dword t = word t of the lane's 16-byte unit (unit 4 ub + g of the row), nibble e at class p is bit
 // 4 e + p of that word, i.e. column 32 t + elem(4 e + p) of the unit, elem(b) = b < 16 ? 2 (15 - b) :
 // 2 (31 - b) + 1 (the "half2" order).  So B lane g needs, for class p, the 16 bytes (words 2 (g & 1),
-// 2 (g & 1) + 1; e = 0..7) of unit 4 ub + (g >> 1) and the same of unit 4 ub + 2 + (g >> 1).
+// 2 (g & 1) + 1; e = 0..7) of unit 4 ub + (g >> 1) and the same of unit 4 ub + 2 + (g >> 1), and the scale of
+// lane g is the one of unit 4 ub + g: the four bytes of a lane's scale register are the scales of its unit for
+// class 0..3 (exponent + 2, + 1, + 0, + 0).
 // LDS layout in 16-byte chunks: chunk(j, u, p, hf) = j * pitch + 8 u + 2 p + hf holds, for column j, unit u,
 // class p, the bytes of words 2 hf, 2 hf + 1 (8 bytes each, e = 0..7).  pitch = 8 * units4 + 1 with units4 the
-// number of staged units rounded up to a multiple of 4 (the padding is staged as zeros).
+// number of staged units rounded up to a multiple of 4 (the padding is staged as zeros).  Scales: one dword per
+// batch row and unit.
 constexpr int kQ8Pieces = 3;
 typedef int v8i_t __attribute__((ext_vector_type(8)));
 
 __host__ __device__ constexpr int q8_units4(int units) { return (units + 3) & ~3; }
 __host__ __device__ constexpr int q8_pitch(int units4) { return 8 * units4 + 1; }
 __host__ __device__ constexpr int q8_chunks(int batch, int units4) { return batch * kQ8Pieces * q8_pitch(units4); }
+// 16-byte chunks of unit scales (one dword per batch row and unit) in front of the pieces
+__host__ __device__ constexpr int q8_scale_chunks(int batch, int units4) { return (batch * units4 + 3) / 4; }
 
 template <int CTRL>
 __device__ __forceinline__ uint32_t dpp_mov_u32(uint32_t v) {
@@ -507,30 +521,30 @@ __device__ __forceinline__ uint32_t quad_transpose_rev(uint32_t m, bool odd, boo
     return __builtin_amdgcn_perm(p2, y, upper ? 0x06070203u : 0x00010405u);
 }
 
-// power of two S = 2^(7 - E) for a slice maximum with biased exponent eb = E + 127 (clamped below so that an
-// all-zero slice gives a finite S), and the factor -2 / S that takes an accumulator back
-__device__ __forceinline__ uint32_t q8_exponent(uint32_t max_bits) { return max(max_bits >> 23, 32u); }
+// Biased exponent eb of a unit's largest |u| (clamped so that an all-zero unit, an infinity or a NaN still give
+// finite powers of two), the scale S = 2^(134 - eb) that brings it into [128, 256), its inverse, and the block
+// scale bytes of the four classes: 2^(eb - 134) times 4, 2, 1, 1.
+__device__ __forceinline__ uint32_t q8_exponent(uint32_t max_bits) { return min(max(max_bits >> 23, 32u), 240u); }
 __device__ __forceinline__ float q8_scale(uint32_t eb) { return as_float((261u - eb) << 23); }
-__device__ __forceinline__ float q8_unscale_neg2(uint32_t eb) { return as_float(0x80000000u | ((eb - 6u) << 23)); }
-// the same for accumulators that hold 0.5 * sum b * u
-__device__ __forceinline__ float q8_unscale_neg4(uint32_t eb) { return as_float(0x80000000u | ((eb - 5u) << 23)); }
+__device__ __forceinline__ float q8_inv_scale(uint32_t eb) { return as_float((eb - 7u) << 23); }
+__device__ __forceinline__ uint32_t q8_scale_bytes(uint32_t eb) {
+    const uint32_t e8 = eb - 7u;
+    return (e8 + 2u) | ((e8 + 1u) << 8) | (e8 << 16) | (e8 << 24);
+}
 
-// Stage units [c0, c0 + cu_n) (plus zero padding up to q8_units4(cu_n)) of BATCH rows.  smax[b] (uint32,
-// zeroed by the caller, barrier before) receives the bit pattern of max |u| per batch row, xtot[b] the sum of
-// the staged values.  The wavefronts of the workgroup are divided among the batch rows (nthreads / 64 must be a
-// multiple of BATCH), so a lane reduces maximum and sum over all its chunks before anything crosses lanes.
-// Contains one workgroup barrier; a barrier must follow before the staged data is read.
+// Stage units [c0, c0 + cu_n) (plus zero padding up to q8_units4(cu_n)) of BATCH rows: pieces into xq, unit scales
+// into scl[b * (pitch - 1) / 8 + unit], and xtot[b] (zeroed by the caller, barrier before) += the sum of the staged values in
+// the columns of classes 0..2.  One pass, no barrier inside: a lane holds the 8 columns of one chunk, the 16 lanes
+// of a DPP row hold one unit, so the unit maximum never leaves the row.  A barrier must follow before the staged
+// data is read.
 template <int DT, int BATCH, int THREADS>
-__device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* smax, float* xtot, const StageInput& st, int c0,
+__device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* scl, float* xtot, const StageInput& st, int c0,
                                                int cu_n, int pitch) {
     using E = Elem<DT>;
-    constexpr int nthreads = THREADS;
-    // chunks per lane and round trip.  When a batch row fits into one round trip (16384 columns at batch 1 and 1024
-    // lanes, 8192 at batch 2) the values stay in registers across the barrier; longer inputs are read twice.
-    constexpr int kBurst = 2;
-    const int nchunks = q8_units4(cu_n) * 16;            // 8-column chunks per batch row, a multiple of 64
-    const int tpr = nthreads / BATCH;                    // lanes per batch row
-    const int b = threadIdx.x / tpr, tl = threadIdx.x - b * tpr;
+    constexpr int kBurst = 2;                            // chunks per lane in flight
+    const int units4 = q8_units4(cu_n);
+    const int nchunks = units4 * 16;                     // 8-column chunks per batch row, a multiple of 64
+    const int total = BATCH * nchunks;
     const int lane = threadIdx.x & 63;
     const uint32_t esize = st.in_f32 ? 4u : 2u;
     const bool fast = st.vec_in && (st.K & 7) == 0;
@@ -539,9 +553,10 @@ __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* smax, float*
     const __amdgpu_buffer_rsrc_t rsc = raw_buffer(scaled ? (const void*)st.s_col : st.in, scaled ? (uint32_t)st.K * 2u : 0u);
     const bool coherent = st.in_f32 && st.in_coherent;
 
-    auto issue = [&](int q, u32x4_t& ra, u32x4_t& rb) {
+    auto issue = [&](int it, u32x4_t& ra, u32x4_t& rb) {
+        const int b = it / nchunks, q = it - b * nchunks;
         const int col = c0 * 128 + 8 * q;
-        const bool live = fast && q < nchunks && col < st.K;
+        const bool live = fast && it < total && col < st.K;
         const uint32_t off = live ? (uint32_t)(((size_t)b * st.in_stride + col) * esize) : kPastEnd;
         if (coherent) {
             ra = __builtin_amdgcn_raw_buffer_load_b128(rin, off, 0, kCacheAgentCoherent);
@@ -552,8 +567,8 @@ __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* smax, float*
             else rb = __builtin_amdgcn_raw_buffer_load_b128(rsc, live ? (uint32_t)col * 2u : kPastEnd, 0, kCacheDefault);
         }
     };
-    // the 8 values of chunk q as fp32, input scale applied; running maximum of |v| and sum
-    auto values = [&](int q, const u32x4_t& ra, const u32x4_t& rb, float (&v)[8], float& m, float& tot) {
+    // the 8 values of chunk (b, q) as fp32, input scale applied
+    auto values = [&](int it, const u32x4_t& ra, const u32x4_t& rb, float (&v)[8]) {
         if (fast) {
             if (!st.in_f32) {
 #pragma unroll
@@ -571,11 +586,12 @@ __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* smax, float*
             }
         } else {
             // element-wise fallback: odd K or rows that allow no 16-byte loads
+            const int b = it / nchunks, q = it - b * nchunks;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const int c = c0 * 128 + 8 * q + e;
                 float t = 0.f;
-                if (q < nchunks && c < st.K) {
+                if (it < total && c < st.K) {
                     if (!st.in_f32) {
                         t = E::to_float(((const uint16_t*)st.in)[(size_t)b * st.in_stride + c]);
                         if (st.s_col) t *= E::to_float(st.s_col[c]);
@@ -589,33 +605,25 @@ __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* smax, float*
                 v[e] = t;
             }
         }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            m = fmaxf(m, fabsf(v[e]));
-            tot += v[e];
-        }
     };
-    // wavefront maximum and sum into smax / xtot: one LDS atomic each per wavefront
-    auto publish = [&](float m, float tot) {
+    // chunk (b, q): unit scale, pieces into LDS, and the chunk's share of xtot
+    auto quantize = [&](int it, float (&v)[8]) -> float {
+        const int b = it / nchunks, q = it - b * nchunks;
+        const int cu = q >> 4, t = (q >> 2) & 3, qq = q & 3;
+        float m = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) m = fmaxf(m, fabsf(v[e]));
         uint32_t mb = __builtin_bit_cast(uint32_t, m);
-        mb = max(mb, dpp_mov_u32<0xB1>(mb));
+        mb = max(mb, dpp_mov_u32<0xB1>(mb));                // the 16 lanes of a DPP row hold one unit
         mb = max(mb, dpp_mov_u32<0x4E>(mb));
         mb = max(mb, dpp_mov_u32<0x141>(mb));
         mb = max(mb, dpp_mov_u32<0x140>(mb));
-        mb = max(mb, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mb, 0x142, 0xA, 0xF, false));
-        mb = max(mb, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mb, 0x143, 0xC, 0xF, false));
-        tot = group_sum_tail(tot, 64);
-        if (lane == 63) {
-            atomicMax(&smax[b], mb);
-            atomicAdd(&xtot[b], tot);
-        }
-    };
-    // pieces of chunk q into LDS: q_k = fp8(u - q_0 - .. - q_{k-1}), all on the scale of u
-    auto quantize = [&](int q, float (&v)[8], float S) {
-        const int cu = q >> 4, t = (q >> 2) & 3, qq = q & 3;
+        const uint32_t eb = q8_exponent(mb);
+        const float S = q8_scale(eb);
         float u[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) u[e] = v[e] * S;
+        const float before = ((u[2] + u[3]) + (u[4] + u[5])) + (u[6] + u[7]);
         uint2* dst = (uint2*)xq + 2 * ((size_t)(b * kQ8Pieces) * pitch + 8 * cu + 2 * qq + (t >> 1)) + (t & 1);
 #pragma unroll
         for (int k = 0; k < kQ8Pieces; ++k) {
@@ -624,64 +632,43 @@ __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* smax, float*
             lo = __builtin_amdgcn_cvt_pk_fp8_f32(u[2], u[0], lo, true);
             int hi = __builtin_amdgcn_cvt_pk_fp8_f32(u[7], u[5], 0, false);
             hi = __builtin_amdgcn_cvt_pk_fp8_f32(u[3], u[1], hi, true);
-            if (k + 1 < kQ8Pieces) {
+            {   // residuals: what the following pieces (or nobody) still have to carry
                 const auto l0 = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false), l1 = __builtin_amdgcn_cvt_pk_f32_fp8(lo, true);
                 const auto h0 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false), h1 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
                 u[6] -= l0[0]; u[4] -= l0[1]; u[2] -= l1[0]; u[0] -= l1[1];
                 u[7] -= h0[0]; u[5] -= h0[1]; u[3] -= h1[0]; u[1] -= h1[1];
             }
+            // classes 0..2 ride negated (bytes 0..2 of the packed quadruples)
             uint2 out;
-            out.x = quad_transpose_rev((uint32_t)lo, lane & 1, lane & 2);
-            out.y = quad_transpose_rev((uint32_t)hi, lane & 1, lane & 2);
-            if (q < nchunks) dst[(size_t)k * pitch * 2] = out;
+            out.x = quad_transpose_rev((uint32_t)lo ^ 0x00808080u, lane & 1, lane & 2);
+            out.y = quad_transpose_rev((uint32_t)hi ^ 0x00808080u, lane & 1, lane & 2);
+            if (it < total) dst[(size_t)k * pitch * 2] = out;
         }
+        if (it < total && (q & 15) == 0) scl[b * ((pitch - 1) >> 3) + cu] = q8_scale_bytes(eb);
+        // sum of the staged values (= input - last residual) over the columns of classes 0..2, in the input's units
+        const float after = ((u[2] + u[3]) + (u[4] + u[5])) + (u[6] + u[7]);
+        return (before - after) * q8_inv_scale(eb);
     };
 
-    if (nchunks <= tpr * kBurst) {
-        // everything in one round trip; the values stay in registers across the barrier
+#pragma unroll 1
+    for (int it0 = threadIdx.x; it0 - lane < total; it0 += kBurst * THREADS) {     // wave-uniform trip count
         u32x4_t ra[kBurst], rb[kBurst];
-        float v[kBurst][8];
-        float m = 0.f, tot = 0.f;
 #pragma unroll
-        for (int j = 0; j < kBurst; ++j) issue(tl + j * tpr, ra[j], rb[j]);
-#pragma unroll
-        for (int j = 0; j < kBurst; ++j) values(tl + j * tpr, ra[j], rb[j], v[j], m, tot);
-        publish(m, tot);
-        lds_barrier();
-        const float S = q8_scale(q8_exponent(smax[b]));
+        for (int j = 0; j < kBurst; ++j) issue(it0 + j * THREADS, ra[j], rb[j]);
+        float tot[kBurst];
 #pragma unroll
         for (int j = 0; j < kBurst; ++j) {
-            const int q = tl + j * tpr;
-            if (q - lane < nchunks) quantize(q, v[j], S);
-        }
-    } else {
-        // long inputs: one pass for the maximum, a second one (re-reading the input) for the pieces, kBurst chunks
-        // per lane and round trip
-        float m = 0.f, tot = 0.f;
-#pragma unroll 1
-        for (int q0 = tl; q0 - lane < nchunks; q0 += kBurst * tpr) {
-            u32x4_t ra[kBurst], rb[kBurst];
             float v[8];
-#pragma unroll
-            for (int j = 0; j < kBurst; ++j) issue(q0 + j * tpr, ra[j], rb[j]);
-#pragma unroll
-            for (int j = 0; j < kBurst; ++j) values(q0 + j * tpr, ra[j], rb[j], v, m, tot);
+            values(it0 + j * THREADS, ra[j], rb[j], v);
+            tot[j] = quantize(it0 + j * THREADS, v);
         }
-        publish(m, tot);
-        lds_barrier();
-        const float S = q8_scale(q8_exponent(smax[b]));
-#pragma unroll 1
-        for (int q0 = tl; q0 - lane < nchunks; q0 += kBurst * tpr) {
-            u32x4_t ra[kBurst], rb[kBurst];
+        // a wavefront's 64 chunks belong to one batch row (nchunks is a multiple of 64): one LDS atomic per
+        // wavefront and burst slot
 #pragma unroll
-            for (int j = 0; j < kBurst; ++j) issue(q0 + j * tpr, ra[j], rb[j]);
-#pragma unroll
-            for (int j = 0; j < kBurst; ++j) {
-                float v[8], m2 = 0.f, t2 = 0.f;
-                const int q = q0 + j * tpr;
-                values(q, ra[j], rb[j], v, m2, t2);
-                if (q - lane < nchunks) quantize(q, v, S);
-            }
+        for (int j = 0; j < kBurst; ++j) {
+            const int it = it0 + j * THREADS;
+            const float t = group_sum_tail(tot[j], 64);
+            if (lane == 63 && it - lane < total) atomicAdd(&xtot[(it - lane) / nchunks], t);
         }
     }
 }
@@ -701,27 +688,30 @@ __device__ __forceinline__ void q8_read_operand(Q8Operand& o, const uint4* bp) {
     o.lo3 = p[6]; o.hi3 = p[22];
 }
 
-// One class of two row groups that share the input operand: (w >> P) & 0x11111111 is the fp4 operand of
-// value 0.5 per set bit whatever the class, so all four classes add into ONE accumulator per row group; the two
-// row groups alternate, which keeps dependent MFMAs two issues apart.
+// One class of two row groups that share the input operand; `scale` holds the lane's four class scales, byte P is
+// picked by the instruction.  All four classes add into ONE accumulator per row group; the two row groups
+// alternate, which keeps dependent MFMAs two issues apart.
 template <int P>
 __device__ __forceinline__ void q8_class_pair(const uint4& wa, const uint4& wb, const u32x4_t& lo, const u32x4_t& hi,
-                                              float4_t& acc_a, float4_t& acc_b) {
-    constexpr uint32_t M = 0x11111111u;
+                                              int scale, float4_t& acc_a, float4_t& acc_b) {
+    constexpr uint32_t M = 0x11111111u << P;
+    constexpr uint32_t C = P == 3 ? 0x22222222u : 0u;   // P == 3: the packed bit is the sign of 1.0
+    constexpr int kOneScale = 0x7F7F7F7F;               // 2^0 for the weights
     const v8i_t b = {(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-    const v8i_t aa = {(int)((wa.x >> P) & M), (int)((wa.y >> P) & M), (int)((wa.z >> P) & M), (int)((wa.w >> P) & M), 0, 0, 0, 0};
-    const v8i_t ab = {(int)((wb.x >> P) & M), (int)((wb.y >> P) & M), (int)((wb.z >> P) & M), (int)((wb.w >> P) & M), 0, 0, 0, 0};
-    acc_a = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aa, b, acc_a, 4 /* A: fp4 */, 0 /* B: fp8 */, 0, 0, 0, 0);
-    acc_b = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ab, b, acc_b, 4, 0, 0, 0, 0, 0);
+    const v8i_t aa = {(int)((wa.x & M) | C), (int)((wa.y & M) | C), (int)((wa.z & M) | C), (int)((wa.w & M) | C), 0, 0, 0, 0};
+    const v8i_t ab = {(int)((wb.x & M) | C), (int)((wb.y & M) | C), (int)((wb.z & M) | C), (int)((wb.w & M) | C), 0, 0, 0, 0};
+    acc_a = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aa, b, acc_a, 4 /* A: fp4 */, 0 /* B: fp8 */, 0, kOneScale, P, scale);
+    acc_b = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ab, b, acc_b, 4, 0, 0, kOneScale, P, scale);
 }
 
-// acc += 0.5 * sum b * u per (row, column) of the lane, for the units wa / wb of two row groups 16 rows apart
-__device__ __forceinline__ void unit_mfma_q8_pair(const uint4& wa, const uint4& wb, const Q8Operand& o, float4_t& acc_a,
-                                                  float4_t& acc_b) {
-    q8_class_pair<0>(wa, wb, o.lo0, o.hi0, acc_a, acc_b);
-    q8_class_pair<1>(wa, wb, o.lo1, o.hi1, acc_a, acc_b);
-    q8_class_pair<2>(wa, wb, o.lo2, o.hi2, acc_a, acc_b);
-    q8_class_pair<3>(wa, wb, o.lo3, o.hi3, acc_a, acc_b);
+// acc += the signed sum (less the staged total of classes 0..2) per (row, column) of the lane, for the units
+// wa / wb of two row groups 16 rows apart
+__device__ __forceinline__ void unit_mfma_q8_pair(const uint4& wa, const uint4& wb, const Q8Operand& o, int scale,
+                                                  float4_t& acc_a, float4_t& acc_b) {
+    q8_class_pair<0>(wa, wb, o.lo0, o.hi0, scale, acc_a, acc_b);
+    q8_class_pair<1>(wa, wb, o.lo1, o.hi1, scale, acc_a, acc_b);
+    q8_class_pair<2>(wa, wb, o.lo2, o.hi2, scale, acc_a, acc_b);
+    q8_class_pair<3>(wa, wb, o.lo3, o.hi3, scale, acc_a, acc_b);
 }
 
 // Sum over the kQ8Pieces neighbouring columns of a batch row; valid in the lane of the last piece.

@@ -47,7 +47,8 @@ int stream_chunk_cap(int dtype, int batch, int max_units);
 int stream_row_granule(int dtype, int batch);
 hipError_t gemv_stream(int dtype, int batch, const RunStage* stages, int nstages, int nphases, const int* seg_index,
                        const RunSegment* segs, unsigned long long* counters, unsigned* status, int nwg, int max_units,
-                       hipStream_t stream, const void* ext_in = nullptr, void* ext_out = nullptr);
+                       hipStream_t stream, const void* ext_in = nullptr, void* ext_out = nullptr, bool tiled = false);
+bool stream_needs_uniform_order(int dtype, int batch);
 
 // One stage on its own through the run-list kernel (no tables, no counters); batch 16 only.
 hipError_t gemv_stream_single(int dtype, int batch, const RunStage& st, hipStream_t stream);

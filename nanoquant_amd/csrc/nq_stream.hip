@@ -93,8 +93,7 @@ __device__ __forceinline__ void trim_unit(const BitsView& v, uint4& w, int unit)
     }
 }
 
-// Bytes of LDS in front of the staged input: row sums, the input totals [16] and the per-row maxima of the fp4 x
-// fp8 path [16].
+// Bytes of LDS in front of the staged input: row sums and two sets of input totals [2][16].
 __host__ __device__ constexpr size_t stream_head_bytes(int batch, int arith) {
     (void)arith;
     return (size_t)row_block(batch) * batch * sizeof(float) + 128;
@@ -104,7 +103,9 @@ __host__ __device__ constexpr size_t stream_head_bytes(int batch, int arith) {
 __host__ __device__ __forceinline__ int mfma_items_per_wave(int nitems, int waves) { return (nitems + waves - 1) / waves; }
 
 // ARITH: 1 = MFMA with 16-bit operands, 2 = MFMA with one-bit fp4 weights and fp8 pieces of the input (batch <= 4).
-template <int DT, int BATCH, int ARITH, int THREADS, bool SINGLE>
+// TILED (fp4 x fp8 arithmetic only): every stage of the list has its words in tile order; the 16-bit arithmetic reads
+// either order, stage by stage.
+template <int DT, int BATCH, int ARITH, int THREADS, bool SINGLE, bool TILED>
 __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __restrict__ stages, int nstages,
                                                                      int nphases, const int* __restrict__ seg_index,
                                                                      const RunSegment* __restrict__ segs,
@@ -123,13 +124,16 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
     constexpr bool kTotals = kPow2Mfma || kQ8;                  // signed sum = (sum of x) - 2 (sum of b x)
     static_assert(!kQ8 || BATCH * kQ8Pieces <= 16, "pieces of all batch rows must fit the 16 operand columns");
     float* racc = (float*)lds_raw;                              // [kRowBlock][BATCH] row sums
-    float* xtot = racc + kRowBlock * BATCH;                     // [16] sum of the staged input per batch row
-    uint32_t* smax = (uint32_t*)(xtot + 16);                    // kQ8: [16] largest |input| per batch row (bits)
-    uint4* xs = lds_raw + stream_head_bytes(BATCH, ARITH) / sizeof(uint4);
+    // [2][16] sum of the staged input per batch row; slices alternate between the two, so that the one of the next
+    // slice is cleared a barrier ahead of its staging instead of costing a barrier of its own
+    float* xtot_base = racc + kRowBlock * BATCH;
+    uint4* xs_base = lds_raw + stream_head_bytes(BATCH, ARITH) / sizeof(uint4);
     __shared__ int s_flag;
     const int tid = threadIdx.x;
     const int wg = blockIdx.x;
     if (tid == 0) s_flag = 0;
+    if (tid < 32) xtot_base[tid] = 0.f;
+    int slice_count = 0;
 
     // Which launch of this run list is this?  Needed only by waiting slices; the load is issued now and
     // its latency is hidden behind phase 0.
@@ -171,6 +175,12 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
             const int chunk_units = min(st.units, chunk_cap);
             const int upad = kQ8 ? q8_pitch(q8_units4(chunk_units)) : (chunk_units | 1);
             const bool one_chunk = chunk_units == st.units;
+            float* xtot = xtot_base + 16 * (slice_count & 1);
+            float* xtot_other = xtot_base + 16 * ((slice_count + 1) & 1);
+            ++slice_count;
+            // kQ8: the unit scales (one dword per batch row and staged unit) sit in front of the pieces
+            uint32_t* scl = (uint32_t*)xs_base;
+            uint4* xs = xs_base + (kQ8 ? q8_scale_chunks(BATCH, q8_units4(chunk_units)) : 0);
             StageInput sin;
             sin.in = st.in; sin.s_col = st.s_col; sin.K = st.K; sin.in_stride = st.in_stride;
             sin.in_f32 = st.in_f32; sin.in_coherent = st.in_coherent; sin.vec_in = st.vec_in;
@@ -179,8 +189,53 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
             // path: its staging needs the registers, and holding fetched words across it (measured with one, two and
             // three items per wavefront) costs more in spills than the head start gains.
             uint4 wnext = make_uint4(0, 0, 0, 0);
+            // kQ8: fetch cursor of this wavefront over its items = (pair of 16-row groups, 4-unit group) of the
+            // current (row block, input chunk), unit group fastest, and the three item fetches it keeps in flight
+            const int qlane = tid & 63;
+            const int qwave = __builtin_amdgcn_readfirstlane(tid >> 6);           // scalar item arithmetic
+            int q_ngroups = 1, q_it_begin = 0, q_it_end = 0, q_it_f = 0, q_rp_f = 0, q_ub_f = 0, q_rb = 0, q_c0 = 0, q_cu_n = 0, q_nr = 0;
+            uint4 wa0 = make_uint4(0, 0, 0, 0), wb0 = wa0, wa1 = wa0, wb1 = wa0, wa2 = wa0, wb2 = wa0;
+            auto q_setup = [&](int rb, int c0) {
+                q_nr = min(seg.row_end - rb, kRowBlock);
+                q_cu_n = min(chunk_units, st.units - c0);
+                q_ngroups = (q_cu_n + 3) >> 2;
+                const int nitems = q_ngroups * ((q_nr + 31) >> 5);
+                const int per = mfma_items_per_wave(nitems, kWaves);
+                q_it_begin = qwave * per;
+                q_it_end = min(q_it_begin + per, nitems);
+                q_it_f = q_it_begin;
+                q_rp_f = q_it_begin / q_ngroups;
+                q_ub_f = q_it_begin - q_rp_f * q_ngroups;
+                q_rb = rb;
+                q_c0 = c0;
+            };
+            auto q_fetch = [&](uint4& wa, uint4& wb) {
+                const bool live = q_it_f < q_it_end;
+                if constexpr (TILED) {
+                    // tile order: an item is 2 KiB contiguous (row group a, then b), lane l owns bytes 16 l of each half:
+                    // the address is a scalar item offset plus a lane constant, no lane arithmetic per fetch
+                    const uint32_t item = (uint32_t)((q_rb >> 5) + q_rp_f) * (uint32_t)bv.groups + (uint32_t)((q_c0 >> 2) + q_ub_f);
+                    const uint32_t soff = live ? item * 2048u : 0u;
+                    const uint32_t voff = live ? (uint32_t)qlane * 16u : kPastEnd;
+                    const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(bv.rsrc, voff, soff, 2 /* nt */);
+                    const u32x4_t b = __builtin_amdgcn_raw_buffer_load_b128(bv.rsrc, voff + 1024u, soff, 2 /* nt */);
+                    wa = make_uint4(a.x, a.y, a.z, a.w);
+                    wb = make_uint4(b.x, b.y, b.z, b.w);
+                } else {
+                    const int u = 4 * q_ub_f + (qlane >> 4);
+                    const int row = q_rb + 32 * q_rp_f + (qlane & 15);
+                    const bool ok = live && u < q_cu_n;
+                    wa = load_unit(bv, min(row, st.rows - 1), q_c0 + u, ok);
+                    wb = load_unit(bv, min(row + 16, st.rows - 1), q_c0 + u, ok);
+                }
+                ++q_it_f;
+                if (++q_ub_f == q_ngroups) { q_ub_f = 0; ++q_rp_f; }
+            };
             if constexpr (kQ8) {
-                // nothing: see the loop (registers are scarcer than the head start is worth)
+                // The packed words depend on nothing: the first three items of the slice are asked for before the
+                // dependency wait and the staging of the input, and arrive while those run.
+                q_setup(seg.row_begin, 0);
+                q_fetch(wa0, wb0); q_fetch(wa1, wb1); q_fetch(wa2, wb2);
             } else {
                 // wavefront w starts with item w of the first row block: 16 rows x 4 units, lane (row l & 15,
                 // unit l >> 4)
@@ -231,6 +286,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
             }
             lds_barrier();                                       // s_flag; previous slice is done with xs / racc
             aborted = aborted || (s_flag != 0);
+            if (tid < 16) xtot_other[tid] = 0.f;                 // every reader of it (the previous slice) is past the barrier
 
             if (!aborted) {
                 bool staged = false;
@@ -243,13 +299,14 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                         const int cu_n = min(chunk_units, st.units - c0);
                         if (!(one_chunk && staged)) {
                             if (c0) lds_barrier();
-                            if (kTotals && (c0 == 0 || kQ8)) {
-                                // every reader of the previous totals has passed a barrier by now
-                                if (tid < 16 && c0 == 0) xtot[tid] = 0.f;
-                                if (kQ8 && tid >= 16 && tid < 32) smax[tid - 16] = 0u;
+                            if (kTotals && c0 == 0 && staged) {
+                                // the input is staged again for a further row block: the totals start over (the first
+                                // staging of a slice finds them cleared a barrier ahead); every reader of the previous
+                                // totals has passed a barrier by now
+                                if (tid < 16) xtot[tid] = 0.f;
                                 lds_barrier();
                             }
-                            if constexpr (kQ8) stage_units_q8<DT, BATCH, THREADS>(xs, smax, xtot, sin, c0, cu_n, upad);
+                            if constexpr (kQ8) stage_units_q8<DT, BATCH, THREADS>(xs, scl, xtot, sin, c0, cu_n, upad);
                             else stage_units<DT, BATCH, kPow2Mfma>(xs, nullptr, sin, c0, cu_n, upad, kStreamThreads,
                                                                    kPow2Mfma ? xtot : nullptr);
                             staged = true;
@@ -260,63 +317,56 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                             // operand (eight 16-byte LDS reads per lane) serves two row groups, and a wavefront takes a
                             // contiguous run of items, so it adds its two accumulators to the row sums only when the
                             // pair changes (LDS float atomics cost about 2.5 cycles per lane).
-                            const int lane = tid & 63, r16 = lane & 15, g = lane >> 4;
-                            const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar item arithmetic
-                            const int ngroups = (cu_n + 3) >> 2, nrp = (nr + 31) >> 5;
-                            const int nitems = ngroups * nrp;
-                            const int per = mfma_items_per_wave(nitems, kWaves);
-                            const int it_begin = wave * per, it_end = min(it_begin + per, nitems);
-                            // operand column of this lane (batch row, piece), its first chunk, and the factor that takes
-                            // an accumulator back to the unscaled signed sum; columns beyond the last piece are never
-                            // read back, so their lanes skip the LDS reads (40 % less LDS time per read)
+                            const int r16 = qlane & 15, g = qlane >> 4;
+                            if (rb != seg.row_begin || c0 != 0) {        // the first pass was set up ahead of the wait
+                                q_setup(rb, c0);
+                                q_fetch(wa0, wb0); q_fetch(wa1, wb1); q_fetch(wa2, wb2);
+                            }
+                            const int ngroups = q_ngroups, it_begin = q_it_begin, it_end = q_it_end;
+                            // operand column of this lane (batch row, piece) and its first chunk; columns beyond the
+                            // last piece are never read back, so their lanes skip the LDS reads (40 % less LDS time)
                             const bool qlive = r16 < BATCH * kQ8Pieces;
                             const int qcol = min(r16, BATCH * kQ8Pieces - 1);
                             const uint4* qbase = xs + (size_t)qcol * upad + 8 * (g >> 1) + (g & 1);
-                            const float qfac = q8_unscale_neg4(q8_exponent(smax[qcol / kQ8Pieces]));
+                            // the lane's block scale: the four class bytes of unit 4 ub + g of its batch row
+                            const uint32_t* qscl = scl + (qcol / kQ8Pieces) * ((upad - 1) >> 3) + g;
                             const bool qlast = qlive && r16 % kQ8Pieces == kQ8Pieces - 1;   // holds the sum over the pieces
                             float* rdst = racc + (4 * g) * BATCH + qcol / kQ8Pieces;
-                            // fetch cursor (kQ8Depth items ahead) and compute cursor, advanced without divisions
-                            int it_f = it_begin, rp_f = it_begin / ngroups, ub_f = it_begin - rp_f * ngroups;
-                            int rp = rp_f, ub = ub_f;
-                            auto fetch = [&](uint4& wa, uint4& wb) {
-                                const int u = 4 * ub_f + g;
-                                const int row = rb + 32 * rp_f + r16;
-                                const bool live = it_f < it_end && u < cu_n;
-                                wa = load_unit(bv, min(row, st.rows - 1), c0 + u, live);
-                                wb = load_unit(bv, min(row + 16, st.rows - 1), c0 + u, live);
-                                ++it_f;
-                                if (++ub_f == ngroups) { ub_f = 0; ++rp_f; }
-                            };
-                            // kQ8Depth register pairs in rotation, each refilled right after its use: nothing in flight
-                            // is ever copied, and the main loop has no early exit.
-                            static_assert(kQ8Depth == 3, "the rotation below is written out for three register pairs");
-                            uint4 wa0, wb0, wa1, wb1, wa2, wb2;
-                            fetch(wa0, wb0); fetch(wa1, wb1); fetch(wa2, wb2);
+                            int rp = it_begin / ngroups, ub = it_begin - rp * ngroups;      // compute cursor
                             Q8Operand opnd = {};
+                            int qscale = 0x7F7F7F7F;
                             float4_t acc_a = {0.f, 0.f, 0.f, 0.f}, acc_b = {0.f, 0.f, 0.f, 0.f};
                             int rp_run = rp;
                             auto flush = [&]() {
                                 // acc[v] = partial sum of row 32 rp_run + 4 g + v (acc_b: 16 rows further) for column r16
 #pragma unroll
                                 for (int v = 0; v < 4; ++v) {
-                                    const float sa = q8_piece_sum(acc_a[v] * qfac), sb = q8_piece_sum(acc_b[v] * qfac);
+                                    const float sa = q8_piece_sum(acc_a[v]), sb = q8_piece_sum(acc_b[v]);
                                     const int row = 32 * rp_run + 4 * g + v;
                                     if (qlast && row < nr) atomicAdd(&rdst[(32 * rp_run + v) * BATCH], sa);
                                     if (qlast && row + 16 < nr) atomicAdd(&rdst[(32 * rp_run + 16 + v) * BATCH], sb);
                                 }
                             };
+                            // three register pairs in rotation, each refilled right after its use: nothing in flight
+                            // is ever copied, and the main loop has no early exit
+                            static_assert(kQ8Depth == 3, "the rotation below is written out for three register pairs");
                             auto step = [&](uint4& wa, uint4& wb) {
                                 if (rp != rp_run) {
                                     flush();
                                     acc_a = acc_b = (float4_t){0.f, 0.f, 0.f, 0.f};
                                     rp_run = rp;
                                 }
-                                if (qlive) q8_read_operand(opnd, qbase + 32 * ub);
-                                trim_unit(bv, wa, c0 + 4 * ub + g);       // w = 0 beyond cu_n, padding staged as 0
-                                trim_unit(bv, wb, c0 + 4 * ub + g);
-                                unit_mfma_q8_pair(wa, wb, opnd, acc_a, acc_b);
+                                if (qlive) {
+                                    q8_read_operand(opnd, qbase + 32 * ub);
+                                    qscale = (int)qscl[4 * ub];
+                                }
+                                if constexpr (!TILED) {
+                                    trim_unit(bv, wa, c0 + 4 * ub + g);   // w = 0 beyond cu_n, padding staged as 0
+                                    trim_unit(bv, wb, c0 + 4 * ub + g);
+                                }
+                                unit_mfma_q8_pair(wa, wb, opnd, qscale, acc_a, acc_b);
                                 if (++ub == ngroups) { ub = 0; ++rp; }
-                                fetch(wa, wb);
+                                q_fetch(wa, wb);
                             };
                             int it = it_begin;
 #pragma unroll 1
@@ -325,7 +375,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                             }
                             if (it < it_end) step(wa0, wb0);
                             if (it + 1 < it_end) step(wa1, wb1);
-                            if (it_begin < it_end) flush();              // + sum of x at the end
+                            if (it_begin < it_end) flush();              // + the staged total of classes 0..2 at the end
                         } else {
                             // Items = (16-row group, 4-unit group), unit group fastest; every wavefront takes a
                             // contiguous run of items, so it mostly stays on one row group and adds its
@@ -438,11 +488,12 @@ static void stream_lds_plan(int batch, int arith, int max_units, int* chunk_cap_
     const int racc_bytes = (int)stream_head_bytes(batch, arith);
     if (arith == 2) {
         // kQ8Pieces bytes per column and batch row, staged in whole groups of four units
-        int chunk_cap = (kStreamLdsMax - racc_bytes - batch * kQ8Pieces * (int)sizeof(uint4)) / (batch * kQ8Pieces * 128);
+        // plus one scale dword per batch row and unit
+        int chunk_cap = (kStreamLdsMax - racc_bytes - batch * kQ8Pieces * (int)sizeof(uint4) - 16) / (batch * (kQ8Pieces * 128 + 4));
         chunk_cap &= ~3;
         const int chunk_units = max_units < chunk_cap ? max_units : chunk_cap;
         *chunk_cap_out = chunk_cap;
-        *lds_out = (size_t)racc_bytes + (size_t)q8_chunks(batch, q8_units4(chunk_units)) * sizeof(uint4);
+        *lds_out = (size_t)racc_bytes + (size_t)(q8_scale_chunks(batch, q8_units4(chunk_units)) + q8_chunks(batch, q8_units4(chunk_units))) * sizeof(uint4);
         return;
     }
     int chunk_cap = (kStreamLdsMax - racc_bytes - batch * (int)sizeof(uint4)) / (batch * 16 * (int)sizeof(uint4));
@@ -476,8 +527,9 @@ template <int DT, int BATCH>
 struct StreamKernel {
     static constexpr int kArith = NQ_STREAM_ARITH(DT, BATCH);
     static constexpr int kThreads = NQ_STREAM_THREADS(DT, BATCH);
-    static constexpr auto fn = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false>;
-    static constexpr auto fn_single = gemv_stream_kernel<DT, BATCH, kArith, kThreads, true>;
+    static constexpr auto fn = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, false>;
+    static constexpr auto fn_tiled = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2>;
+    static constexpr auto fn_single = gemv_stream_kernel<DT, BATCH, kArith, kThreads, true, false>;
 };
 
 template <int DT, int BATCH>
@@ -486,6 +538,9 @@ static hipError_t prepare_kernel(size_t lds) {
     if (lds > 64 * 1024 && !attr_done) {
         hipError_t e = hipFuncSetAttribute((const void*)StreamKernel<DT, BATCH>::fn,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute((const void*)StreamKernel<DT, BATCH>::fn_tiled,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
         if (e != hipSuccess) return e;
         attr_done = true;
     }
@@ -510,15 +565,19 @@ static int capacity_of(int max_units) {
 template <int DT, int BATCH>
 static hipError_t launch_stream(const RunStage* stages, int nstages, int nphases, const int* seg_index,
                                 const RunSegment* segs, unsigned long long* counters, unsigned* status, int nwg,
-                                int max_units, hipStream_t stream, const void* ext_in, void* ext_out) {
+                                int max_units, hipStream_t stream, const void* ext_in, void* ext_out, bool tiled) {
     int chunk_cap;
     size_t lds;
     stream_lds_plan(BATCH, StreamKernel<DT, BATCH>::kArith, max_units, &chunk_cap, &lds);
     hipError_t e = prepare_kernel<DT, BATCH>(lds);
     if (e != hipSuccess) return e;
     using SK = StreamKernel<DT, BATCH>;
-    hipLaunchKernelGGL((SK::fn), dim3(nwg), dim3(SK::kThreads), lds, stream, stages, nstages,
-                       nphases, seg_index, segs, counters, status, (unsigned)(1u << 21), chunk_cap, RunStage{}, 0, ext_in, ext_out);
+    if (tiled && SK::kArith == 2)
+        hipLaunchKernelGGL((SK::fn_tiled), dim3(nwg), dim3(SK::kThreads), lds, stream, stages, nstages,
+                           nphases, seg_index, segs, counters, status, (unsigned)(1u << 21), chunk_cap, RunStage{}, 0, ext_in, ext_out);
+    else
+        hipLaunchKernelGGL((SK::fn), dim3(nwg), dim3(SK::kThreads), lds, stream, stages, nstages,
+                           nphases, seg_index, segs, counters, status, (unsigned)(1u << 21), chunk_cap, RunStage{}, 0, ext_in, ext_out);
     return hipGetLastError();
 }
 
@@ -592,6 +651,14 @@ int stream_chunk_cap(int dtype, int batch, int max_units) {
     return 0;
 }
 
+// The fp4 x fp8 arithmetic has one kernel per word order: all stages of such a list must agree.
+bool stream_needs_uniform_order(int dtype, int batch) {
+#define NQ_UNI(D, B) (StreamKernel<D, B>::kArith == 2)
+    NQ_STREAM_DISPATCH(NQ_UNI)
+#undef NQ_UNI
+    return false;
+}
+
 // Rows that one wave-load spans: slices of tile-order stages are cut at multiples of it.
 int stream_row_granule(int dtype, int batch) {
 #define NQ_GRAN(D, B) (StreamKernel<D, B>::kArith == 2 ? 32 : 16)
@@ -602,8 +669,8 @@ int stream_row_granule(int dtype, int batch) {
 
 hipError_t gemv_stream(int dtype, int batch, const RunStage* stages, int nstages, int nphases, const int* seg_index,
                        const RunSegment* segs, unsigned long long* counters, unsigned* status, int nwg, int max_units,
-                       hipStream_t stream, const void* ext_in, void* ext_out) {
-#define NQ_RUN(D, B) launch_stream<D, B>(stages, nstages, nphases, seg_index, segs, counters, status, nwg, max_units, stream, ext_in, ext_out)
+                       hipStream_t stream, const void* ext_in, void* ext_out, bool tiled) {
+#define NQ_RUN(D, B) launch_stream<D, B>(stages, nstages, nphases, seg_index, segs, counters, status, nwg, max_units, stream, ext_in, ext_out, tiled)
     NQ_STREAM_DISPATCH(NQ_RUN)
 #undef NQ_RUN
     return hipErrorInvalidValue;

@@ -284,17 +284,20 @@ def fp8_pieces(u, pieces: int = 3) -> np.ndarray:
     return np.stack(out)
 
 
-def staged_input(v, pieces: int = 3) -> np.ndarray:
-    """What the run-list kernel multiplies the signs with, per row of v [batch, K]: v scaled by the power of two
-    S that brings max |v| of the row into [128, 256), cut into fp8 pieces, summed and scaled back."""
+def staged_input(v, pieces: int = 3, block: int = 128) -> np.ndarray:
+    """What the run-list kernel multiplies the signs with, per row of v [batch, K]: every block of 128 consecutive
+    columns (one 16-byte unit of packed signs) scaled by the power of two S that brings its max |v| into [128, 256),
+    cut into fp8 pieces, summed and scaled back."""
     v = np.asarray(v, dtype=np.float64)
     out = np.zeros_like(v)
     for b in range(v.shape[0]):
-        mx = np.abs(v[b]).max()
-        if mx == 0:
-            continue
-        s = np.exp2(7 - np.floor(np.log2(mx)))
-        out[b] = fp8_pieces(v[b] * s, pieces).sum(axis=0) / s
+        for c in range(0, v.shape[1], block):
+            seg = v[b, c:c + block]
+            mx = np.abs(seg).max()
+            if mx == 0:
+                continue
+            s = np.exp2(7 - np.floor(np.log2(mx)))
+            out[b, c:c + block] = fp8_pieces(seg * s, pieces).sum(axis=0) / s
     return out
 
 
