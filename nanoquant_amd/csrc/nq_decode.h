@@ -673,6 +673,17 @@ __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* scl, float* 
     }
 }
 
+// One pass of a wavefront over a (row block, input chunk) of a stage whose words are in tile order: where its items
+// lie and how many there are.  All members are wave-uniform.
+struct Q8Pass {
+    const uint32_t* bits;           // the stage's packed words
+    uint32_t bytes;                 // their size
+    int item_base;                  // item index of (first row pair, first unit group) of the pass; an item is the 2 KiB
+                                    // at item index * 2048, the items of a row pair are consecutive
+    int ngroups, skip;              // unit groups of the pass, and of the stage's rows outside the pass
+    int it_begin, count;            // this wavefront's items: [it_begin, it_begin + count) of the pass, unit group fastest
+};
+
 // The B operand of one unit group held in registers: per class p the two 16-byte halves read from
 // xq + column * pitch + 8 * (4 ub + (g >> 1)) + (g & 1) + 2 p (lo) and 16 chunks further (hi).  Named native
 // vectors on purpose: arrays of uint4 captured by a lambda end up in scratch memory.

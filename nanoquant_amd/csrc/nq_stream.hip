@@ -148,6 +148,62 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
     }
     bool aborted = false;
 
+    // fp4 x fp8 arithmetic: the three item fetches (2 KB of packed words each) that a wavefront keeps in flight.  In
+    // tile order they run on across passes and slices: while a wavefront works off the last items of a pass, its
+    // refills already ask for the first items of the next pass (next input chunk, next row block or next slice --
+    // packed words depend on nothing), so the stream does not stop for the epilogue, the dependency wait and the
+    // staging in between.  A pass is walked in P = 3 ceil(max(items, 3) / 3) positions (positions past the last
+    // item only refill), so the rotation of the three register pairs starts every pass at pair 0.
+    const int qlane = tid & 63;
+    const int qwave = __builtin_amdgcn_readfirstlane(tid >> 6);                   // scalar item arithmetic
+    uint4 wa0 = make_uint4(0, 0, 0, 0), wb0 = wa0, wa1 = wa0, wb1 = wa0, wa2 = wa0, wb2 = wa0;
+    Q8Pass q_cur = {}, q_nxt = {};
+    bool q_chained = false;                      // the three fetches in flight are the first positions of the next pass
+    bool q_nxt_valid = false;                    // there is a next pass (it may hold no item for this wavefront)
+    int q_pos = 0, q_P = 3;                      // next position to fetch, positions of the current pass
+    int slices_end = 0;                          // end of this workgroup's slices in `segs`
+    if constexpr (kQ8 && TILED && !SINGLE) slices_end = seg_index[(wg + 1) * nphases];
+    auto q_make = [&](const uint32_t* bits, int rows, int words, int units, int row_end, int rb, int c0) -> Q8Pass {
+        Q8Pass p;
+        const int groups = (words + 15) >> 4;
+        p.bits = bits;
+        p.bytes = (uint32_t)((size_t)((rows + 31) >> 5) * groups * 2048);
+        const int cu_n = min(min(units, chunk_cap), units - c0);
+        p.ngroups = (cu_n + 3) >> 2;
+        p.skip = groups - p.ngroups;
+        const int nitems = p.ngroups * ((min(row_end - rb, kRowBlock) + 31) >> 5);
+        const int per = mfma_items_per_wave(nitems, kWaves);
+        p.it_begin = qwave * per;
+        p.count = max(min(p.it_begin + per, nitems) - p.it_begin, 0);
+        p.item_base = (rb >> 5) * groups + (c0 >> 2);
+        return p;
+    };
+    // One fetch = position q_pos of [items of the current pass][idle positions up to q_P][first items of the next pass]:
+    // always the same two load instructions, so that the compiler can count the fetches in flight.  Everything but
+    // the lane's byte offset is wave-uniform (selected field by field and pinned to scalar registers).
+    auto q_fetch_tiled = [&](uint4& wa, uint4& wb) {
+        const bool in_cur = q_pos < q_P;
+        const int j = in_cur ? q_pos : q_pos - q_P;
+        const bool live = j < (in_cur ? q_cur.count : q_nxt.count);
+        const int idx = (in_cur ? q_cur.it_begin : q_nxt.it_begin) + j;      // item of the pass: (row pair, unit group)
+        const int ngroups = in_cur ? q_cur.ngroups : q_nxt.ngroups;
+        const int skip = in_cur ? q_cur.skip : q_nxt.skip;                   // unit groups of the row outside the pass
+        int item = (in_cur ? q_cur.item_base : q_nxt.item_base) + idx;
+        if (skip != 0) item += (idx / ngroups) * skip;
+        const uint64_t bits = (uint64_t)(in_cur ? q_cur.bits : q_nxt.bits);
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)bits);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(bits >> 32));
+        const uint32_t bytes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(in_cur ? q_cur.bytes : q_nxt.bytes));
+        const __amdgpu_buffer_rsrc_t rs = raw_buffer((const void*)(((uint64_t)hi << 32) | lo), bytes);
+        const uint32_t soff = live ? (uint32_t)__builtin_amdgcn_readfirstlane(item) * 2048u : 0u;
+        const uint32_t voff = live ? (uint32_t)qlane * 16u : kPastEnd;
+        const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, soff, 2 /* nt */);
+        const u32x4_t b = __builtin_amdgcn_raw_buffer_load_b128(rs, voff + 1024u, soff, 2 /* nt */);
+        wa = make_uint4(a.x, a.y, a.z, a.w);
+        wb = make_uint4(b.x, b.y, b.z, b.w);
+        ++q_pos;
+    };
+
 #pragma unroll 1
     for (int ph = 0; ph < nphases; ++ph) {
         // SINGLE: one stage given by value, no tables and no counters; workgroup w takes rows
@@ -189,12 +245,9 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
             // path: its staging needs the registers, and holding fetched words across it (measured with one, two and
             // three items per wavefront) costs more in spills than the head start gains.
             uint4 wnext = make_uint4(0, 0, 0, 0);
-            // kQ8: fetch cursor of this wavefront over its items = (pair of 16-row groups, 4-unit group) of the
-            // current (row block, input chunk), unit group fastest, and the three item fetches it keeps in flight
-            const int qlane = tid & 63;
-            const int qwave = __builtin_amdgcn_readfirstlane(tid >> 6);           // scalar item arithmetic
+            // kQ8, row-major words: fetch cursor of this wavefront over its items = (pair of 16-row groups, 4-unit group)
+            // of the current (row block, input chunk), unit group fastest
             int q_ngroups = 1, q_it_begin = 0, q_it_end = 0, q_it_f = 0, q_rp_f = 0, q_ub_f = 0, q_rb = 0, q_c0 = 0, q_cu_n = 0, q_nr = 0;
-            uint4 wa0 = make_uint4(0, 0, 0, 0), wb0 = wa0, wa1 = wa0, wb1 = wa0, wa2 = wa0, wb2 = wa0;
             auto q_setup = [&](int rb, int c0) {
                 q_nr = min(seg.row_end - rb, kRowBlock);
                 q_cu_n = min(chunk_units, st.units - c0);
@@ -211,31 +264,57 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
             };
             auto q_fetch = [&](uint4& wa, uint4& wb) {
                 const bool live = q_it_f < q_it_end;
-                if constexpr (TILED) {
-                    // tile order: an item is 2 KiB contiguous (row group a, then b), lane l owns bytes 16 l of each half:
-                    // the address is a scalar item offset plus a lane constant, no lane arithmetic per fetch
-                    const uint32_t item = (uint32_t)((q_rb >> 5) + q_rp_f) * (uint32_t)bv.groups + (uint32_t)((q_c0 >> 2) + q_ub_f);
-                    const uint32_t soff = live ? item * 2048u : 0u;
-                    const uint32_t voff = live ? (uint32_t)qlane * 16u : kPastEnd;
-                    const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(bv.rsrc, voff, soff, 2 /* nt */);
-                    const u32x4_t b = __builtin_amdgcn_raw_buffer_load_b128(bv.rsrc, voff + 1024u, soff, 2 /* nt */);
-                    wa = make_uint4(a.x, a.y, a.z, a.w);
-                    wb = make_uint4(b.x, b.y, b.z, b.w);
-                } else {
-                    const int u = 4 * q_ub_f + (qlane >> 4);
-                    const int row = q_rb + 32 * q_rp_f + (qlane & 15);
-                    const bool ok = live && u < q_cu_n;
-                    wa = load_unit(bv, min(row, st.rows - 1), q_c0 + u, ok);
-                    wb = load_unit(bv, min(row + 16, st.rows - 1), q_c0 + u, ok);
-                }
+                const int u = 4 * q_ub_f + (qlane >> 4);
+                const int row = q_rb + 32 * q_rp_f + (qlane & 15);
+                const bool ok = live && u < q_cu_n;
+                wa = load_unit(bv, min(row, st.rows - 1), q_c0 + u, ok);
+                wb = load_unit(bv, min(row + 16, st.rows - 1), q_c0 + u, ok);
                 ++q_it_f;
                 if (++q_ub_f == q_ngroups) { q_ub_f = 0; ++q_rp_f; }
             };
+            // kQ8, tile order: the pass after (rb, c0) of this slice -- its next input chunk, its next row block, or the
+            // first pass of this workgroup's next slice, whose description is fetched here, well ahead of its use
+            RunSegment seg_n = seg;
+            const uint32_t* bits_n = nullptr;
+            int rows_n = 0, words_n = 0, units_n = 0;
+            if constexpr (kQ8 && TILED && !SINGLE) {
+                if (sg + 1 < slices_end) {
+                    seg_n = segs[sg + 1];
+                    const RunStage& sn = stages[seg_n.stage];
+                    bits_n = sn.bits; rows_n = sn.rows; words_n = sn.words; units_n = sn.units;
+                }
+            }
+            auto q_has_next = [&](int rb, int c0) -> bool {
+                return c0 + chunk_units < st.units || rb + kRowBlock < seg.row_end || bits_n != nullptr;
+            };
+            auto q_next_pass = [&](int rb, int c0) -> Q8Pass {
+                if (c0 + chunk_units < st.units) return q_make(st.bits, st.rows, st.words, st.units, seg.row_end, rb, c0 + chunk_units);
+                if (rb + kRowBlock < seg.row_end) return q_make(st.bits, st.rows, st.words, st.units, seg.row_end, rb + kRowBlock, 0);
+                if (bits_n) return q_make(bits_n, rows_n, words_n, units_n, seg_n.row_end, seg_n.row_begin, 0);
+                Q8Pass none = q_cur;             // no next pass: nothing of it is ever live
+                none.count = 0;
+                return none;
+            };
+            // Entering pass (rb, c0): its first three positions are already in flight (asked for by the previous pass)
+            // or are asked for now.
+            auto q_enter = [&](int rb, int c0) {
+                q_cur = q_make(st.bits, st.rows, st.words, st.units, seg.row_end, rb, c0);
+                q_P = (max(q_cur.count, 3) + 2) / 3 * 3;
+                q_nxt = q_next_pass(rb, c0);
+                q_pos = q_chained ? 3 : 0;
+                q_nxt_valid = q_has_next(rb, c0);
+                if (!q_chained) { q_fetch_tiled(wa0, wb0); q_fetch_tiled(wa1, wb1); q_fetch_tiled(wa2, wb2); }
+            };
             if constexpr (kQ8) {
                 // The packed words depend on nothing: the first three items of the slice are asked for before the
-                // dependency wait and the staging of the input, and arrive while those run.
-                q_setup(seg.row_begin, 0);
-                q_fetch(wa0, wb0); q_fetch(wa1, wb1); q_fetch(wa2, wb2);
+                // dependency wait and the staging of the input (in tile order: unless the previous pass already did),
+                // and arrive while those run.
+                if constexpr (TILED) {
+                    if (!aborted) q_enter(seg.row_begin, 0);
+                } else {
+                    q_setup(seg.row_begin, 0);
+                    q_fetch(wa0, wb0); q_fetch(wa1, wb1); q_fetch(wa2, wb2);
+                }
             } else {
                 // wavefront w starts with item w of the first row block: 16 rows x 4 units, lane (row l & 15,
                 // unit l >> 4)
@@ -319,10 +398,16 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                             // pair changes (LDS float atomics cost about 2.5 cycles per lane).
                             const int r16 = qlane & 15, g = qlane >> 4;
                             if (rb != seg.row_begin || c0 != 0) {        // the first pass was set up ahead of the wait
-                                q_setup(rb, c0);
-                                q_fetch(wa0, wb0); q_fetch(wa1, wb1); q_fetch(wa2, wb2);
+                                if constexpr (TILED) {
+                                    q_enter(rb, c0);
+                                } else {
+                                    q_setup(rb, c0);
+                                    q_fetch(wa0, wb0); q_fetch(wa1, wb1); q_fetch(wa2, wb2);
+                                }
                             }
-                            const int ngroups = q_ngroups, it_begin = q_it_begin, it_end = q_it_end;
+                            const int ngroups = TILED ? q_cur.ngroups : q_ngroups;
+                            const int it_begin = TILED ? q_cur.it_begin : q_it_begin;
+                            const int it_end = TILED ? q_cur.it_begin + q_cur.count : q_it_end;
                             // operand column of this lane (batch row, piece) and its first chunk; columns beyond the
                             // last piece are never read back, so their lanes skip the LDS reads (40 % less LDS time)
                             const bool qlive = r16 < BATCH * kQ8Pieces;
@@ -347,10 +432,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                                     if (qlast && row + 16 < nr) atomicAdd(&rdst[(32 * rp_run + 16 + v) * BATCH], sb);
                                 }
                             };
-                            // three register pairs in rotation, each refilled right after its use: nothing in flight
-                            // is ever copied, and the main loop has no early exit
-                            static_assert(kQ8Depth == 3, "the rotation below is written out for three register pairs");
-                            auto step = [&](uint4& wa, uint4& wb) {
+                            auto work = [&](uint4& wa, uint4& wb) {
                                 if (rp != rp_run) {
                                     flush();
                                     acc_a = acc_b = (float4_t){0.f, 0.f, 0.f, 0.f};
@@ -366,15 +448,40 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const RunStage* __
                                 }
                                 unit_mfma_q8_pair(wa, wb, opnd, qscale, acc_a, acc_b);
                                 if (++ub == ngroups) { ub = 0; ++rp; }
-                                q_fetch(wa, wb);
                             };
-                            int it = it_begin;
+                            // three register pairs in rotation, each refilled right after its use: nothing in flight
+                            // is ever copied
+                            static_assert(kQ8Depth == 3, "the rotation below is written out for three register pairs");
+                            if constexpr (TILED) {
+                                const int count = q_cur.count;
+                                // A full wait ahead of the loop (what is in flight was asked for a staging ago and has
+                                // arrived): without it the compiler carries the possibility of an outstanding generic-
+                                // address access (staging fallback, epilogue) into the loop and waits for ALL fetches at
+                                // every step instead of for the oldest one.
+                                __builtin_amdgcn_s_waitcnt(0);
 #pragma unroll 1
-                            for (; it + kQ8Depth <= it_end; it += kQ8Depth) {
-                                step(wa0, wb0); step(wa1, wb1); step(wa2, wb2);
+                                for (int i = 0; i < q_P; i += kQ8Depth) {
+                                    if (i < count) work(wa0, wb0);
+                                    q_fetch_tiled(wa0, wb0);
+                                    if (i + 1 < count) work(wa1, wb1);
+                                    q_fetch_tiled(wa1, wb1);
+                                    if (i + 2 < count) work(wa2, wb2);
+                                    q_fetch_tiled(wa2, wb2);
+                                }
+                                q_chained = q_nxt_valid;                 // what is in flight now belongs to the next pass
+                            } else {
+                                auto step = [&](uint4& wa, uint4& wb) {
+                                    work(wa, wb);
+                                    q_fetch(wa, wb);
+                                };
+                                int it = it_begin;
+#pragma unroll 1
+                                for (; it + kQ8Depth <= it_end; it += kQ8Depth) {
+                                    step(wa0, wb0); step(wa1, wb1); step(wa2, wb2);
+                                }
+                                if (it < it_end) step(wa0, wb0);
+                                if (it + 1 < it_end) step(wa1, wb1);
                             }
-                            if (it < it_end) step(wa0, wb0);
-                            if (it + 1 < it_end) step(wa1, wb1);
                             if (it_begin < it_end) flush();              // + the staged total of classes 0..2 at the end
                         } else {
                             // Items = (16-row group, 4-unit group), unit group fastest; every wavefront takes a
