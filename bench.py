@@ -1,15 +1,17 @@
 #!/usr/bin/env python3
 """Benchmark of the binary low-rank linear layer on one MI355X.
 
-Headline workload (N=1): the decode GEMV over one Llama-2-7B-shaped decoder layer at 1.0 bpw --
-q/k/v/o 4096x4096 (r=2048), gate/up 11008x4096 and down 4096x11008 (r = round(mn/(m+n)) = 2985) --
-batch 1, fp16 activations.  One "step" is one pass over the 7 linears of the layer.  Successive steps
-walk over distinct copies of the layer's weights (more than the 256 MB Infinity Cache in total), so
-the packed words come from HBM, not from cache.  `value` is algorithmic bytes / time.
+Headline workload (N=1): the batch-1 decode GEMV over Llama-2-7B-shaped decoder layers at 1.0 bpw -- per layer q/k/v/o
+4096x4096 (r=2048), gate/up 11008x4096 and down 4096x11008 (r = round(mn/(m+n)) = 2985) -- fp16 activations.  One
+"step" is one token step over the linear layers of a whole 32-layer decoder stack (224 linears, 810 MB of packed
+words, every word read once per step, so the words come from HBM and not from the 256 MB Infinity Cache), enqueued as
+ONE run-list launch, the way a decoder would run it.  `value` is algorithmic bytes / time; `us_per_layer` = step time
+/ 32.  The same layer as one launch per layer (rotating over the 32 weight copies) is in `extra`, with a roofline
+object of its own.
 
-Prints ONE JSON line.  Extra keys report the same layer at batch 4 and 16, the prefill GEMM at 128, 512
-and 4096 tokens, the two-term Qwen3-8B-like layer (cfg3) and the Llama-3-70B weight stream (cfg4); `roofline` is for the decode kernel, `cpu_baseline` is the reference's dense CPU path (two
-F.linear on unpacked +-1 factors) timed on this host.
+Prints ONE JSON line.  Extra keys report batch 4 and 16, the prefill GEMM at 128, 512 and 4096 tokens (`roofline_prefill`
+is the 128-token headline), the two-term Qwen3-8B-like layer (cfg3) and the Llama-3-70B weight stream (cfg4);
+`cpu_baseline` is the reference's dense CPU path (two F.linear on unpacked +-1 factors) timed on this host.
 """
 from __future__ import annotations
 
@@ -26,8 +28,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the headline kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
-# copy kernel of known size (profiles/gemv_stream_llama2_7b_layer_b1.md); valid for the default workload only.
-MEASURED_TRAFFIC_BYTES = 28070400
+# copy kernel of known size (profiles/gemv_stream_llama2_7b_stack_b1.md); valid for the default workload only.
+MEASURED_TRAFFIC_BYTES = 840352768
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 LLAMA2_7B_LAYER = (("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096),
@@ -103,9 +105,10 @@ def build_layers(torch, dev, shapes, copies, seed):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=520)
-    ap.add_argument("--warmup", type=int, default=52)
-    ap.add_argument("--copies", type=int, default=26, help="distinct weight copies of the layer (26 x 25.3 MB > 256 MB)")
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--copies", type=int, default=32, help="decoder layers of the stack = distinct weight copies of the layer "
+                                                           "(32 x 25.3 MB = 810 MB > 256 MB Infinity Cache)")
     ap.add_argument("--no-extra", action="store_true", help="skip batch 4/16, prefill and CPU legs")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -197,19 +200,49 @@ def main():
     def layer_bytes(batch):
         return sum(gemv_bytes(lin.m, lin.n, lin.r, batch) for lin in layers[0])
 
-    # ---- headline: batch 1 -------------------------------------------------------------------
+    # ---- headline: batch 1, one token step over the whole stack in one launch -------------------------------
+    from nanoquant_amd import DecodeRunList
+
+    def make_stack(io, batch, dtype=torch.float16):
+        xs, _, ys = io
+        rl = DecodeRunList(batch, dtype, dev)
+        for layer in layers:
+            for lin, x, y in zip(layer, xs, ys):
+                lin.add_to(rl, x, y=y)
+        rl.build()
+        return rl
+
+    def timed_launches(fn, steps, warmup):
+        """Exactly `steps` launches of fn, back to back on the current stream, between two events on that stream."""
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps  # ms per launch
+
     io1 = make_io(1)
-    lists1 = make_runlists(io1, 1)
-    ms = timed([rl.run for rl in lists1], args.steps, args.warmup)
-    for rl in lists1:
-        if rl.status() != 0:
-            raise RuntimeError("run list reported an expired dependency wait")
+    stack1 = make_stack(io1, 1)
+    # set-up, not part of the W warm-up steps: 300 launches (45 ms) take the device to its sustained state (the first
+    # 25 ms of back-to-back launches after the weights were generated run up to 15 % slower), and the step is captured
+    # once as a HIP graph so that the timed loop costs the host a replay per step
+    for _ in range(300):
+        stack1.run()
+    torch.cuda.synchronize()
+    step_graph = capture_rotation([stack1.run])
+    ms = timed_launches(step_graph.replay, args.steps, args.warmup)
+    if stack1.status() != 0:
+        raise RuntimeError("run list reported an expired dependency wait")
+    nlayers = len(layers)
     bytes1 = layer_bytes(1)
-    gbs = bytes1 / (ms * 1e-3) / 1e9
-    launches_per_step = 1
-    launch_us = ms * 1e3 / launches_per_step
+    bytes_step = bytes1 * nlayers
+    gbs = bytes_step / (ms * 1e-3) / 1e9
     result = {
-        "metric": "batch-1 binary GEMV sustained GB/s over one Llama-2-7B decoder layer (1.0 bpw)",
+        "metric": "batch-1 binary GEMV sustained GB/s over Llama-2-7B decoder layers (1.0 bpw)",
         "value": round(gbs, 2),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -222,28 +255,29 @@ def main():
         "dtype": "f16 in/out; one-bit fp4 x fp8-piece MFMA products (exact), f32 accumulate",
         "data": "synthetic",
         "config": {
-            "workload": "cfg1: decode GEMV over the 7 linears of one Llama-2-7B decoder layer, batch 1, 1.0 bpw "
-                        "(q/k/v/o 4096x4096 r2048; gate/up 11008x4096, down 4096x11008 r2985 padded to 3008 with "
-                        "zero mid scale); %d rotating weight copies (%.0f MB) so words come from HBM; the packed words are "
-                        "handed over in the run list's tile order, a fixed permutation of the reference's row-major words "
-                        "done once at load"
-                        % (args.copies, args.copies * sum(lin.r * (lin.m + lin.n) / 8 for lin in layers[0]) / 1e6),
+            "workload": "cfg1: batch-1 decode GEMV, one token step over the linear layers of a %d-layer Llama-2-7B-shaped "
+                        "decoder stack (%d linears; per layer q/k/v/o 4096x4096 r2048, gate/up 11008x4096 and down 4096x11008 "
+                        "r2985 padded to 3008 with zero mid scale; 1.0 bpw, %.0f MB of packed words, every word read once per "
+                        "step, so from HBM) in ONE run-list launch; the packed words are handed over in the run list's tile "
+                        "order, a fixed permutation of the reference's row-major words done once at load"
+                        % (nlayers, 7 * nlayers, nlayers * sum(lin.r * (lin.m + lin.n) / 8 for lin in layers[0]) / 1e6),
             "batch": 1,
-            "algorithmic_bytes_per_step": int(bytes1),
-            "launches_per_step": launches_per_step,
+            "layers_per_step": nlayers,
+            "algorithmic_bytes_per_step": int(bytes_step),
+            "launches_per_step": 1,
         },
-        "us_per_layer": round(ms * 1e3, 3),
+        "us_per_layer": round(ms * 1e3 / nlayers, 3),
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_stream_kernel<fp16, batch 1, fp4 x fp8 MFMA, 1024 lanes> (one launch per layer: 14 stages in "
-                      "2 phases, 256 resident workgroups)",
-            "achieved": round(bytes1 / launches_per_step / (launch_us * 1e-6) / 1e9, 2),
+            "kernel": "gemv_stream_kernel<fp16, batch 1, fp4 x fp8 MFMA, 1024 lanes, tile order> (one launch per token step: "
+                      "%d stages in 2 phases, 256 resident workgroups)" % (14 * nlayers),
+            "achieved": round(gbs, 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": round(bytes1 / launches_per_step / (launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES if args.copies == 26 else None,
-            "bytes_per_launch": int(bytes1 / launches_per_step),
-            "avg_launch_us": round(launch_us, 3),
+            "frac": round(gbs / HBM_PEAK_GBS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES if (args.copies == 32 and MEASURED_TRAFFIC_BYTES) else None,
+            "bytes_per_launch": int(bytes_step),
+            "avg_launch_us": round(ms * 1e3, 3),
         },
     }
 
@@ -273,32 +307,37 @@ def main():
         for b in (4, 16):
             io = make_io(b)
             lists = make_runlists(io, b)
-            msb = timed([rl.run for rl in lists], max(args.steps // 4, args.copies), args.copies)
-            extra[f"batch{b}"] = {"us_per_layer": round(msb * 1e3, 3),
-                                  "GBps": round(layer_bytes(b) / (msb * 1e-3) / 1e9, 2)}
-            del lists
+            msb = timed([rl.run for rl in lists], 4 * len(layers), len(layers))
+            st_b = make_stack(io, b)
+            ms_sb = timed_launches(st_b.run, 10, 2) / len(layers)
+            extra[f"batch{b}"] = {"us_per_layer_stack_one_launch": round(ms_sb * 1e3, 3),
+                                  "GBps_stack_one_launch": round(layer_bytes(b) / (ms_sb * 1e-3) / 1e9, 2),
+                                  "us_per_layer_one_launch_per_layer": round(msb * 1e3, 3),
+                                  "GBps_one_launch_per_layer": round(layer_bytes(b) / (msb * 1e-3) / 1e9, 2)}
+            del lists, st_b
         # bf16 activations and scales (what the reference's module defaults to), same layer and launch shape
         io_bf = make_io(1, torch.bfloat16)
-        lists = make_runlists(io_bf, 1)
-        ms_bf = timed([rl.run for rl in lists], max(args.steps // 4, args.copies), args.copies)
-        extra["batch1_bf16"] = {"us_per_layer": round(ms_bf * 1e3, 3), "GBps": round(bytes1 / (ms_bf * 1e-3) / 1e9, 2)}
-        del lists, io_bf
-        # all weight copies in ONE run list (= one launch over copies x 7 linears): the per-launch latencies
-        # (descriptor fetch, two dependency phases, drain) are paid once for the whole stack
-        from nanoquant_amd import DecodeRunList
-        stack = DecodeRunList(1, torch.float16, dev)
-        for layer in layers:
-            for lin, x, y in zip(layer, io1[0], io1[2]):
-                lin.add_to(stack, x, y=y)
-        stack.build()
-        ms_stack = timed([stack.run], 10, 2) / len(layers)
-        if stack.status() != 0:
-            raise RuntimeError("run list reported an expired dependency wait")
-        extra["batch1_stack_one_launch"] = {"us_per_layer": round(ms_stack * 1e3, 3),
-                                            "GBps": round(bytes1 / (ms_stack * 1e-3) / 1e9, 2),
-                                            "note": "%d layers (%d linears) in one run-list launch" % (len(layers), 7 * len(layers))}
-        del stack
-        ms_pl = timed(per_linear_steps(io1, 1), max(args.steps // 4, args.copies), args.copies)
+        st_bf = make_stack(io_bf, 1, torch.bfloat16)
+        ms_bf = timed_launches(st_bf.run, 10, 2) / len(layers)
+        extra["batch1_bf16"] = {"us_per_layer": round(ms_bf * 1e3, 3), "GBps": round(bytes1 / (ms_bf * 1e-3) / 1e9, 2),
+                                "note": "the headline stack with bf16 activations and scales"}
+        del st_bf, io_bf
+        # the same layer as ONE launch per layer (14 stages in 2 phases), rotating over the weight copies: what a
+        # caller gets who launches layer by layer; bound by the serial latencies inside a launch, not by HBM
+        lists1 = make_runlists(io1, 1)
+        ms_l = timed([rl.run for rl in lists1], 8 * len(layers), len(layers))
+        for rl in lists1:
+            if rl.status() != 0:
+                raise RuntimeError("run list reported an expired dependency wait")
+        extra["batch1_one_launch_per_layer"] = {
+            "us_per_layer": round(ms_l * 1e3, 3), "GBps": round(bytes1 / (ms_l * 1e-3) / 1e9, 2),
+            "roofline": {"bound": "hbm", "kernel": "gemv_stream_kernel, one launch per layer (14 stages in 2 phases)",
+                         "achieved": round(bytes1 / (ms_l * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(bytes1 / (ms_l * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "bytes_per_launch": int(bytes1),
+                         "avg_launch_us": round(ms_l * 1e3, 3)},
+            "note": "graph replays of one launch per layer over %d rotating weight copies" % len(layers)}
+        del lists1
+        ms_pl = timed(per_linear_steps(io1, 1), 4 * len(layers), len(layers))
         extra["batch1_per_linear_launches"] = {"us_per_layer": round(ms_pl * 1e3, 3),
                                                "GBps": round(bytes1 / (ms_pl * 1e-3) / 1e9, 2),
                                                "note": "same layer through nq_gemv_forward: 14 launches per layer"}
@@ -358,6 +397,14 @@ def main():
                 "us_per_layer": round(us, 2), "TFLOPs": round(tf, 2), "frac_of_f16_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
                 "note": "7 linears of the layer in two launches (nq_gemm_nanoquant_group); q,k,v,o share one weight copy here"}
             del g
+            if tokens == 128:
+                # the second headline metric (128-token GEMM TFLOP/s) as a roofline object of its own
+                result["roofline_prefill"] = {
+                    "bound": "mfma", "tokens": 128,
+                    "kernel": "gemm_kwave_group_kernel<fp16> x 2 launches (first GEMMs of the 7 linears, then second GEMMs)",
+                    "achieved": round(tf, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "flops_per_layer": int(group_flops),
+                    "us_per_layer": round(us, 2), "traffic": None}
             if tokens == 16:
                 # the same 16 rows as extra.batch16, on the prefill kernels and with cold weights as there: every
                 # linear of every rotation step reads its own copy of the packed tiles (args.copies x 7 clones)

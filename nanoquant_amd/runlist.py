@@ -127,6 +127,7 @@ class DecodeRunList:
                                             ctypes.c_void_p(ws.data_ptr()), nbytes, ctypes.byref(plan), stream))
         self._plan = plan
         self._workspace = ws
+        self._needs = (any(e["x"] is None for e in self._entries), any(e["y"] is None for e in self._entries))
 
     def _dtype_id(self) -> int:
         return _lib.NQ_F16 if self.dtype == torch.float16 else _lib.NQ_BF16
@@ -137,8 +138,7 @@ class DecodeRunList:
         the tensors of the entries added with `x=None` / `bind_y=True`."""
         if self._workspace is None:
             self.build()
-        need_x = any(e["x"] is None for e in self._entries)
-        need_y = any(e["y"] is None for e in self._entries)
+        need_x, need_y = self._needs        # fixed at build(): a launch costs microseconds, a scan of a long list more
         if need_x != (x is not None) or need_y != (y is not None):
             raise RuntimeError("run(x=, y=) must be given exactly when the list has late-bound entries")
         for name, t, key in (("x", x, "n"), ("y", y, "m")):
