@@ -564,6 +564,34 @@ def main():
             if time.perf_counter() > t_bf_end + 20:
                 break
         bf_times.sort()
+
+        # the same dense factors, packed and run through the headline kernel (one layer, batch 1, fp16, tile order);
+        # error figures of the GPU result against the layer definition evaluated in fp64 on the same fp16 operands
+        import numpy as np
+        from nanoquant_amd import packing
+        rl_chk = DecodeRunList(1, torch.float16, dev)
+        refs = []
+        for (x, vt, u, s_in, s_mid, s_out) in cpu_terms:
+            h16 = lambda t: t.to(torch.float16)
+            f64 = lambda t: h16(t).double().numpy()
+            vt_p, u_p, mid_p = oracle.pad_rank(vt.numpy().astype(np.int8), u.numpy().astype(np.int8),
+                                               h16(s_mid).numpy(), 32)
+            words = lambda w: packing.tile_words(packing.binary_packer(torch.from_numpy(w), "half2").to(dev))
+            rl_chk.add(h16(x).to(dev), h16(s_in).to(dev), words(vt_p), torch.from_numpy(mid_p).to(dev), words(u_p),
+                       h16(s_out).to(dev), tiled=True, out_f32=True)
+            refs.append(oracle.layer_forward(f64(x), vt.numpy(), u.numpy(), f64(s_in), f64(s_mid), f64(s_out),
+                                             dtype=np.float64))
+        got = [y.cpu().numpy() for y in rl_chk.run()]
+        torch.cuda.synchronize()
+        if rl_chk.status() != 0:
+            raise RuntimeError("run list reported an expired dependency wait")
+        result["parity"] = {
+            "max_rel_err": float("%.3e" % max(oracle.max_rel_err(y, r) for y, r in zip(got, refs))),
+            "elementwise_err": float("%.3e" % max(oracle.elementwise_err(y, r) for y, r in zip(got, refs))),
+            "definition": "worst of the 7 linears; max|dy|/max|y_ref| and max(|dy|/(|y_ref| + 0.1 rms(y_ref))), "
+                          "fp32 outputs of the headline kernel against the fp64 layer definition on the CPU baseline's factors",
+        }
+        del rl_chk
         result["cpu_baseline"] = {
             "value": round(bytes1 / med / 1e9, 3),
             "unit": "GB/s",

@@ -23,8 +23,11 @@ checkout):
   torch_dense_forward     the same _compute_forward with torch.nn.functional.linear on dense
                           +-1 factors: the reference's CPU path, timed as the CPU baseline
   fp8_e4m3_round / fp8_pieces / staged_input   no counterpart in the reference: the number format (OCP e4m3,
-                          round to nearest even) and the three-piece decomposition in which the gfx950 run-list
-                          kernel stages its input; lets a test state exactly what that kernel must compute
+                          round to nearest even) and the three-piece decomposition, with one power-of-two scale
+                          per block of 128 columns, in which the gfx950 run-list kernel stages its input; lets a
+                          test state exactly what that kernel must compute
+  max_rel_err / elementwise_err   the two error figures of the tests: max|dy| / max|y_ref| (the tolerance
+                          metric) and max(|dy| / (|y_ref| + 0.1 rms(y_ref))) (every element judged on its own)
 
 Pinning of the fp8 helpers: against torch.float8_e4m3fn conversion on every finite fp8 value, on midpoints and on
 random inputs, and against the closed-form error bound of the decomposition (tests/test_oracle_layer.py).
@@ -222,6 +225,18 @@ def max_rel_err(y, y_ref) -> float:
     if denom == 0.0:
         return float(np.max(np.abs(y)))
     return float(np.max(np.abs(y - y_ref)) / denom)
+
+
+def elementwise_err(y, y_ref, floor_frac: float = 0.1) -> float:
+    """max over elements of |y - y_ref| / (|y_ref| + floor), floor = floor_frac * rms(y_ref) per output tensor.
+    The absolute floor keeps outputs that happen to lie near zero from deciding the figure; everything above the
+    floor is judged relative to itself, which `max_rel_err` (one denominator for the whole tensor) does not do."""
+    y = np.asarray(y, dtype=np.float64)
+    y_ref = np.asarray(y_ref, dtype=np.float64)
+    floor = floor_frac * float(np.sqrt(np.mean(y_ref * y_ref)))
+    if floor == 0.0:
+        return float(np.max(np.abs(y)))
+    return float(np.max(np.abs(y - y_ref) / (np.abs(y_ref) + floor)))
 
 
 # --------------------------------------------------------------------------------------

@@ -71,8 +71,14 @@ def test_cfg1_layer_run_list_as_benchmarked(dev, batch):
         torch.cuda.synchronize()
         assert rl.status() == 0
         for (name, rows, ref), y in zip(cases, ys):
-            e = _err(y.float().cpu().numpy()[:, rows], ref)
+            got = y.float().cpu().numpy()[:, rows]
+            e, ee = _err(got, ref), oracle.elementwise_err(got, ref)
+            if rep == 0:
+                print(f"  {name}: max_rel_err {e:.2e}, element-wise (floor 0.1 rms) {ee:.2e}", flush=True)
             assert e < 1e-3, (name, batch, rep, e)
+            # fp16 outputs cost 2^-11 of the element by themselves; the 16-bit arithmetic (more than 4 rows) also rounds
+            # x * s_in and the intermediate vector to fp16, as the reference's kernels do
+            assert ee < (5e-3 if batch <= 4 else 5e-2), (name, batch, rep, ee)
 
 
 # ---- cfg2 --------------------------------------------------------------------------------------------

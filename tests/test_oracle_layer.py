@@ -168,3 +168,14 @@ def test_three_fp8_pieces_reproduce_the_input():
     assert np.all(np.abs(sv - v) <= np.maximum(2.0 ** -12 * np.abs(v), 2.0 ** -17 * np.abs(v).max(axis=1, keepdims=True)))
     assert np.array_equal(oracle.staged_input(v * 8.0), sv * 8.0)
     assert np.array_equal(oracle.staged_input(np.zeros((1, 64))), np.zeros((1, 64)))
+
+
+def test_error_figures_known_answers():
+    ref = np.array([3.0, -4.0, 0.0, 5.0])                              # rms = sqrt(50 / 4)
+    y = ref + np.array([0.0, 0.5, 0.25, -1.0])
+    floor = 0.1 * np.sqrt(12.5)
+    assert oracle.max_rel_err(y, ref) == pytest.approx(1.0 / 5.0)
+    assert oracle.elementwise_err(y, ref) == pytest.approx(max(0.5 / (4 + floor), 0.25 / floor, 1.0 / (5 + floor)))
+    assert oracle.elementwise_err(y, ref, floor_frac=1.0) == pytest.approx(1.0 / (5 + np.sqrt(12.5)))
+    assert oracle.elementwise_err(ref, ref) == 0.0
+    assert oracle.elementwise_err(np.array([0.5]), np.zeros(1)) == 0.5   # a zero reference: the absolute error
