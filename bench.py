@@ -303,6 +303,15 @@ def main():
         extra["hbm_copy_kernel"] = {"GBps_read_plus_write": round(2 * nbytes / (ms_copy * 1e-3) / 1e9, 1),
                                     "note": "plain 16-byte copy kernel, 256 MiB each way: a measured ceiling for streaming "
                                             "kernels on this box (vendor peak 8000 GB/s)"}
+        # launch floor of this box: the same copy kernel on 16 bytes (one workgroup, nothing to do) and on 1 MiB regions
+        # of the 256 MiB buffers (so that every launch reads HBM), 256 launches per graph replay
+        def floor_us(nb):
+            fns = [(lambda o=o: _lib.check(lib.nq_stream_copy(vp(cdst_.data_ptr() + o), vp(csrc_.data_ptr() + o), nb,
+                                                              vp(torch.cuda.current_stream().cuda_stream))))
+                   for o in range(0, nbytes, nbytes // 256)]
+            return round(timed(fns, 1024, 256) * 1e3, 2)
+        extra["launch_floor"] = {"us_per_launch_16_bytes": floor_us(16), "us_per_launch_1MiB_copy": floor_us(1 << 20),
+                                 "note": "back-to-back launches in graph replay; the 1 MiB copy reads 1 MiB and writes 1 MiB"}
         del csrc_, cdst_
         for b in (4, 16):
             io = make_io(b)

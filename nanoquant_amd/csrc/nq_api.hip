@@ -159,16 +159,15 @@ int nq_gemv_stage(const void* in, const void* s_col, const uint32_t* bits, const
 }
 
 // ---- run list ---------------------------------------------------------------------------------
-// workspace layout: [0,256): status word; completion counters; 2n RunStage records; the slice index
-// (one int per workgroup and phase, +1); the slices.  Every block is rounded to 256 bytes.
+// workspace layout: [0,256): status word; completion counters; the slice records (each with a copy of its stage).
+// Every block is rounded to 256 bytes.
 static size_t round256(size_t v) { return (v + 255) / 256 * 256; }
 static size_t runlist_counter_bytes(int n) { return round256(nq::stream_counter_bytes(2 * n)); }
-static size_t runlist_table_bytes(int n) { return round256((size_t)2 * n * sizeof(nq::RunStage)); }
-constexpr int kMaxResidentWorkgroups = 256 * 8 * 2;   // upper bound used for sizing only
+constexpr int kMaxResidentWorkgroups = 1024;   // upper bound used for sizing only (1024-lane workgroups: 1-2 per CU)
 
-static size_t runlist_index_bytes(int nwg, int nphases) { return round256(((size_t)nwg * nphases + 1) * sizeof(int)); }
-static size_t runlist_seg_bytes(int nwg, int nphases, int nstages) {
-    return round256(((size_t)nwg * nphases + nstages) * sizeof(nq::RunSegment));
+// slices: one first record per workgroup, then at most one more per workgroup and phase and one per stage
+static size_t runlist_slice_bytes(int nwg, int nphases, int nstages) {
+    return round256(((size_t)nwg * (nphases + 1) + nstages) * sizeof(nq::RunSlice));
 }
 
 size_t nq_runlist_workspace_bytes(const nq_linear* linears, int nlinears) {
@@ -178,9 +177,7 @@ size_t nq_runlist_workspace_bytes(const nq_linear* linears, int nlinears) {
     for (int i = 0; i < nlinears; ++i)
         if (linears[i].x_from >= 0 || linears[i].y_from >= 0) depth_bound += 2;
     if (depth_bound > 2 * nlinears) depth_bound = 2 * nlinears;
-    return 256 + runlist_counter_bytes(nlinears) + runlist_table_bytes(nlinears) +
-           runlist_index_bytes(kMaxResidentWorkgroups, depth_bound) +
-           runlist_seg_bytes(kMaxResidentWorkgroups, depth_bound, 2 * nlinears);
+    return 256 + runlist_counter_bytes(nlinears) + runlist_slice_bytes(kMaxResidentWorkgroups, depth_bound, 2 * nlinears);
 }
 
 static inline bool al16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
@@ -284,11 +281,9 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
     int nwg = nq::stream_capacity(dtype, batch, max_units);
     if (nwg <= 0) return NQ_ERR_HIP;
     if (nwg > kMaxResidentWorkgroups) nwg = kMaxResidentWorkgroups;
-    std::vector<int> seg_index((size_t)nwg * nphases + 1, 0);
-    std::vector<nq::RunSegment> segs;
     std::vector<std::vector<int>> by_phase((size_t)nphases);
     for (int s = 0; s < nstages; ++s) by_phase[table[s].phase].push_back(s);
-    // slices are emitted workgroup-major so that seg_index[wg*nphases + ph] is monotonic
+    // slices per phase and workgroup, in the order in which the workgroup works them off
     std::vector<std::vector<std::vector<nq::RunSegment>>> slice((size_t)nphases);
     for (int ph = 0; ph < nphases; ++ph) {
         slice[ph].resize((size_t)nwg);
@@ -439,27 +434,43 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
             if (fill(lo, true) > nwg) return NQ_ERR_SHAPE;               // cannot happen: hi always fits
         }
     }
-    for (int w = 0; w < nwg; ++w)
-        for (int ph = 0; ph < nphases; ++ph) {
-            seg_index[(size_t)w * nphases + ph] = (int)segs.size();
-            for (const auto& sg : slice[ph][w]) segs.push_back(sg);
-        }
-    seg_index[(size_t)nwg * nphases] = (int)segs.size();
+    // Slice records: record w is the first slice of workgroup w (phase by phase, in the order of `slice`), the others
+    // follow behind the nwg first records, contiguous per workgroup.  Each record carries a copy of its stage.
+    for (auto& st : table) {
+        st.dep_segs = st.dep >= 0 ? table[(size_t)st.dep].seg_count : 0;
+        st.dep2_segs = st.dep2 >= 0 ? table[(size_t)st.dep2].seg_count : 0;
+    }
+    std::vector<nq::RunSlice> records((size_t)nwg);
+    for (int w = 0; w < nwg; ++w) {
+        nq::RunSlice first = {};
+        first.seg = nq::RunSegment{-1, 0, 0, 0};
+        first.more_begin = first.more_end = (int)records.size();
+        bool have_first = false;
+        for (int ph = 0; ph < nphases; ++ph)
+            for (const auto& sg : slice[ph][w]) {
+                nq::RunSlice r = {};
+                r.seg = sg;
+                r.st = table[(size_t)sg.stage];
+                if (!have_first) {
+                    r.more_begin = first.more_begin;
+                    first = r;
+                    have_first = true;
+                } else {
+                    records.push_back(r);
+                }
+            }
+        first.more_end = (int)records.size();
+        records[(size_t)w] = first;
+    }
 
-    const size_t off_table = 256 + runlist_counter_bytes(nlinears);
-    const size_t off_index = off_table + runlist_table_bytes(nlinears);
-    const size_t off_segs = off_index + round256(seg_index.size() * sizeof(int));
-    if (off_segs + segs.size() * sizeof(nq::RunSegment) > workspace_bytes) return NQ_ERR_WORKSPACE;
+    const size_t off_slices = 256 + runlist_counter_bytes(nlinears);
+    if (off_slices + records.size() * sizeof(nq::RunSlice) > workspace_bytes) return NQ_ERR_WORKSPACE;
 
     hipStream_t hs = (hipStream_t)stream;
     char* base = (char*)workspace;
-    hipError_t e = hipMemsetAsync(base, 0, off_table, hs);
+    hipError_t e = hipMemsetAsync(base, 0, off_slices, hs);
     if (e != hipSuccess) return hip_status(e);
-    e = hipMemcpyAsync(base + off_table, table.data(), table.size() * sizeof(nq::RunStage), hipMemcpyHostToDevice, hs);
-    if (e != hipSuccess) return hip_status(e);
-    e = hipMemcpyAsync(base + off_index, seg_index.data(), seg_index.size() * sizeof(int), hipMemcpyHostToDevice, hs);
-    if (e != hipSuccess) return hip_status(e);
-    e = hipMemcpyAsync(base + off_segs, segs.data(), segs.size() * sizeof(nq::RunSegment), hipMemcpyHostToDevice, hs);
+    e = hipMemcpyAsync(base + off_slices, records.data(), records.size() * sizeof(nq::RunSlice), hipMemcpyHostToDevice, hs);
     if (e != hipSuccess) return hip_status(e);
     plan_out->nlinears = nlinears;
     plan_out->nstages = nstages;
@@ -468,7 +479,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
     plan_out->max_units = max_units;
     plan_out->batch = batch;
     plan_out->dtype = dtype;
-    plan_out->index_words = (int)seg_index.size();
+    plan_out->index_words = (int)records.size();
     plan_out->bound = 0;
     for (int i = 0; i < nlinears; ++i) plan_out->bound |= (linears[i].x ? 0 : 1) | (linears[i].y ? 0 : 2);
     if (linears[0].tiled) plan_out->bound |= 4;
@@ -485,17 +496,14 @@ int nq_runlist_run_bound(const void* workspace, const nq_runlist_plan* plan, con
     if (((uintptr_t)x) & 15u) return NQ_ERR_ALIGN;
     if (plan->dtype != NQ_F16 && plan->dtype != NQ_BF16) return NQ_ERR_DTYPE;
     if (plan->nlinears <= 0 || plan->nstages != 2 * plan->nlinears || plan->workgroups <= 0 || plan->max_units <= 0 ||
-        plan->nphases <= 0 || plan->index_words != plan->workgroups * plan->nphases + 1)
+        plan->nphases <= 0 || plan->index_words < plan->workgroups)
         return NQ_ERR_SHAPE;
     const int batch = plan->batch;
     if (batch != 1 && batch != 2 && batch != 4 && batch != 8 && batch != 16) return NQ_ERR_SHAPE;
     char* base = (char*)workspace;
-    const size_t off_table = 256 + runlist_counter_bytes(plan->nlinears);
-    const size_t off_index = off_table + runlist_table_bytes(plan->nlinears);
-    const size_t off_segs = off_index + round256((size_t)plan->index_words * sizeof(int));
-    return hip_status(nq::gemv_stream(plan->dtype, batch, (const nq::RunStage*)(base + off_table), plan->nstages,
-                                      plan->nphases, (const int*)(base + off_index),
-                                      (const nq::RunSegment*)(base + off_segs), (unsigned long long*)(base + 256),
+    const size_t off_slices = 256 + runlist_counter_bytes(plan->nlinears);
+    return hip_status(nq::gemv_stream(plan->dtype, batch, plan->nstages, (const nq::RunSlice*)(base + off_slices),
+                                      (unsigned long long*)(base + 256),
                                       (unsigned*)base, plan->workgroups, plan->max_units, (hipStream_t)stream, x, y,
                                       (plan->bound & 4) != 0));
 }

@@ -35,19 +35,29 @@ struct RunStage {
     int heavy_acquire;      // 16-bit input written by an earlier stage: full device-scope acquire after the wait
     int tiled;              // `bits` is in the tile order of tile_words() instead of row-major
     int in_ext, out_ext;    // `in` / `out` are given with the launch instead (bound input / output of the list)
+    int dep_segs, dep2_segs;  // seg_count of the stages `dep` / `dep2` (what a waiting slice compares the counter with)
     int pad_;
 };
 // One workgroup's share of one stage: rows [row_begin, row_end).
 struct RunSegment {
     int stage, row_begin, row_end, pad_;
 };
+// What the kernel reads per slice, in one record: the slice and a copy of its stage (one dependent memory access
+// between the kernel arguments and the first load of data instead of three).  Record w of the table is the first
+// slice of workgroup w (stage -1: the workgroup has none); its further slices are the records [more_begin,
+// more_end), in the order in which it works them off.
+struct RunSlice {
+    RunSegment seg;
+    int more_begin, more_end;   // meaningful in the first record of a workgroup only
+    RunStage st;
+};
 size_t stream_counter_bytes(int nstages);
 int stream_capacity(int dtype, int batch, int max_units);
 int stream_chunk_cap(int dtype, int batch, int max_units);
 int stream_row_granule(int dtype, int batch);
-hipError_t gemv_stream(int dtype, int batch, const RunStage* stages, int nstages, int nphases, const int* seg_index,
-                       const RunSegment* segs, unsigned long long* counters, unsigned* status, int nwg, int max_units,
-                       hipStream_t stream, const void* ext_in = nullptr, void* ext_out = nullptr, bool tiled = false);
+hipError_t gemv_stream(int dtype, int batch, int nstages, const RunSlice* slices, unsigned long long* counters,
+                       unsigned* status, int nwg, int max_units, hipStream_t stream, const void* ext_in = nullptr,
+                       void* ext_out = nullptr, bool tiled = false);
 bool stream_needs_uniform_order(int dtype, int batch);
 
 // One stage on its own through the run-list kernel (no tables, no counters); batch 16 only.
