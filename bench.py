@@ -203,9 +203,9 @@ def main():
     # ---- headline: batch 1, one token step over the whole stack in one launch -------------------------------
     from nanoquant_amd import DecodeRunList
 
-    def make_stack(io, batch, dtype=torch.float16):
+    def make_stack(io, batch, dtype=torch.float16, deterministic=False):
         xs, _, ys = io
-        rl = DecodeRunList(batch, dtype, dev)
+        rl = DecodeRunList(batch, dtype, dev, deterministic=deterministic)
         for layer in layers:
             for lin, x, y in zip(layer, xs, ys):
                 lin.add_to(rl, x, y=y)
@@ -331,6 +331,14 @@ def main():
         extra["batch1_bf16"] = {"us_per_layer": round(ms_bf * 1e3, 3), "GBps": round(bytes1 / (ms_bf * 1e-3) / 1e9, 2),
                                 "note": "the headline stack with bf16 activations and scales"}
         del st_bf, io_bf
+        # the headline stack with reproducible sums (every launch gives the same bits)
+        st_det = make_stack(io1, 1, deterministic=True)
+        ms_det = timed_launches(st_det.run, 10, 2) / len(layers)
+        extra["batch1_deterministic"] = {"us_per_layer": round(ms_det * 1e3, 3),
+                                         "GBps": round(bytes1 / (ms_det * 1e-3) / 1e9, 2),
+                                         "note": "DecodeRunList(deterministic=True): partial sums rounded to a grid on which "
+                                                 "additions are exact"}
+        del st_det
         # the same layer as ONE launch per layer (14 stages in 2 phases), rotating over the weight copies: what a
         # caller gets who launches layer by layer; bound by the serial latencies inside a launch, not by HBM
         lists1 = make_runlists(io1, 1)

@@ -133,7 +133,8 @@ typedef struct nq_linear {
 typedef struct nq_runlist_plan {
     int nlinears, nstages, nphases, workgroups, max_units, batch, dtype, index_words;
     int bound;              /* bit 0: some x was NULL, bit 1: some y was NULL (nq_runlist_run_bound must supply them);
-                               bit 2: the linears are in tile order (up to batch 4 all linears of a list must agree) */
+                               bit 2: the linears are in tile order (up to batch 4 all linears of a list must agree);
+                               bit 3: reproducible sums (nq_runlist_set_deterministic) */
 } nq_runlist_plan;
 
 size_t nq_runlist_workspace_bytes(const nq_linear* linears, int nlinears);
@@ -147,6 +148,14 @@ int nq_runlist_run(const void* workspace, const nq_runlist_plan* plan, void* str
  * by x_from / y_from. */
 int nq_runlist_run_bound(const void* workspace, const nq_runlist_plan* plan, const void* x, void* y, void* stream);
 int nq_runlist_status(const void* workspace, int* status_out, void* stream);
+/* Reproducible sums for the launches of this plan, on (1) or off (0, as built).  The run-list kernel finishes a row
+ * sum with additions from several wavefronts whose order differs from launch to launch, so outputs may differ in
+ * the last bit between launches (the reference's reductions are ordered: kernel/cuda/gemv_kernel.cu:148-170,
+ * shuffles inside one warp).  With this switch every launch of the plan gives bit-identical outputs: partial sums
+ * are rounded to a grid on which their additions are exact.  The results stay within the same tolerance but lose up
+ * to 16 bits below (columns x largest input value); available for batch 1, 2 and 4 (NQ_ERR_SHAPE otherwise).  Sets
+ * bit 3 of plan->bound. */
+int nq_runlist_set_deterministic(nq_runlist_plan* plan, int on);
 
 /* One matmul-free stage: out[b,row] = s_row[row] * sum_c sgn(bits[row,c]) * in[b,c] * s_col[c].
  * Replaces nanoquant_stage1_dyn_kernel / nanoquant_stage2_dyn_kernel launches

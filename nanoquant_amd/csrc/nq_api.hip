@@ -41,7 +41,7 @@ const char* nq_status_string(int status) {
 
 int nq_last_hip_error(void) { return g_last_hip_error; }
 
-int nq_abi_version(void) { return 5; }
+int nq_abi_version(void) { return 6; }
 
 int nq_device_query(int attr, int* value) {
     if (!value) return NQ_ERR_NULL;
@@ -505,7 +505,15 @@ int nq_runlist_run_bound(const void* workspace, const nq_runlist_plan* plan, con
     return hip_status(nq::gemv_stream(plan->dtype, batch, plan->nstages, (const nq::RunSlice*)(base + off_slices),
                                       (unsigned long long*)(base + 256),
                                       (unsigned*)base, plan->workgroups, plan->max_units, (hipStream_t)stream, x, y,
-                                      (plan->bound & 4) != 0));
+                                      (plan->bound & 4) != 0, (plan->bound & 8) != 0));
+}
+
+int nq_runlist_set_deterministic(nq_runlist_plan* plan, int on) {
+    if (!plan) return NQ_ERR_NULL;
+    if (plan->dtype != NQ_F16 && plan->dtype != NQ_BF16) return NQ_ERR_DTYPE;
+    if (on && !nq::stream_has_deterministic(plan->dtype, plan->batch)) return NQ_ERR_SHAPE;
+    plan->bound = on ? (plan->bound | 8) : (plan->bound & ~8);
+    return NQ_OK;
 }
 
 int nq_runlist_status(const void* workspace, int* status_out, void* stream) {

@@ -537,9 +537,12 @@ __device__ __forceinline__ uint32_t q8_scale_bytes(uint32_t eb) {
 // the columns of classes 0..2.  One pass, no barrier inside: a lane holds the 8 columns of one chunk, the 16 lanes
 // of a DPP row hold one unit, so the unit maximum never leaves the row.  A barrier must follow before the staged
 // data is read.
-template <int DT, int BATCH, int THREADS>
+// DET (reproducible sums): xtot is [wavefronts][4] instead, every wavefront adds to its own entries (in program order,
+// no atomics), and *ebmax (zeroed by the caller) receives the largest unit exponent eb of the staged chunk.
+template <int DT, int BATCH, int THREADS, bool DET = false>
 __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* scl, float* xtot, const StageInput& st, int c0,
-                                               int cu_n, int pitch) {
+                                               int cu_n, int pitch, uint32_t* ebmax = nullptr) {
+    static_assert(!DET || BATCH <= 4, "per-wavefront totals are laid out [wavefront][4]");
     using E = Elem<DT>;
     constexpr int kBurst = 2;                            // chunks per lane in flight
     const int units4 = q8_units4(cu_n);
@@ -644,7 +647,10 @@ __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* scl, float* 
             out.y = quad_transpose_rev((uint32_t)hi ^ 0x00808080u, lane & 1, lane & 2);
             if (it < total) dst[(size_t)k * pitch * 2] = out;
         }
-        if (it < total && (q & 15) == 0) scl[b * ((pitch - 1) >> 3) + cu] = q8_scale_bytes(eb);
+        if (it < total && (q & 15) == 0) {
+            scl[b * ((pitch - 1) >> 3) + cu] = q8_scale_bytes(eb);
+            if constexpr (DET) atomicMax(ebmax, eb);
+        }
         // sum of the staged values (= input - last residual) over the columns of classes 0..2, in the input's units
         const float after = ((u[2] + u[3]) + (u[4] + u[5])) + (u[6] + u[7]);
         return (before - after) * q8_inv_scale(eb);
@@ -668,7 +674,10 @@ __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* scl, float* 
         for (int j = 0; j < kBurst; ++j) {
             const int it = it0 + j * THREADS;
             const float t = group_sum_tail(tot[j], 64);
-            if (lane == 63 && it - lane < total) atomicAdd(&xtot[(it - lane) / nchunks], t);
+            if (lane == 63 && it - lane < total) {
+                if constexpr (DET) xtot[(threadIdx.x >> 6) * 4 + (it - lane) / nchunks] += t;
+                else atomicAdd(&xtot[(it - lane) / nchunks], t);
+            }
         }
     }
 }
@@ -723,6 +732,14 @@ __device__ __forceinline__ void unit_mfma_q8_pair(const uint4& wa, const uint4& 
     q8_class_pair<1>(wa, wb, o.lo1, o.hi1, scale, acc_a, acc_b);
     q8_class_pair<2>(wa, wb, o.lo2, o.hi2, scale, acc_a, acc_b);
     q8_class_pair<3>(wa, wb, o.lo3, o.hi3, scale, acc_a, acc_b);
+}
+
+// v rounded to the grid 2^-23 of the binade of c (c = 1.5 * 2^k, |v| < 2^(k-1)): sums of such values that stay below
+// 2^(k-1) are exact in fp32, so they do not depend on the order of the additions.
+__device__ __forceinline__ float grid_round(float v, float c) {
+    float t = v + c;
+    asm volatile("" : "+v"(t));
+    return t - c;
 }
 
 // Sum over the kQ8Pieces neighbouring columns of a batch row; valid in the lane of the last piece.

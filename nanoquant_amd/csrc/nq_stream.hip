@@ -93,19 +93,26 @@ __device__ __forceinline__ void trim_unit(const BitsView& v, uint4& w, int unit)
     }
 }
 
-// Bytes of LDS in front of the staged input: row sums and two sets of input totals [2][16].
-__host__ __device__ constexpr size_t stream_head_bytes(int batch, int arith) {
+// Bytes of LDS in front of the staged input: row sums and two sets of input totals [2][16].  Reproducible sums (det):
+// a second set of row sums (what earlier input chunks of the row block added up to), two sets of per-wavefront input
+// totals [2][16][4] and two exponent words.
+__host__ __device__ constexpr size_t stream_head_bytes(int batch, int arith, bool det = false) {
     (void)arith;
-    return (size_t)row_block(batch) * batch * sizeof(float) + 128;
+    return (size_t)row_block(batch) * batch * sizeof(float) * (det ? 2 : 1) + (det ? 1024 : 128);
 }
 
 // Items of the MFMA path that each wavefront of a workgroup takes (contiguous runs).
 __host__ __device__ __forceinline__ int mfma_items_per_wave(int nitems, int waves) { return (nitems + waves - 1) / waves; }
 
 // ARITH: 1 = MFMA with 16-bit operands, 2 = MFMA with one-bit fp4 weights and fp8 pieces of the input (batch <= 4).
+// DET (fp4 x fp8 arithmetic only): row sums that do not depend on the order in which the wavefronts of a workgroup add
+// their partial sums.  Every partial sum is rounded to a grid fine enough (2^-22 of columns x largest staged value, a
+// bound on every sum of the chunk) that all additions into a row sum are exact; the input totals are kept per wavefront
+// and added in wavefront order; the row sums of successive input chunks (different grids) are added one chunk after
+// the other.  Costs up to 16 bits below that bound in precision, two barriers per chunk of a long input, 4 KiB of LDS.
 // TILED (fp4 x fp8 arithmetic only): every stage of the list has its words in tile order; the 16-bit arithmetic reads
 // either order, stage by stage.
-template <int DT, int BATCH, int ARITH, int THREADS, bool SINGLE, bool TILED>
+template <int DT, int BATCH, int ARITH, int THREADS, bool SINGLE, bool TILED, bool DET = false>
 __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const RunSlice* __restrict__ slices,
                                                                      unsigned long long* counters, unsigned* status,
                                                                      unsigned spin_limit, int chunk_cap,
@@ -121,16 +128,21 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
     constexpr bool kPow2Mfma = ARITH == 1 && DT == 0;           // fp16 MFMA path: single-bit operands, pair-major x
     constexpr bool kTotals = kPow2Mfma || kQ8;                  // signed sum = (sum of x) - 2 (sum of b x)
     static_assert(!kQ8 || BATCH * kQ8Pieces <= 16, "pieces of all batch rows must fit the 16 operand columns");
+    static_assert(!DET || kQ8, "reproducible sums exist for the fp4 x fp8 arithmetic only");
     float* racc = (float*)lds_raw;                              // [kRowBlock][BATCH] row sums
-    // [2][16] sum of the staged input per batch row; slices alternate between the two, so that the one of the next
-    // slice is cleared a barrier ahead of its staging instead of costing a barrier of its own
-    float* xtot_base = racc + kRowBlock * BATCH;
-    uint4* xs_base = lds_raw + stream_head_bytes(BATCH, ARITH) / sizeof(uint4);
+    float* rtot = racc + kRowBlock * BATCH;                     // DET: the same, summed over the input chunks done so far
+    // [2][16] sum of the staged input per batch row (DET: [2][16 wavefronts][4]); slices alternate between the two, so
+    // that the one of the next slice is cleared a barrier ahead of its staging instead of costing a barrier of its own
+    constexpr int kTotStride = DET ? 64 : 16;
+    float* xtot_base = racc + kRowBlock * BATCH * (DET ? 2 : 1);
+    uint32_t* ebmax_base = (uint32_t*)(xtot_base + 2 * kTotStride);   // DET: [2] largest unit exponent of the staged input
+    uint4* xs_base = lds_raw + stream_head_bytes(BATCH, ARITH, DET) / sizeof(uint4);
     __shared__ int s_flag;
     const int tid = threadIdx.x;
     const int wg = blockIdx.x;
     if (tid == 0) s_flag = 0;
-    if (tid < 32) xtot_base[tid] = 0.f;
+    if (tid < 2 * kTotStride) xtot_base[tid] = 0.f;
+    if (DET && tid < 2) ebmax_base[tid] = 0u;
     int slice_count = 0;
 
     // Which launch of this run list is this?  Needed only by waiting slices; the load is issued now and
@@ -233,8 +245,9 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
             const int chunk_units = min(st.units, chunk_cap);
             const int upad = kQ8 ? q8_pitch(q8_units4(chunk_units)) : (chunk_units | 1);
             const bool one_chunk = chunk_units == st.units;
-            float* xtot = xtot_base + 16 * (slice_count & 1);
-            float* xtot_other = xtot_base + 16 * ((slice_count + 1) & 1);
+            float* xtot = xtot_base + kTotStride * (slice_count & 1);
+            float* xtot_other = xtot_base + kTotStride * ((slice_count + 1) & 1);
+            uint32_t* ebmax = ebmax_base + (slice_count & 1);
             ++slice_count;
             // kQ8: the unit scales (one dword per batch row and staged unit) sit in front of the pieces
             uint32_t* scl = (uint32_t*)xs_base;
@@ -368,14 +381,18 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
             }
             lds_barrier();                                       // s_flag; previous slice is done with xs / racc
             aborted = aborted || (s_flag != 0);
-            if (tid < 16) xtot_other[tid] = 0.f;                 // every reader of it (the previous slice) is past the barrier
+            if (tid < kTotStride) xtot_other[tid] = 0.f;         // every reader of it (the previous slice) is past the barrier
+            if (DET && tid == 0) ebmax_base[slice_count & 1] = 0u;   // slice_count was advanced: this is the other one
 
             if (!aborted) {
                 bool staged = false;
 #pragma unroll 1
                 for (int rb = seg.row_begin; rb < seg.row_end; rb += kRowBlock) {
                     const int nr = min(seg.row_end - rb, kRowBlock);
-                    for (int i = tid; i < nr * BATCH; i += kStreamThreads) racc[i] = 0.f;
+                    for (int i = tid; i < nr * BATCH; i += kStreamThreads) {
+                        racc[i] = 0.f;
+                        if constexpr (DET) rtot[i] = 0.f;
+                    }
 #pragma unroll 1
                     for (int c0 = 0; c0 < st.units; c0 += chunk_units) {
                         const int cu_n = min(chunk_units, st.units - c0);
@@ -385,10 +402,11 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                                 // the input is staged again for a further row block: the totals start over (the first
                                 // staging of a slice finds them cleared a barrier ahead); every reader of the previous
                                 // totals has passed a barrier by now
-                                if (tid < 16) xtot[tid] = 0.f;
+                                if (tid < kTotStride) xtot[tid] = 0.f;
+                                if (DET && tid == 0) *ebmax = 0u;
                                 lds_barrier();
                             }
-                            if constexpr (kQ8) stage_units_q8<DT, BATCH, THREADS>(xs, scl, xtot, sin, c0, cu_n, upad);
+                            if constexpr (kQ8) stage_units_q8<DT, BATCH, THREADS, DET>(xs, scl, xtot, sin, c0, cu_n, upad, ebmax);
                             else stage_units<DT, BATCH, kPow2Mfma>(xs, nullptr, sin, c0, cu_n, upad, kStreamThreads,
                                                                    kPow2Mfma ? xtot : nullptr);
                             staged = true;
@@ -425,11 +443,23 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                             int qscale = 0x7F7F7F7F;
                             float4_t acc_a = {0.f, 0.f, 0.f, 0.f}, acc_b = {0.f, 0.f, 0.f, 0.f};
                             int rp_run = rp;
+                            // DET: 1.5 * 2^k with 2^(k-1) above every partial and complete row sum of this chunk:
+                            // (columns) x (largest staged value) x 2 (classes 0..2 count twice, the totals make up for it)
+                            float det_c = 0.f;
+                            if constexpr (DET) {
+                                const uint32_t cols = (uint32_t)q8_units4(cu_n) * 128u;
+                                const uint32_t e = min(*ebmax + (32u - (uint32_t)__builtin_clz(cols - 1u)) + 3u, 254u);
+                                det_c = as_float((e << 23) | 0x400000u);
+                            }
                             auto flush = [&]() {
                                 // acc[v] = partial sum of row 32 rp_run + 4 g + v (acc_b: 16 rows further) for column r16
 #pragma unroll
                                 for (int v = 0; v < 4; ++v) {
-                                    const float sa = q8_piece_sum(acc_a[v]), sb = q8_piece_sum(acc_b[v]);
+                                    float sa = q8_piece_sum(acc_a[v]), sb = q8_piece_sum(acc_b[v]);
+                                    if constexpr (DET) {
+                                        sa = grid_round(sa, det_c);
+                                        sb = grid_round(sb, det_c);
+                                    }
                                     const int row = 32 * rp_run + 4 * g + v;
                                     if (qlast && row < nr) atomicAdd(&rdst[(32 * rp_run + v) * BATCH], sa);
                                     if (qlast && row + 16 < nr) atomicAdd(&rdst[(32 * rp_run + 16 + v) * BATCH], sb);
@@ -486,6 +516,18 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                                 if (it + 1 < it_end) step(wa1, wb1);
                             }
                             if (it_begin < it_end) flush();              // + the staged total of classes 0..2 at the end
+                            if constexpr (DET) {
+                                if (!one_chunk) {
+                                    // the next input chunk has a grid of its own: its sums are added to what the chunks
+                                    // so far came to, element by element (the loop top or the barrier below orders this
+                                    // against the next partial sums)
+                                    lds_barrier();
+                                    for (int i = tid; i < nr * BATCH; i += kStreamThreads) {
+                                        rtot[i] += racc[i];
+                                        racc[i] = 0.f;
+                                    }
+                                }
+                            }
                         } else {
                             // Items = (16-row group, 4-unit group), unit group fastest; every wavefront takes a
                             // contiguous run of items, so it mostly stays on one row group and adds its
@@ -540,7 +582,15 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                     for (int i = tid; i < nr * BATCH; i += kStreamThreads) {
                         const int row = rb + i / BATCH, b = i % BATCH;
                         float v = racc[i];
-                        if constexpr (kTotals) v += xtot[b];
+                        if constexpr (DET) {
+                            if (!one_chunk) v += rtot[i];
+                            float xt = 0.f;
+#pragma unroll
+                            for (int w = 0; w < kWaves; ++w) xt += xtot[4 * w + b];   // wavefront order
+                            v += xt;
+                        } else if constexpr (kTotals) {
+                            v += xtot[b];
+                        }
                         if (st.s_row) v *= E::to_float(st.s_row[row]);
                         if (st.bias) v += E::to_float(st.bias[row]);
                         const size_t o = (size_t)b * st.out_stride + row;
@@ -594,8 +644,8 @@ size_t stream_counter_bytes(int nstages) {
 }
 
 // ---- host side --------------------------------------------------------------------------------
-static void stream_lds_plan(int batch, int arith, int max_units, int* chunk_cap_out, size_t* lds_out) {
-    const int racc_bytes = (int)stream_head_bytes(batch, arith);
+static void stream_lds_plan(int batch, int arith, int max_units, int* chunk_cap_out, size_t* lds_out, bool det = false) {
+    const int racc_bytes = (int)stream_head_bytes(batch, arith, det && arith == 2);
     if (arith == 2) {
         // kQ8Pieces bytes per column and batch row, staged in whole groups of four units
         // plus one scale dword per batch row and unit
@@ -640,6 +690,10 @@ struct StreamKernel {
     static constexpr auto fn = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, false>;
     static constexpr auto fn_tiled = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2>;
     static constexpr auto fn_single = gemv_stream_kernel<DT, BATCH, kArith, kThreads, true, false>;
+    // reproducible sums: fp4 x fp8 arithmetic only (elsewhere these name the ordinary kernels and are never launched)
+    static constexpr bool kHasDet = kArith == 2;
+    static constexpr auto fn_det = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, false, kHasDet>;
+    static constexpr auto fn_tiled_det = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2, kHasDet>;
 };
 
 template <int DT, int BATCH>
@@ -650,6 +704,12 @@ static hipError_t prepare_kernel(size_t lds) {
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
         if (e != hipSuccess) return e;
         e = hipFuncSetAttribute((const void*)StreamKernel<DT, BATCH>::fn_tiled,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute((const void*)StreamKernel<DT, BATCH>::fn_det,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute((const void*)StreamKernel<DT, BATCH>::fn_tiled_det,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
         if (e != hipSuccess) return e;
         attr_done = true;
@@ -674,14 +734,18 @@ static int capacity_of(int max_units) {
 
 template <int DT, int BATCH>
 static hipError_t launch_stream(int nstages, const RunSlice* slices, unsigned long long* counters, unsigned* status, int nwg,
-                                int max_units, hipStream_t stream, const void* ext_in, void* ext_out, bool tiled) {
+                                int max_units, hipStream_t stream, const void* ext_in, void* ext_out, bool tiled, bool det) {
+    using SK = StreamKernel<DT, BATCH>;
+    if (det && !SK::kHasDet) return hipErrorInvalidValue;
     int chunk_cap;
     size_t lds;
-    stream_lds_plan(BATCH, StreamKernel<DT, BATCH>::kArith, max_units, &chunk_cap, &lds);
+    stream_lds_plan(BATCH, SK::kArith, max_units, &chunk_cap, &lds, det);
     hipError_t e = prepare_kernel<DT, BATCH>(lds);
     if (e != hipSuccess) return e;
-    using SK = StreamKernel<DT, BATCH>;
-    if (tiled && SK::kArith == 2)
+    if (det)
+        hipLaunchKernelGGL((tiled ? SK::fn_tiled_det : SK::fn_det), dim3(nwg), dim3(SK::kThreads), lds, stream, nstages, slices,
+                           counters, status, (unsigned)(1u << 21), chunk_cap, RunStage{}, 0, ext_in, ext_out);
+    else if (tiled && SK::kArith == 2)
         hipLaunchKernelGGL((SK::fn_tiled), dim3(nwg), dim3(SK::kThreads), lds, stream, nstages, slices, counters, status,
                            (unsigned)(1u << 21), chunk_cap, RunStage{}, 0, ext_in, ext_out);
     else
@@ -776,10 +840,18 @@ int stream_row_granule(int dtype, int batch) {
     return 32;
 }
 
+// Reproducible sums exist for the fp4 x fp8 arithmetic.
+bool stream_has_deterministic(int dtype, int batch) {
+#define NQ_DET(D, B) (StreamKernel<D, B>::kHasDet)
+    NQ_STREAM_DISPATCH(NQ_DET)
+#undef NQ_DET
+    return false;
+}
+
 hipError_t gemv_stream(int dtype, int batch, int nstages, const RunSlice* slices, unsigned long long* counters,
                        unsigned* status, int nwg, int max_units, hipStream_t stream, const void* ext_in, void* ext_out,
-                       bool tiled) {
-#define NQ_RUN(D, B) launch_stream<D, B>(nstages, slices, counters, status, nwg, max_units, stream, ext_in, ext_out, tiled)
+                       bool tiled, bool det) {
+#define NQ_RUN(D, B) launch_stream<D, B>(nstages, slices, counters, status, nwg, max_units, stream, ext_in, ext_out, tiled, det)
     NQ_STREAM_DISPATCH(NQ_RUN)
 #undef NQ_RUN
     return hipErrorInvalidValue;

@@ -38,7 +38,12 @@ class NqRunlistPlan(ctypes.Structure):
 class DecodeRunList:
     BATCHES = (1, 2, 4, 8, 16)
 
-    def __init__(self, batch: int, dtype: torch.dtype = torch.float16, device=None, interleave: int = 2):
+    def __init__(self, batch: int, dtype: torch.dtype = torch.float16, device=None, interleave: int = 2,
+                 deterministic: bool = False):
+        """`deterministic=True`: every launch of the list gives bit-identical outputs (batch 1, 2 and 4; partial sums
+        are rounded to a grid on which additions are exact, at a small cost in precision).  By default the order in
+        which the wavefronts of a workgroup add up a row sum is left to the hardware and the last bit may differ
+        from launch to launch."""
         if batch not in self.BATCHES:
             raise ValueError(f"run-list batch must be one of {self.BATCHES}, got {batch}")
         if dtype not in (torch.float16, torch.bfloat16):
@@ -47,6 +52,7 @@ class DecodeRunList:
         self.dtype = dtype
         self.device = torch.device(device if device is not None else "cuda")
         self.interleave = interleave
+        self.deterministic = bool(deterministic)
         self._entries: List[dict] = []
         self._keep: list = []          # tensors referenced by raw pointers stay alive here
         self._workspace: Optional[torch.Tensor] = None
@@ -125,6 +131,8 @@ class DecodeRunList:
             plan = NqRunlistPlan()
             _lib.check(lib.nq_runlist_build(arr, n, self.batch, self._dtype_id(), self.interleave,
                                             ctypes.c_void_p(ws.data_ptr()), nbytes, ctypes.byref(plan), stream))
+        if self.deterministic:
+            _lib.check(lib.nq_runlist_set_deterministic(ctypes.byref(plan), 1))
         self._plan = plan
         self._workspace = ws
         self._needs = (any(e["x"] is None for e in self._entries), any(e["y"] is None for e in self._entries))

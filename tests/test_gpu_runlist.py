@@ -322,3 +322,73 @@ def test_outlier_channels_leave_the_other_contributions_intact(dev, dtype, batch
     # 16-bit arithmetic (more than 4 rows) makes exactly the two roundings; in bf16 they carry 8 bits
     assert oracle.max_rel_err(y, ref) < (4e-3 if batch > 4 and dtype == torch.bfloat16 else 1e-3)
     assert figure <= 1.25 * allowed
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("batch,tiled", [(1, True), (1, False), (2, True), (4, True), (4, False)])
+def test_deterministic_lists_repeat_bit_for_bit(dev, batch, tiled, dtype):
+    """`deterministic=True`: every launch of a list gives the same bits (eager launches and graph replays alike), and
+    the results still meet the tolerance.  The shapes make many wavefronts add into the same row sums (few rows per
+    workgroup), include an input of 16384 columns (more than one staged chunk at batch 4) and a ragged one, and
+    the second linear reads the first one's output, so a difference anywhere upstream would show."""
+    shapes = [(1024, 4096, 512), (512, 16384, 736), (1376, 1000, 96)]
+    rl = DecodeRunList(batch, dtype, dev, deterministic=True)
+    plain = DecodeRunList(batch, dtype, dev)
+    refs = []
+    to = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev).to(dtype)
+    f64 = lambda t: t.float().cpu().numpy().astype(np.float64)
+    for i, (m, n, r) in enumerate(shapes):
+        vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, 600 + i)
+        vt_p, u_p, mid_p = oracle.pad_rank(vt, u, s_mid, 32)
+        words = lambda w: packing.binary_packer(torch.from_numpy(w), "half2").to(dev)
+        vt_d, u_d = words(vt_p), words(u_p)
+        if tiled:
+            vt_d, u_d = packing.tile_words(vt_d), packing.tile_words(u_d)
+        x = to(oracle.synth_x(batch, n, 610 + i))
+        sc = (to(s_in), to(mid_p), to(s_out))
+        for lst in (rl, plain):
+            lst.add(x, sc[0], vt_d, sc[1], u_d, sc[2], tiled=tiled, out_f32=True)
+        refs.append(oracle.layer_forward(f64(x), vt, u, f64(sc[0]), f64(to(s_mid)), f64(sc[2]), dtype=np.float64))
+    print(f"deterministic list batch={batch} tiled={tiled} {dtype}", flush=True)
+    first = [y.clone() for y in rl.run()]
+    torch.cuda.synchronize()
+    assert rl.status() == 0
+    for y, ref in zip(first, refs):
+        assert oracle.max_rel_err(y.cpu().numpy(), ref) < 1e-3
+    for rep in range(20):
+        for y in rl.outputs:
+            y.fill_(float("nan"))
+        ys = rl.run()
+        torch.cuda.synchronize()
+        for y, e in zip(ys, first):
+            assert torch.equal(y, e), rep
+    side = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        rl.run()
+    for rep in range(5):
+        for y in rl.outputs:
+            y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for y, e in zip(rl.outputs, first):
+            assert torch.equal(y, e), ("replay", rep)
+    assert rl.status() == 0
+    # for the record: how often the default mode repeats itself on the same list
+    base = [y.clone() for y in plain.run()]
+    torch.cuda.synchronize()
+    differing = 0
+    for rep in range(20):
+        ys = plain.run()
+        torch.cuda.synchronize()
+        differing += int(any(not torch.equal(y, e) for y, e in zip(ys, base)))
+    print(f"  default mode: {differing} of 20 launches differ from the first in some bit", flush=True)
+
+
+def test_deterministic_mode_is_refused_where_it_does_not_exist(dev):
+    _, ops = _term(dev, 256, 512, 64, seed=650)
+    rl = DecodeRunList(8, torch.float16, dev, deterministic=True)
+    rl.add(torch.from_numpy(oracle.synth_x(8, 512, 651)).to(dev), *ops)
+    with pytest.raises(RuntimeError):
+        rl.build()
