@@ -110,6 +110,9 @@ def main():
     ap.add_argument("--copies", type=int, default=32, help="decoder layers of the stack = distinct weight copies of the layer "
                                                            "(32 x 25.3 MB = 810 MB > 256 MB Infinity Cache)")
     ap.add_argument("--no-extra", action="store_true", help="skip batch 4/16, prefill and CPU legs")
+    ap.add_argument("--cfg4-only", action="store_true",
+                    help="after the headline run only the Llama-3-70B-shaped stream (cfg4) of the extra legs: the short "
+                         "command that the profiles of that leg are taken with")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the library's plain copy kernel on 256 MiB (5x): a known-traffic reference "
@@ -225,6 +228,31 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / steps  # ms per launch
 
+    def cfg4_leg(extra, batches=(1, 8)):
+        # ---- cfg4: Llama-3-70B-shaped weight stream, 80 layers x 7 linears in one launch ----
+        llama70 = (("q", 8192, 8192), ("k", 1024, 8192), ("v", 1024, 8192), ("o", 8192, 8192),
+                   ("gate", 28672, 8192), ("up", 28672, 8192), ("down", 8192, 28672))
+        g70 = torch.Generator(device=dev)
+        g70.manual_seed(5)
+        stack70 = [[SynthLinear(torch, dev, m, n, nominal_rank(m, n), g70) for (_, m, n) in llama70] for _ in range(80)]
+        for b in batches:
+            x70 = {n: torch.randn(b, n, device=dev, generator=g70).to(torch.float16) for n in (8192, 28672)}
+            rl = DecodeRunList(b, torch.float16, dev)
+            for layer in stack70:
+                for lin in layer:
+                    lin.add_to(rl, x70[lin.n])
+            rl.build()
+            ms70 = timed([rl.run], 5, 1)
+            if rl.status() != 0:
+                raise RuntimeError("run list reported an expired dependency wait")
+            bytes70 = 80 * sum(gemv_bytes(lin.m, lin.n, lin.r, b) for lin in stack70[0])
+            extra[f"cfg4_llama3_70b_stream_batch{b}"] = {
+                "us_per_token_step": round(ms70 * 1e3, 1), "GBps": round(bytes70 / (ms70 * 1e-3) / 1e9, 2),
+                "resident_weight_GB": round(80 * sum(lin.r * (lin.m + lin.n) / 8 for lin in stack70[0]) / 1e9, 2),
+                "note": "560 linears in one run-list launch"}
+            del rl
+        del stack70
+
     io1 = make_io(1)
     stack1 = make_stack(io1, 1)
     # set-up, not part of the W warm-up steps: 300 launches (45 ms) take the device to its sustained state (the first
@@ -291,7 +319,11 @@ def main():
         torch.cuda.synchronize()
         result["config"]["calibration_copy_bytes"] = nbytes
 
-    if not args.no_extra:
+    if args.cfg4_only:
+        extra = {}
+        cfg4_leg(extra)
+        result["extra"] = extra
+    elif not args.no_extra:
         extra = {}
         # measured streaming ceiling of this box: the library's plain copy kernel, 256 MiB read + 256 MiB written
         nbytes = 256 << 20
@@ -512,29 +544,7 @@ def main():
                     "flops at the nominal ranks"}
         del g, q_packed, q_groups
 
-        # ---- cfg4: Llama-3-70B-shaped weight stream, 80 layers x 7 linears in one launch ----
-        llama70 = (("q", 8192, 8192), ("k", 1024, 8192), ("v", 1024, 8192), ("o", 8192, 8192),
-                   ("gate", 28672, 8192), ("up", 28672, 8192), ("down", 8192, 28672))
-        g70 = torch.Generator(device=dev)
-        g70.manual_seed(5)
-        stack70 = [[SynthLinear(torch, dev, m, n, nominal_rank(m, n), g70) for (_, m, n) in llama70] for _ in range(80)]
-        for b in (1, 8):
-            x70 = {n: torch.randn(b, n, device=dev, generator=g70).to(torch.float16) for n in (8192, 28672)}
-            rl = DecodeRunList(b, torch.float16, dev)
-            for layer in stack70:
-                for lin in layer:
-                    lin.add_to(rl, x70[lin.n])
-            rl.build()
-            ms70 = timed([rl.run], 5, 1)
-            if rl.status() != 0:
-                raise RuntimeError("run list reported an expired dependency wait")
-            bytes70 = 80 * sum(gemv_bytes(lin.m, lin.n, lin.r, b) for lin in stack70[0])
-            extra[f"cfg4_llama3_70b_stream_batch{b}"] = {
-                "us_per_token_step": round(ms70 * 1e3, 1), "GBps": round(bytes70 / (ms70 * 1e-3) / 1e9, 2),
-                "resident_weight_GB": round(80 * sum(lin.r * (lin.m + lin.n) / 8 for lin in stack70[0]) / 1e9, 2),
-                "note": "560 linears in one run-list launch"}
-            del rl
-        del stack70
+        cfg4_leg(extra)
         result["extra"] = extra
 
         # ---- CPU baseline: the reference's dense path on this host (bounded sample) ----
