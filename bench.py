@@ -390,6 +390,36 @@ def main():
         extra["batch1_per_linear_launches"] = {"us_per_layer": round(ms_pl * 1e3, 3),
                                                "GBps": round(bytes1 / (ms_pl * 1e-3) / 1e9, 2),
                                                "note": "same layer through nq_gemv_forward: 14 launches per layer"}
+        # ---- the module interface (NanoQuantLinear prepared for decode, one call per linear), by row count ----
+        from nanoquant_amd.linear import NanoQuantLinear
+
+        def decode_module(lin):
+            mod = NanoQuantLinear(lin.n, lin.m, lin.rp, dtype=torch.float16, device=dev)
+            for name in ("V", "U"):
+                delattr(mod, name)
+            mod.do_kernel_inference, mod.kernel_type, mod.dtype = True, "gemv", torch.float16
+            mod.V_int8, mod.U_int8 = lin.vt_bits, lin.u_bits
+            for name, t in (("scale_pre", lin.s_in), ("scale_mid", lin.s_mid), ("scale_post", lin.s_out)):
+                setattr(mod, name, torch.nn.Parameter(t, requires_grad=False))
+            mod.kernel_forward = torch.ops.binary_kernels.nanoquant_dyn_forward
+            mod.kernel_kwargs = {}
+            return mod
+
+        mods = [[decode_module(lin) for lin in layer] for layer in layers]
+        for layer in mods:
+            for mod in layer:
+                mod.prepare_mfma_route()       # set-up: otherwise the first call of 3 or more rows builds the tiles
+        by_rows = {}
+        with torch.no_grad():
+            for rows in (1, 2, 4, 16):
+                xs_m = {n: torch.randn(rows, n, device=dev).to(torch.float16) for n in (4096, 11008)}
+                fns = [(lambda layer=layer: [mod(xs_m[mod.in_features]) for mod in layer]) for layer in mods]
+                by_rows[str(rows)] = round(timed(fns, 2 * len(layers), len(layers)) * 1e3, 1)
+        extra["module_forward_us_per_layer_by_rows"] = dict(
+            by_rows, note="NanoQuantLinear.forward of 7 modules prepared with kernel_type='gemv', graph replays over the "
+                          "rotating weight copies: two decode launches per linear up to 2 rows, the few-token MFMA tiles "
+                          "(built once from the decode words) from 3 rows on")
+        del mods
         # ---- prefill GEMM over the three distinct linear shapes of the layer ----
         # Timed as HIP graph replays: through Python the two-GEMM op costs more host time than GPU time.
         op = torch.ops.binary_kernels.marlin_nanoquant_forward

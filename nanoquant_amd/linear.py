@@ -47,6 +47,14 @@ class NanoQuantLinear(nn.Module):
         # scales and the bias) on a list built once per row count, instead of the two launches of the
         # reference's op (linear.py:121-130).  It bypasses the torch op, so leave it off under torch.compile.
         self.fused_launch = False
+        # A module prepared for decode ("gemv") sends calls of at least this many rows to the few-token MFMA tiles of
+        # the prefill path (0: never).  Their cost does not depend on the row count (109 us per Llama-2-7B layer of 7
+        # linears, weights from HBM), that of the decode kernels grows with every row: 75 / 94 / 164 / 131 / 220 / 195 us
+        # at 1 / 2 / 3 / 4 / 6 / 16 rows.  The prefill tiles are built once from the decode words on the first such
+        # call (or by `prepare_mfma_route()`), on the device, and kept beside them: a second copy of the packed
+        # factors.  Needs in_features % 256 == 0 and out_features % 32 == 0; other shapes stay on the decode kernels.
+        self.mfma_from_rows = 3
+        self._mfma_tiles = None
         self._fused_lists = {}
         self._fused_tiled = None
         self._fused_bias = None
@@ -122,6 +130,12 @@ class NanoQuantLinear(nn.Module):
                 bias = self.bias if self.bias.dtype == self.dtype else self.bias.to(self.dtype)
             if self.kernel_type == "gemv" and self.fused_launch and x.shape[0] in DecodeRunList.BATCHES:
                 y = self._fused_forward(x, bias)
+            elif self.kernel_type == "gemv" and self._routes_to_mfma(x):
+                tiles = self._mfma_tiles
+                if bias is not None:
+                    y = ops.gemm_forward_with_bias(x, *tiles, bias)
+                else:
+                    y = torch.ops.binary_kernels.marlin_nanoquant_forward(x, *tiles)
             elif self.kernel_type == "gemv":
                 if bias is not None:
                     y = ops.gemv_forward_with_bias(x, self.scale_pre, self.V_int8, self.scale_mid, self.U_int8,
@@ -146,6 +160,32 @@ class NanoQuantLinear(nn.Module):
         if self.bias is not None:
             y += self.bias
         return y
+
+    def _routes_to_mfma(self, x: torch.Tensor) -> bool:
+        """Whether this decode call runs on the prefill path's few-token tiles; builds them on first use (eagerly:
+        under torch.compile and during a stream capture only tiles made beforehand are used)."""
+        if not self.mfma_from_rows or x.shape[0] < self.mfma_from_rows or not x.is_cuda:
+            return False
+        if self.in_features % 256 != 0 or self.out_features % 32 != 0:
+            return False
+        if self._mfma_tiles is None or self._mfma_tiles[0].device != x.device:
+            # never build inside a trace or a stream capture (the packing pass and its allocations would become part
+            # of the graph): such a call stays on the decode kernels unless the tiles were prepared beforehand
+            if torch.compiler.is_compiling() or torch.cuda.is_current_stream_capturing():
+                return False
+            self.prepare_mfma_route()
+        return True
+
+    def prepare_mfma_route(self) -> None:
+        """Prefill tiles (the 6-tuple of `marlin_nanoquant_packer`) from the decode words of a module prepared with
+        kernel_type "gemv": one pass over the words on their device, no dense matrix."""
+        if not getattr(self, "do_kernel_inference", False) or self.kernel_type != "gemv":
+            raise RuntimeError("prepare_mfma_route() needs a module prepared with kernel_type='gemv'")
+        if self.in_features % 256 != 0 or self.out_features % 32 != 0:
+            raise ValueError("the prefill path needs in_features % 256 == 0 and out_features % 32 == 0")
+        self._mfma_tiles = pack_binary_marlin_fused_from_words(
+            self.V_int8, self.U_int8, self.rank, self.scale_pre.data,
+            None if self.scale_mid is None else self.scale_mid.data, self.scale_post.data, "half2")
 
     def _fused_forward(self, x: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
         """One launch for the whole layer: a one-entry run list per row count whose input and output are
@@ -217,6 +257,7 @@ class NanoQuantLinear(nn.Module):
         self.kernel_type = kernel_type
         self.dtype = dtype
         self._fused_lists, self._fused_tiled, self._fused_bias = {}, None, None
+        self._mfma_tiles = None
 
         self.scale_pre = nn.Parameter(self.scale_pre.to(dtype).squeeze(0), requires_grad=False)
         self.scale_post = nn.Parameter(self.scale_post.to(dtype).squeeze(0), requires_grad=False)
@@ -298,6 +339,7 @@ class NanoQuantLinear(nn.Module):
                 delattr(self, name)
         self.in_features, self.out_features = v_shape[1], u_shape[0]
         self._fused_lists, self._fused_tiled, self._fused_bias = {}, None, None   # built on the previous words
+        self._mfma_tiles = None
         self._prepare_scales_only(dtype)
         if kernel_type == "gemv":
             self.V_int8 = repack_words(v_words, "lsb_first", "half2")
