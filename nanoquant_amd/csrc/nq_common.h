@@ -3,7 +3,24 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace nq {
+
+// Host side: "done once on this device" for settings that HIP keeps per device (function attributes) and for values
+// queried per device.  One bit per device ordinal; devices beyond 63 simply repeat the (idempotent) work.  Safe for
+// concurrent first calls: two threads may both do the work, none skips it.
+struct PerDeviceFlag {
+    std::atomic<unsigned long long> bits{0};
+    bool test(int dev) const { return dev >= 0 && dev < 64 && ((bits.load(std::memory_order_acquire) >> dev) & 1ull); }
+    void set(int dev) {
+        if (dev >= 0 && dev < 64) bits.fetch_or(1ull << dev, std::memory_order_release);
+    }
+};
+inline int current_device() {
+    int dev = -1;
+    return hipGetDevice(&dev) == hipSuccess ? dev : -1;
+}
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf162_t __attribute__((ext_vector_type(2)));

@@ -538,11 +538,12 @@ size_t gemm_scratch_bytes(int T, int K, int R) {
 template <int DT, int TT, int RT, int KS, bool SPLIT, bool SCALED>
 static hipError_t launch_variant(const GemmArgs& a, dim3 grid, size_t lds, hipStream_t stream) {
     auto kern = gemm_onebit_kernel<DT, TT, RT, KS, SPLIT, SCALED>;
-    static bool attr_done = false;
-    if (lds > 64 * 1024 && !attr_done) {
+    static PerDeviceFlag attr_done;              // per template instance and device
+    const int dev = current_device();
+    if (lds > 64 * 1024 && !attr_done.test(dev)) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        attr_done = true;
+        attr_done.set(dev);
     }
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);
     return hipSuccess;

@@ -174,11 +174,12 @@ static hipError_t launch_stage(StageArgs a, hipStream_t stream) {
     const int grid = (a.rows + rows_per_block - 1) / rows_per_block;
     const size_t lds_bytes = (size_t)BATCH * kXsumBytesPerRow + (size_t)xs_chunks(BATCH, a.chunk_units | 1) * sizeof(uint4);
     auto kern = gemv_stage_kernel<DT, FIRST, BATCH, RPW>;
-    static bool attr_done = false;  // per template instance; raised once to the full budget
-    if (lds_bytes > 64 * 1024 && !attr_done) {
+    static PerDeviceFlag attr_done;  // per template instance and device; raised once to the full budget
+    const int dev = current_device();
+    if (lds_bytes > 64 * 1024 && !attr_done.test(dev)) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
         if (e != hipSuccess) return e;
-        attr_done = true;
+        attr_done.set(dev);
     }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, a);
     return hipGetLastError();

@@ -698,8 +698,9 @@ struct StreamKernel {
 
 template <int DT, int BATCH>
 static hipError_t prepare_kernel(size_t lds) {
-    static bool attr_done = false;
-    if (lds > 64 * 1024 && !attr_done) {
+    static PerDeviceFlag attr_done;              // per template instance and device
+    const int dev = current_device();
+    if (lds > 64 * 1024 && !attr_done.test(dev)) {
         hipError_t e = hipFuncSetAttribute((const void*)StreamKernel<DT, BATCH>::fn,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
         if (e != hipSuccess) return e;
@@ -712,7 +713,7 @@ static hipError_t prepare_kernel(size_t lds) {
         e = hipFuncSetAttribute((const void*)StreamKernel<DT, BATCH>::fn_tiled_det,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
         if (e != hipSuccess) return e;
-        attr_done = true;
+        attr_done.set(dev);
     }
     return hipSuccess;
 }
@@ -761,22 +762,26 @@ static hipError_t launch_single(const RunStage& st, hipStream_t stream) {
     int chunk_cap;
     size_t lds;
     stream_lds_plan(BATCH, SK::kArith, st.units, &chunk_cap, &lds);
-    static bool attr_done = false;
-    if (lds > 64 * 1024 && !attr_done) {
+    static PerDeviceFlag attr_done;              // per template instance and device
+    const int dev = current_device();
+    if (lds > 64 * 1024 && !attr_done.test(dev)) {
         hipError_t e = hipFuncSetAttribute((const void*)SK::fn_single, hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
         if (e != hipSuccess) return e;
-        attr_done = true;
+        attr_done.set(dev);
     }
-    static size_t cached_lds = 0;                // per template instance: the occupancy query is host time
-    static int cached_cap = 0;
-    if (cached_cap <= 0 || cached_lds != lds) {
-        int per_cu = 0, dev = 0, cus = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)SK::fn_single, SK::kThreads, lds) != hipSuccess ||
-            hipGetDevice(&dev) != hipSuccess ||
+    // resident workgroups of this kernel on this device: the query is host time, so the last answer per calling thread
+    // is kept (keyed by device and LDS size)
+    static thread_local size_t cached_lds = 0;
+    static thread_local int cached_dev = -1, cached_cap = 0;
+    if (cached_cap <= 0 || cached_lds != lds || cached_dev != dev) {
+        int per_cu = 0, cus = 0;
+        if (dev < 0 ||
+            hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)SK::fn_single, SK::kThreads, lds) != hipSuccess ||
             hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
             return hipErrorInvalidValue;
         cached_cap = per_cu * cus;
         cached_lds = lds;
+        cached_dev = dev;
     }
     const int cap = cached_cap;
     if (cap <= 0) return hipErrorInvalidValue;
