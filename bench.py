@@ -256,13 +256,13 @@ def main():
     io1 = make_io(1)
     stack1 = make_stack(io1, 1)
     # set-up, not part of the W warm-up steps: 300 launches (45 ms) take the device to its sustained state (the first
-    # 25 ms of back-to-back launches after the weights were generated run up to 15 % slower), and the step is captured
-    # once as a HIP graph so that the timed loop costs the host a replay per step
+    # 25 ms of back-to-back launches after the weights were generated run up to 15 % slower).  The W warm-up steps and
+    # the K timed steps are then launched back to back on the current stream (a launch costs the host 10 us, a step
+    # takes the device 140: the queue never runs dry; replaying a one-launch graph per step leaves 4 us between steps)
     for _ in range(300):
         stack1.run()
     torch.cuda.synchronize()
-    step_graph = capture_rotation([stack1.run])
-    ms = timed_launches(step_graph.replay, args.steps, args.warmup)
+    ms = timed_launches(stack1.run, args.steps, args.warmup)
     if stack1.status() != 0:
         raise RuntimeError("run list reported an expired dependency wait")
     nlayers = len(layers)
