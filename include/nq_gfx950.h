@@ -135,6 +135,9 @@ typedef struct nq_runlist_plan {
     int bound;              /* bit 0: some x was NULL, bit 1: some y was NULL (nq_runlist_run_bound must supply them);
                                bit 2: the linears are in tile order (up to batch 4 all linears of a list must agree);
                                bit 3: reproducible sums (nq_runlist_set_deterministic) */
+    int spin_limit;         /* polls after which a dependency wait gives up and sets the status word; 0 (as built) =
+                               the default of 2^21 polls, about a second.  The caller may lower it, e.g. to exercise
+                               its handling of an expired wait: every kernel still runs to its end */
 } nq_runlist_plan;
 
 size_t nq_runlist_workspace_bytes(const nq_linear* linears, int nlinears);

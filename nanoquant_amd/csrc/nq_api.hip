@@ -41,7 +41,7 @@ const char* nq_status_string(int status) {
 
 int nq_last_hip_error(void) { return g_last_hip_error; }
 
-int nq_abi_version(void) { return 6; }
+int nq_abi_version(void) { return 7; }
 
 int nq_device_query(int attr, int* value) {
     if (!value) return NQ_ERR_NULL;
@@ -481,6 +481,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
     plan_out->dtype = dtype;
     plan_out->index_words = (int)records.size();
     plan_out->bound = 0;
+    plan_out->spin_limit = 0;
     for (int i = 0; i < nlinears; ++i) plan_out->bound |= (linears[i].x ? 0 : 1) | (linears[i].y ? 0 : 2);
     if (linears[0].tiled) plan_out->bound |= 4;
     return hip_status(hipStreamSynchronize(hs));   // the tables are host memory: finish before they die
@@ -505,7 +506,8 @@ int nq_runlist_run_bound(const void* workspace, const nq_runlist_plan* plan, con
     return hip_status(nq::gemv_stream(plan->dtype, batch, plan->nstages, (const nq::RunSlice*)(base + off_slices),
                                       (unsigned long long*)(base + 256),
                                       (unsigned*)base, plan->workgroups, plan->max_units, (hipStream_t)stream, x, y,
-                                      (plan->bound & 4) != 0, (plan->bound & 8) != 0));
+                                      (plan->bound & 4) != 0, (plan->bound & 8) != 0,
+                                      plan->spin_limit > 0 ? (unsigned)plan->spin_limit : 0u));
 }
 
 int nq_runlist_set_deterministic(nq_runlist_plan* plan, int on) {

@@ -57,7 +57,7 @@ int stream_chunk_cap(int dtype, int batch, int max_units);
 int stream_row_granule(int dtype, int batch);
 hipError_t gemv_stream(int dtype, int batch, int nstages, const RunSlice* slices, unsigned long long* counters,
                        unsigned* status, int nwg, int max_units, hipStream_t stream, const void* ext_in = nullptr,
-                       void* ext_out = nullptr, bool tiled = false, bool det = false);
+                       void* ext_out = nullptr, bool tiled = false, bool det = false, unsigned spin_limit = 0);
 bool stream_needs_uniform_order(int dtype, int batch);
 bool stream_has_deterministic(int dtype, int batch);
 

@@ -367,7 +367,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                             unsigned flagged = 0;
                             if (tid == 0) flagged = __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                             flagged = __shfl(flagged, 0, kWave);
-                            if (++spins > spin_limit || flagged) {
+                            if (++spins >= spin_limit || flagged) {
                                 if (tid == 0) atomicOr(status, 1u);   // bounded wait: flag it, let the grid drain
                                 bad = true;
                                 break;
@@ -736,8 +736,10 @@ static int capacity_of(int max_units) {
 
 template <int DT, int BATCH>
 static hipError_t launch_stream(int nstages, const RunSlice* slices, unsigned long long* counters, unsigned* status, int nwg,
-                                int max_units, hipStream_t stream, const void* ext_in, void* ext_out, bool tiled, bool det) {
+                                int max_units, hipStream_t stream, const void* ext_in, void* ext_out, bool tiled, bool det,
+                                unsigned spin_limit) {
     using SK = StreamKernel<DT, BATCH>;
+    if (spin_limit == 0) spin_limit = 1u << 21;                  // about a second of polling
     if (det && !SK::kHasDet) return hipErrorInvalidValue;
     int chunk_cap;
     size_t lds;
@@ -746,13 +748,13 @@ static hipError_t launch_stream(int nstages, const RunSlice* slices, unsigned lo
     if (e != hipSuccess) return e;
     if (det)
         hipLaunchKernelGGL((tiled ? SK::fn_tiled_det : SK::fn_det), dim3(nwg), dim3(SK::kThreads), lds, stream, nstages, slices,
-                           counters, status, (unsigned)(1u << 21), chunk_cap, RunStage{}, 0, ext_in, ext_out);
+                           counters, status, spin_limit, chunk_cap, RunStage{}, 0, ext_in, ext_out);
     else if (tiled && SK::kArith == 2)
         hipLaunchKernelGGL((SK::fn_tiled), dim3(nwg), dim3(SK::kThreads), lds, stream, nstages, slices, counters, status,
-                           (unsigned)(1u << 21), chunk_cap, RunStage{}, 0, ext_in, ext_out);
+                           spin_limit, chunk_cap, RunStage{}, 0, ext_in, ext_out);
     else
         hipLaunchKernelGGL((SK::fn), dim3(nwg), dim3(SK::kThreads), lds, stream, nstages, slices, counters, status,
-                           (unsigned)(1u << 21), chunk_cap, RunStage{}, 0, ext_in, ext_out);
+                           spin_limit, chunk_cap, RunStage{}, 0, ext_in, ext_out);
     return hipGetLastError();
 }
 
@@ -856,8 +858,8 @@ bool stream_has_deterministic(int dtype, int batch) {
 
 hipError_t gemv_stream(int dtype, int batch, int nstages, const RunSlice* slices, unsigned long long* counters,
                        unsigned* status, int nwg, int max_units, hipStream_t stream, const void* ext_in, void* ext_out,
-                       bool tiled, bool det) {
-#define NQ_RUN(D, B) launch_stream<D, B>(nstages, slices, counters, status, nwg, max_units, stream, ext_in, ext_out, tiled, det)
+                       bool tiled, bool det, unsigned spin_limit) {
+#define NQ_RUN(D, B) launch_stream<D, B>(nstages, slices, counters, status, nwg, max_units, stream, ext_in, ext_out, tiled, det, spin_limit)
     NQ_STREAM_DISPATCH(NQ_RUN)
 #undef NQ_RUN
     return hipErrorInvalidValue;

@@ -32,7 +32,8 @@ class NqRunlistPlan(ctypes.Structure):
     """Mirror of `nq_runlist_plan`."""
     _fields_ = [("nlinears", ctypes.c_int), ("nstages", ctypes.c_int), ("nphases", ctypes.c_int),
                 ("workgroups", ctypes.c_int), ("max_units", ctypes.c_int), ("batch", ctypes.c_int),
-                ("dtype", ctypes.c_int), ("index_words", ctypes.c_int), ("bound", ctypes.c_int)]
+                ("dtype", ctypes.c_int), ("index_words", ctypes.c_int), ("bound", ctypes.c_int),
+                ("spin_limit", ctypes.c_int)]
 
 
 class DecodeRunList:
@@ -53,6 +54,9 @@ class DecodeRunList:
         self.device = torch.device(device if device is not None else "cuda")
         self.interleave = interleave
         self.deterministic = bool(deterministic)
+        # polls after which a dependency wait inside the kernel gives up (then status() == 1 and the outputs of that
+        # launch are invalid); 0 = the library's default, about a second.  Takes effect with the next run().
+        self.spin_limit = 0
         self._entries: List[dict] = []
         self._keep: list = []          # tensors referenced by raw pointers stay alive here
         self._workspace: Optional[torch.Tensor] = None
@@ -160,6 +164,7 @@ class DecodeRunList:
             if not t.is_cuda or not t.is_contiguous() or t.dtype != dt or t.numel() != self.batch * width:
                 raise RuntimeError(f"{name} must be a contiguous {dt} tensor of {self.batch} x {width} on the GPU")
         p = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())
+        self._plan.spin_limit = int(self.spin_limit)
         with torch.cuda.device(self.device):
             stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
             _lib.check(_lib.lib().nq_runlist_run_bound(ctypes.c_void_p(self._workspace.data_ptr()),

@@ -392,3 +392,34 @@ def test_deterministic_mode_is_refused_where_it_does_not_exist(dev):
     rl.add(torch.from_numpy(oracle.synth_x(8, 512, 651)).to(dev), *ops)
     with pytest.raises(RuntimeError):
         rl.build()
+
+
+def test_an_expired_wait_is_reported_and_the_list_stays_usable(dev):
+    """The dependency waits inside the kernel are bounded.  With the bound lowered to one poll from the host, the first
+    workgroup that finds its producers unfinished gives up and flags the launch; every kernel still runs to its end.
+    The status word reports it once (reading clears it), and the same list works again with the default bound."""
+    batch = 1
+    rl = DecodeRunList(batch, torch.float16, dev)
+    refs = []
+    # rank 40: two workgroups compute the first stage, the workgroups of the second stage have nothing else to do and
+    # poll while those two are still at work
+    for i, (m, n, r) in enumerate([(8192, 4096, 40)]):
+        term, ops = _term(dev, m, n, r, seed=800 + i)
+        x = oracle.synth_x(batch, n, 810 + i)
+        rl.add(torch.from_numpy(x).to(dev), *ops)
+        refs.append(oracle.layer_forward(x.astype(np.float64), *term, dtype=np.float64))
+    rl.run()
+    torch.cuda.synchronize()
+    assert rl.status() == 0
+    print("run list with a dependency wait of one poll", flush=True)
+    rl.spin_limit = 1
+    rl.run()
+    torch.cuda.synchronize()
+    assert rl.status() == 1                                            # reported ...
+    assert rl.status() == 0                                            # ... once: reading cleared it
+    rl.spin_limit = 0
+    ys = rl.run()
+    torch.cuda.synchronize()
+    assert rl.status() == 0
+    for y, ref in zip(ys, refs):
+        assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < 1e-2   # rank 40: the fp16-output budget
