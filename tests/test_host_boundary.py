@@ -243,3 +243,40 @@ def test_ops_trace_under_fake_tensors_and_make_fx():
         g = make_fx(layer, tracing_mode="real")(*args)
     targets = [n.target for n in g.graph.nodes if n.op == "call_function"]
     assert targets == [torch.ops.binary_kernels.nanoquant_dyn_forward.default]
+
+
+def test_row_routing_and_run_list_options_need_no_gpu():
+    """Host logic of the options added to the module and the run list: defaults, state checks, plan mirror."""
+    import ctypes
+    from nanoquant_amd.runlist import DecodeRunList, NqRunlistPlan
+    vt, u, s_in, s_mid, s_out = oracle.synth_term(64, 256, 32, seed=9)
+    f = lambda a: torch.from_numpy(a.astype(np.float32))
+    mod = NanoQuantLinear.from_factors(f(vt), f(u), f(s_in), f(s_mid), f(s_out), dtype=torch.float32)
+    assert mod.mfma_from_rows == 3 and mod._mfma_tiles is None
+    with pytest.raises(RuntimeError, match="kernel_type='gemv'"):
+        mod.prepare_mfma_route()                                       # not prepared for decode yet
+    mod._prepare_kernel("gemv", torch.float16)
+    assert not mod._routes_to_mfma(torch.zeros(8, 256))                # CPU tensors never route (and never build tiles)
+    assert mod._mfma_tiles is None
+    mod.prepare_mfma_route()                                           # the packing pass itself runs on any device
+    dense = NanoQuantLinear.from_factors(f(vt), f(u), f(s_in), f(s_mid), f(s_out), dtype=torch.float32)
+    dense._prepare_kernel("gemm", torch.float16)
+    assert torch.equal(mod._mfma_tiles[0], dense.V_int8) and torch.equal(mod._mfma_tiles[1], dense.U_int8)
+    odd = NanoQuantLinear.from_factors(f(vt[:, :96]), f(u), f(s_in[:96]), f(s_mid), f(s_out), dtype=torch.float32)
+    odd._prepare_kernel("gemv", torch.float16)
+    with pytest.raises(ValueError, match="in_features % 256"):
+        odd.prepare_mfma_route()
+    # the plan mirror has the library's layout (the library fills it; a mismatch would shift every field)
+    names = [n for n, _ in NqRunlistPlan._fields_]
+    assert names == ["nlinears", "nstages", "nphases", "workgroups", "max_units", "batch", "dtype", "index_words", "bound",
+                     "spin_limit"]
+    assert ctypes.sizeof(NqRunlistPlan) == 10 * ctypes.sizeof(ctypes.c_int)
+    rl = DecodeRunList(4, torch.float16, "cpu", deterministic=True)
+    assert rl.deterministic and rl.spin_limit == 0
+    with pytest.raises(ValueError):
+        DecodeRunList(3, torch.float16, "cpu")
+    plan = NqRunlistPlan(batch=8, dtype=_lib.NQ_F16)
+    assert _lib.lib().nq_runlist_set_deterministic(ctypes.byref(plan), 1) != 0      # no such kernel at batch 8
+    plan = NqRunlistPlan(batch=4, dtype=_lib.NQ_F16)
+    assert _lib.lib().nq_runlist_set_deterministic(ctypes.byref(plan), 1) == 0 and plan.bound & 8
+    assert _lib.lib().nq_runlist_set_deterministic(ctypes.byref(plan), 0) == 0 and not plan.bound & 8
