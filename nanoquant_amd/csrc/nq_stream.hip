@@ -27,8 +27,9 @@ namespace nq {
 // Rows whose sums a workgroup keeps in LDS at a time (then: barrier, scale, store, barrier): every block of a slice
 // ends with all wavefronts waiting for the slowest one, so few large blocks -- 1024 rows up to batch 4 (16 KiB of row
 // sums at batch 4; 256-row blocks cost the batch-4 stack 8.6 instead of 6.2 us per layer).  The 16-bit arithmetic
-// needs its LDS for the staged rows: 512 rows at batch 8, 256 at batch 16 (= 16 row groups, one per wavefront).
-__host__ __device__ constexpr int row_block(int batch) { return batch <= 4 ? 1024 : batch == 8 ? 512 : 256; }
+// at batch 16 needs its LDS for the staged rows: 256 rows there (= 16 row groups, one per wavefront; 320, 384 and 512
+// measured no better), 1024 at batch 8 (stack 14.5 -> 13.9 us per layer against 512).
+__host__ __device__ constexpr int row_block(int batch) { return batch <= 8 ? 1024 : 256; }
 // Same-address device-scope atomics serialise at the memory side (tens of ns each), so completion
 // counts are spread over kSubCounters addresses per stage and kExitSubs addresses for the exit count,
 // one 64-byte line each.
