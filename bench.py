@@ -30,6 +30,9 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the headline kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
 # copy kernel of known size (profiles/gemv_stream_llama2_7b_stack_b1.md); valid for the default workload only.
 MEASURED_TRAFFIC_BYTES = 840352768
+# The same for the two launches of the 128-token grouped layer (profiles/gemm_group_llama2_7b_layer_prefill.md):
+# (18776 + 27306) KiB x 2.000 fetched + (4352 + 10624) KiB written.
+MEASURED_PREFILL_TRAFFIC_BYTES = (18776 + 27306) * 2 * 1024 + (4352 + 10624) * 1024
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 LLAMA2_7B_LAYER = (("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096),
@@ -483,7 +486,7 @@ def main():
                     "kernel": "gemm_kwave_group_kernel<fp16> x 2 launches (first GEMMs of the 7 linears, then second GEMMs)",
                     "achieved": round(tf, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "flops_per_layer": int(group_flops),
-                    "us_per_layer": round(us, 2), "traffic": None}
+                    "us_per_layer": round(us, 2), "traffic": MEASURED_PREFILL_TRAFFIC_BYTES}
             if tokens == 16:
                 # the same 16 rows as extra.batch16, on the prefill kernels and with cold weights as there: every
                 # linear of every rotation step reads its own copy of the packed tiles (args.copies x 7 clones)
