@@ -423,3 +423,48 @@ def test_an_expired_wait_is_reported_and_the_list_stays_usable(dev):
     assert rl.status() == 0
     for y, ref in zip(ys, refs):
         assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < 1e-2   # rank 40: the fp16-output budget
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_lists_match_the_oracle(dev, seed):
+    """Seeded random lists: batch, type, word order, reproducible sums, 1 to 4 linears of ragged shapes, some fed by
+    the linear before them."""
+    rng = np.random.default_rng(4200 + seed)
+    batch = int(rng.choice([1, 2, 4, 8, 16]))
+    dtype = torch.float16 if rng.random() < 0.6 else torch.bfloat16
+    tiled = bool(rng.random() < 0.5) and batch <= 4
+    det = bool(rng.random() < 0.3) and batch <= 4
+    rl = DecodeRunList(batch, dtype, dev, deterministic=det)
+    to = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev).to(dtype)
+    f64 = lambda t: t.float().cpu().numpy().astype(np.float64)
+    refs, shapes, prev_m, prev_out = [], [], None, None
+    for i in range(int(rng.integers(1, 5))):
+        m = int(rng.choice([32, 96, 200, 512, 1376, 4096, 5000]))
+        r = int(rng.choice([32, 40, 96, 256, 736, 2048]))
+        chain = prev_m is not None and rng.random() < 0.3
+        n = prev_m if chain else int(rng.choice([64, 256, 1000, 4096, 11008, 16384]))
+        vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, 4300 + 10 * seed + i)
+        s_out = (s_out.astype(np.float32) * 30).astype(np.float16)     # keeps chained activations of order one
+        vt_p, u_p, mid_p = oracle.pad_rank(vt, u, s_mid, 32)
+        words = lambda w: packing.binary_packer(torch.from_numpy(w), "half2").to(dev)
+        vd, ud = words(vt_p), words(u_p)
+        if tiled:
+            vd, ud = packing.tile_words(vd), packing.tile_words(ud)
+        sc = (to(s_in), to(mid_p), to(s_out))
+        if chain:
+            xin = prev_out                                             # the previous output as the kernel hands it on
+            rl.add(rl.outputs[-1], sc[0], vd, sc[1], ud, sc[2], tiled=tiled, x_from=i - 1)
+        else:
+            xin = f64(to(oracle.synth_x(batch, n, 4400 + 10 * seed + i)))
+            rl.add(to(xin), sc[0], vd, sc[1], ud, sc[2], tiled=tiled)
+        ref = oracle.layer_forward(xin, vt, u, f64(sc[0]), f64(to(s_mid)), f64(sc[2]), dtype=np.float64)
+        refs.append(ref)
+        prev_m, prev_out = m, f64(torch.from_numpy(ref).to(dtype))
+        shapes.append((m, n, r, chain))
+    print(f"random list {seed}: batch {batch} {dtype} tiled={tiled} deterministic={det} {shapes}", flush=True)
+    ys = rl.run()
+    torch.cuda.synchronize()
+    assert rl.status() == 0
+    for y, ref in zip(ys, refs):
+        assert torch.isfinite(y.float()).all()
+        assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < (2e-2 if dtype == torch.bfloat16 else 1e-2)
