@@ -326,15 +326,16 @@ __device__ __forceinline__ void kwave_tile(const GemmArgs& a, int row_block, int
 #pragma unroll
         for (int v = 0; v < 16; ++v) part[((r * 4 + wave) * 16 + v) * kPartPitch + (lane & 31) + 33 * (lane >> 5)] = acc[r][v];
     __syncthreads();
-    // Thread (token t, row octet o) of the first 128 threads sums the four partial values of 8 consecutive
-    // rows and stores them as one 16-byte chunk.  Accumulator element v of lane l is token
-    // 8*(v>>2) + 4*(l>>5) + (v&3), row l&31.
-    if (threadIdx.x < 128) {
-        const int t = threadIdx.x >> 2, o = threadIdx.x & 3;
+    // Thread (token t, row octet o) of each half of the workgroup sums the four partial values of 8 consecutive
+    // rows and stores them as one 16-byte chunk; the two halves take the row tiles in turn (one half idles when
+    // there is only one).  Accumulator element v of lane l is token 8*(v>>2) + 4*(l>>5) + (v&3), row l&31.
+    {
+        const int th = threadIdx.x & 127, first_r = threadIdx.x >> 7;
+        const int t = th >> 2, o = th & 3;
         const int v = 4 * (t >> 3) + (t & 3), l0 = 33 * ((t >> 2) & 1) + 8 * o;   // lanes 32 h + 8 o + j of the tile row
         const int tok = tok0 + t;
 #pragma unroll
-        for (int r = 0; r < RT; ++r) {
+        for (int r = first_r; r < RT; r += 2) {
             if (r >= ntiles) break;
             const int row0 = (rt + r) * 32 + 8 * o;
             const float* pr = part + (size_t)r * 4 * 16 * kPartPitch;
@@ -378,8 +379,10 @@ struct GemmGroup {
 template <int DT, bool SCALED, int RT>
 __global__ __launch_bounds__(256) void gemm_kwave_group_kernel(GemmGroup g) {
     const int b = blockIdx.x;
+    // first[i] of the unused entries is the grid size, so no count is needed; all of first[] comes with one load
     int p = 0;
-    while (p + 1 < g.count && b >= g.first[p + 1]) ++p;
+#pragma unroll
+    for (int i = 1; i < kGroupMax; ++i) p += b >= g.first[i] ? 1 : 0;
     const GemmArgs a = g.a[p];
     const int local = b - g.first[p];
     const int gx = (a.R / 32 + RT - 1) / RT;
