@@ -661,12 +661,19 @@ __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* scl, float* 
         u32x4_t ra[kBurst], rb[kBurst];
 #pragma unroll
         for (int j = 0; j < kBurst; ++j) issue(it0 + j * THREADS, ra[j], rb[j]);
+        // A wavefront whose 64 chunks of a burst slot all lie past the end skips the slot's arithmetic (a short input
+        // keeps only the first wavefronts busy, and the second slot is empty for every input of up to 8 x THREADS
+        // columns per batch row): the branch is wave-uniform.
+        const int wave_first = __builtin_amdgcn_readfirstlane(it0 - lane);
         float tot[kBurst];
 #pragma unroll
         for (int j = 0; j < kBurst; ++j) {
-            float v[8];
-            values(it0 + j * THREADS, ra[j], rb[j], v);
-            tot[j] = quantize(it0 + j * THREADS, v);
+            tot[j] = 0.f;
+            if (wave_first + j * THREADS < total) {
+                float v[8];
+                values(it0 + j * THREADS, ra[j], rb[j], v);
+                tot[j] = quantize(it0 + j * THREADS, v);
+            }
         }
         // a wavefront's 64 chunks belong to one batch row (nchunks is a multiple of 64): one LDS atomic per
         // wavefront and burst slot
