@@ -175,8 +175,11 @@ __device__ __forceinline__ void stage_units_vector(uint4* xs, float* xsum, float
             if (st.in_f32) raw_b[j] = __builtin_amdgcn_raw_buffer_load_b128(rin, live ? off + 16u : kPastEnd, 0, kCacheDefault);
             else raw_b[j] = __builtin_amdgcn_raw_buffer_load_b128(rsc, live ? (uint32_t)col * 2u : kPastEnd, 0, kCacheDefault);
         }
+        // a wavefront whose 64 chunks of a burst slot all lie past the end skips the slot (wave-uniform branch)
+        const int wave_first = __builtin_amdgcn_readfirstlane(it0 - (int)(threadIdx.x & 63));
 #pragma unroll
         for (int j = 0; j < kBurst; ++j) {
+            if (wave_first + j * nthreads >= total) continue;
             const int it = it0 + j * nthreads;
             const int b = it / nchunks, q = it - b * nchunks;
             float v[8];
@@ -387,11 +390,11 @@ struct Mfma16<1> {
     }
 };
 
-// sign bits of `shifted` (bits 15 and 31) onto the pair (1.0, 1.0): one v_bfi_b32
+// sign bits of `shifted` (bits 15 and 31) onto the pair (1.0, 1.0): one v_and_or_b32.  Plain C, not inline assembly:
+// the result feeds an MFMA and may be written into a register that the previous MFMA still reads, and the compiler
+// keeps the wait states between such instructions only for instructions it knows.
 __device__ __forceinline__ uint32_t sign_onto_one(uint32_t shifted, uint32_t one_pair) {
-    uint32_t r;
-    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(r) : "s"(kSignPair), "v"(shifted), "v"(one_pair));
-    return r;
+    return (shifted & kSignPair) | one_pair;
 }
 
 // acc += signs(w: this lane's unit) x staged activations of unit `cu` (zero contribution when !valid).

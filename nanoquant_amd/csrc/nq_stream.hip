@@ -19,6 +19,8 @@
 //   * inside a workgroup the sign words go to the MFMA units as (16 rows x 4 units) items, one row and unit
 //     per lane; wavefronts take contiguous runs of items and finish per-row sums with LDS float atomics.
 // The arithmetic per 16-byte unit is in nq_decode.h.
+#include <type_traits>
+
 #include "nq_decode.h"
 #include "nq_kernels.h"
 
@@ -71,9 +73,12 @@ __device__ __forceinline__ BitsView bits_view(const RunStage& st) {
 
 // In tile order the 64 units of a wave-load (16 rows x 4 units) are 1 KiB contiguous and every line is read once:
 // streamed with the non-temporal hint (6.5 TB/s in a read-only probe against 5.9 row-major with default policy).
+// ORDER: 0 = as the view says (a branch, two load instructions), 1 = tile order, 2 = row-major: a loop that keeps several
+// fetches in flight wants exactly one load instruction per fetch, or the compiler waits for all of them at every use.
+template <int ORDER = 0>
 __device__ __forceinline__ uint4 load_unit(const BitsView& v, int row, int unit, bool live) {
     u32x4_t w;
-    if (v.groups) {
+    if (ORDER == 1 || (ORDER == 0 && v.groups)) {
         const uint32_t r = (uint32_t)row, u = (uint32_t)unit;
         const uint32_t idx = ((((r >> 5) * (uint32_t)v.groups + (u >> 2)) * 2u + ((r >> 4) & 1u)) * 4u + (u & 3u)) * 16u + (r & 15u);
         w = __builtin_amdgcn_raw_buffer_load_b128(v.rsrc, live ? idx * 16u : kPastEnd, 0, 2 /* nt */);
@@ -98,13 +103,108 @@ __device__ __forceinline__ void trim_unit(const BitsView& v, uint4& w, int unit)
 // Bytes of LDS in front of the staged input: row sums and two sets of input totals [2][16].  Reproducible sums (det):
 // a second set of row sums (what earlier input chunks of the row block added up to), two sets of per-wavefront input
 // totals [2][16][4] and two exponent words.
+// The 16-bit arithmetic keeps the row sums of whole rounds in registers and only those of the last, partial round of a
+// slice in LDS: kTailBytes for up to 128 / batch row pairs at a time, rows padded apart so that the lanes of one LDS
+// atomic fall into different banks (tail_index).
+constexpr int kTailBytes = 20 * 1024;
 __host__ __device__ constexpr size_t stream_head_bytes(int batch, int arith, bool det = false) {
-    (void)arith;
-    return (size_t)row_block(batch) * batch * sizeof(float) * (det ? 2 : 1) + (det ? 1024 : 128);
+    return (arith == 2 ? (size_t)row_block(batch) * batch * sizeof(float) * (det ? 2 : 1) : (size_t)kTailBytes) + (det ? 1024 : 128);
+}
+// Row sum (row, batch row b) of the tail: 16 floats of padding after every 4 rows at batch 16 (the four lane groups of
+// an MFMA result are 4 rows apart: 64 floats, the same bank), 8 after every 8 rows at batch 8.
+template <int BATCH>
+__device__ __forceinline__ int tail_index(int row, int b) {
+    static_assert(BATCH == 8 || BATCH == 16, "tail row sums are laid out for batch 8 and 16");
+    return row * BATCH + b + (BATCH == 16 ? 16 * (row >> 2) : 8 * (row >> 3));
 }
 
 // Items of the MFMA path that each wavefront of a workgroup takes (contiguous runs).
 __host__ __device__ __forceinline__ int mfma_items_per_wave(int nitems, int waves) { return (nitems + waves - 1) / waves; }
+
+// 16-bit MFMA arithmetic, the row groups of a slice that are left over after the whole rounds (see the kernel): `tn`
+// groups of 16 rows from row `row_base` of the matrix (`left` rows of them belong to the slice) times the unit groups of
+// the staged chunk (c0, cu_n).  Items = (16-row group, 4-unit group), unit group fastest, every wavefront a contiguous run of them;
+// the partial sums of a run go to the tail's row sums `racc` (LDS float atomics) when the row group changes and at the
+// end.  Three item fetches (1 KB each) in flight, in three register sets that take turns.  A function of its own, not
+// inlined: inside the kernel its loop shares the 128 registers of a 1024-lane workgroup with everything the slice keeps
+// alive and spills into the item loop.
+// ORDER: 1 = tile order, 2 = row-major (see load_unit).
+template <int DT, int BATCH, int THREADS, bool POW2, int ORDER>
+__device__ __attribute__((noinline)) void stream_tail_items(BitsView bv, const uint4* xs, float* racc, int upad, int st_rows,
+                                                           int row_base, int left, int tn, int c0, int cu_n) {
+    constexpr int kWaves = THREADS / kWave;
+    constexpr int kAccs = POW2 ? kPow2Classes : kMfmaAccs;
+    const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ngroups = (cu_n + 3) >> 2;
+    const int nitems = tn * ngroups;
+    const int per = mfma_items_per_wave(nitems, kWaves);
+    const int it_begin = min(wave * per, nitems), it_end = min(it_begin + per, nitems);
+    int f_it = it_begin, f_rg = it_begin / ngroups, f_ub = it_begin - (it_begin / ngroups) * ngroups;   // fetch cursor
+    int rg = f_rg, ub = f_ub, rg_run = f_rg;                                                           // compute cursor (row group = 16 rows)
+    auto fetch = [&](uint4& w) {
+        if constexpr (ORDER == 1) {
+            // 1 KB = one half of a 2 KB tile (row_base is a multiple of 16)
+            const bool ok = f_it < it_end;
+            const int half = (row_base >> 4) + f_rg;
+            const int tile = (half >> 1) * bv.groups + (c0 >> 2) + f_ub;
+            const uint32_t soff = ok ? (uint32_t)__builtin_amdgcn_readfirstlane(tile * 2048 + (half & 1) * 1024) : 0u;
+            const uint32_t voff = ok ? (uint32_t)lane * 16u : kPastEnd;
+            const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(bv.rsrc, voff, soff, 2 /* nt */);
+            w = make_uint4(a.x, a.y, a.z, a.w);
+        } else {
+            const int u = 4 * f_ub + g;
+            w = load_unit<ORDER>(bv, min(row_base + 16 * f_rg + r16, st_rows - 1), c0 + u, f_it < it_end && u < cu_n);
+        }
+        ++f_it;
+        if (++f_ub == ngroups) { f_ub = 0; ++f_rg; }
+    };
+    float4_t acc[kAccs];
+#pragma unroll
+    for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    auto flush = [&]() {
+        float4_t sum;
+        if constexpr (POW2) sum = pow2_combine(acc) * -2.f;              // signed sum = (sum of x) - 2 (sum of b x)
+        else sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+        if (r16 < BATCH) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int rel = 16 * rg_run + 4 * g + v;
+                if (rel < left) atomicAdd(&racc[tail_index<BATCH>(rel, r16)], sum[v]);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    };
+    auto work = [&](uint4& w) {
+        if (rg != rg_run) {
+            flush();
+            rg_run = rg;
+        }
+        const int u = 4 * ub + g;
+        if constexpr (ORDER == 2) trim_unit(bv, w, c0 + u);              // tile order pads with zero words
+        if constexpr (POW2) unit_mfma_pow2<BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
+        else unit_mfma<DT, BATCH>(w, xs, upad, u, u < cu_n, acc);
+        if (++ub == ngroups) { ub = 0; ++rg; }
+    };
+    // A full wait ahead of the first fetches: from here on they are the only loads in flight and the compiler waits for
+    // the oldest of them only, not for all.
+    __builtin_amdgcn_s_waitcnt(0);
+    uint4 w0, w1, w2;
+    fetch(w0);
+    fetch(w1);
+    fetch(w2);
+    int it = it_begin;
+#pragma unroll 1
+    for (; it + 3 <= it_end; it += 3) {
+        work(w0); fetch(w0);
+        work(w1); fetch(w1);
+        work(w2); fetch(w2);
+    }
+    if (it < it_end) work(w0);
+    if (it + 1 < it_end) work(w1);
+    if (it_begin < it_end) flush();
+}
 
 // ARITH: 1 = MFMA with 16-bit operands, 2 = MFMA with one-bit fp4 weights and fp8 pieces of the input (batch <= 4).
 // DET (fp4 x fp8 arithmetic only): row sums that do not depend on the order in which the wavefronts of a workgroup add
@@ -131,12 +231,13 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
     constexpr bool kTotals = kPow2Mfma || kQ8;                  // signed sum = (sum of x) - 2 (sum of b x)
     static_assert(!kQ8 || BATCH * kQ8Pieces <= 16, "pieces of all batch rows must fit the 16 operand columns");
     static_assert(!DET || kQ8, "reproducible sums exist for the fp4 x fp8 arithmetic only");
+    constexpr int kRaccFloats = kQ8 ? kRowBlock * BATCH : kTailBytes / (int)sizeof(float);   // 16-bit arithmetic: the tail's row sums
     float* racc = (float*)lds_raw;                              // [kRowBlock][BATCH] row sums
-    float* rtot = racc + kRowBlock * BATCH;                     // DET: the same, summed over the input chunks done so far
+    float* rtot = racc + kRaccFloats;                           // DET: the same, summed over the input chunks done so far
     // [2][16] sum of the staged input per batch row (DET: [2][16 wavefronts][4]); slices alternate between the two, so
     // that the one of the next slice is cleared a barrier ahead of its staging instead of costing a barrier of its own
     constexpr int kTotStride = DET ? 64 : 16;
-    float* xtot_base = racc + kRowBlock * BATCH * (DET ? 2 : 1);
+    float* xtot_base = racc + kRaccFloats * (DET ? 2 : 1);
     uint32_t* ebmax_base = (uint32_t*)(xtot_base + 2 * kTotStride);   // DET: [2] largest unit exponent of the staged input
     uint4* xs_base = lds_raw + stream_head_bytes(BATCH, ARITH, DET) / sizeof(uint4);
     __shared__ int s_flag;
@@ -258,10 +359,6 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
             sin.in = st.in; sin.s_col = st.s_col; sin.K = st.K; sin.in_stride = st.in_stride;
             sin.in_f32 = st.in_f32; sin.in_coherent = st.in_coherent; sin.vec_in = st.vec_in;
 
-            // First fetch of the slice, issued before any wait: the weights are always ready.  Not on the fp4 x fp8
-            // path: its staging needs the registers, and holding fetched words across it (measured with one, two and
-            // three items per wavefront) costs more in spills than the head start gains.
-            uint4 wnext = make_uint4(0, 0, 0, 0);
             // kQ8, row-major words: fetch cursor of this wavefront over its items = (pair of 16-row groups, 4-unit group)
             // of the current (row block, input chunk), unit group fastest
             int q_ngroups = 1, q_it_begin = 0, q_it_end = 0, q_it_f = 0, q_rp_f = 0, q_ub_f = 0, q_rb = 0, q_c0 = 0, q_cu_n = 0, q_nr = 0;
@@ -333,15 +430,6 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                     q_setup(seg.row_begin, 0);
                     q_fetch(wa0, wb0); q_fetch(wa1, wb1); q_fetch(wa2, wb2);
                 }
-            } else {
-                // wavefront w starts with item w of the first row block: 16 rows x 4 units, lane (row l & 15,
-                // unit l >> 4)
-                const int ng0 = (chunk_units + 3) >> 2;
-                const int nr0 = min(seg.row_end - seg.row_begin, kRowBlock);
-                const int item0 = __builtin_amdgcn_readfirstlane(tid >> 6) * mfma_items_per_wave(((nr0 + 15) >> 4) * ng0, kWaves);
-                const int u0 = 4 * (item0 % ng0) + ((tid & 63) >> 4);
-                wnext = load_unit(bv, min(seg.row_begin + 16 * (item0 / ng0) + (tid & 15), st.rows - 1), u0,
-                                  item0 < ((nr0 + 15) >> 4) * ng0 && u0 < chunk_units);
             }
 
             if ((st.dep >= 0 || st.dep2 >= 0) && !aborted) {
@@ -386,7 +474,241 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
             if (tid < kTotStride) xtot_other[tid] = 0.f;         // every reader of it (the previous slice) is past the barrier
             if (DET && tid == 0) ebmax_base[slice_count & 1] = 0u;   // slice_count was advanced: this is the other one
 
-            if (!aborted) {
+            if constexpr (!kQ8) {
+              if (!aborted) {
+                // ---- 16-bit MFMA arithmetic (batch 8 and 16): wavefronts own whole row groups ----
+                // A group = 16 consecutive rows of the slice (the rows of one MFMA).  In a round, wavefront w takes group
+                // 16 * round + w and walks ALL columns of it, so a row sum lives in its MFMA accumulators from the first
+                // column to the last and goes from there straight to the output: no row sums in LDS, no LDS atomics (at
+                // batch 16 they cost more than the arithmetic), no barrier between rows.  With an input of one chunk the
+                // wavefronts of a workgroup meet once per slice (after the staging) and the item fetches of a wavefront
+                // run on from group to group; with a longer input the chunks are staged again for every round and the
+                // accumulators are kept across the chunks of a round.  The groups left over after the whole rounds
+                // (fewer than 16: a wavefront needs tens of microseconds for a group, so leaving wavefronts idle there
+                // costs a tenth of a long slice and most of a short one) are shared out item by item instead, every
+                // wavefront a contiguous run, and summed in LDS (stream_tail_items; kTailBytes hold 256 rows at batch 16).
+                const int lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+                const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // scalar item arithmetic
+                constexpr int kAccs = kPow2Mfma ? kPow2Classes : kMfmaAccs;
+                const int ngroups16 = (seg.row_end - seg.row_begin + 15) >> 4;
+                const int full_rounds = ngroups16 / kWaves;                       // the same for every wavefront
+                const int tail_groups = ngroups16 - full_rounds * kWaves;
+                const int tail_base = seg.row_begin + 16 * full_rounds * kWaves;  // first row of the tail
+                float4_t acc[kAccs];
+#pragma unroll
+                for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
+                // rows row0 .. row0 + 3 of batch row b: row scale, bias, addend, store (as the epilogue of the row-block
+                // loop).  The four rows of a lane are consecutive: 8-byte accesses where the alignment allows them.
+                const bool vec_rows = (seg.row_begin & 3) == 0 && (st.out_stride & 3) == 0 &&
+                                      ((((uintptr_t)st.s_row) | ((uintptr_t)st.bias) | ((uintptr_t)st.out)) & 7u) == 0;
+                auto emit4 = [&](int row0, int b, float4_t v4) __attribute__((always_inline)) {
+                    float v[4] = {v4[0], v4[1], v4[2], v4[3]};   // scalars: a device-scope atomic store of a vector element stored element 0 four times
+                    const size_t o = (size_t)b * st.out_stride + row0;
+                    if (vec_rows && row0 + 3 < seg.row_end) {
+                        if (st.s_row) {
+                            const uint2 sw = *(const uint2*)(st.s_row + row0);
+                            v[0] *= E::to_float((uint16_t)(sw.x & 0xFFFFu)); v[1] *= E::to_float((uint16_t)(sw.x >> 16));
+                            v[2] *= E::to_float((uint16_t)(sw.y & 0xFFFFu)); v[3] *= E::to_float((uint16_t)(sw.y >> 16));
+                        }
+                        if (st.bias) {
+                            const uint2 bw = *(const uint2*)(st.bias + row0);
+                            v[0] += E::to_float((uint16_t)(bw.x & 0xFFFFu)); v[1] += E::to_float((uint16_t)(bw.x >> 16));
+                            v[2] += E::to_float((uint16_t)(bw.y & 0xFFFFu)); v[3] += E::to_float((uint16_t)(bw.y >> 16));
+                        }
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            if (row0 + k >= seg.row_end) break;
+                            if (st.s_row) v[k] *= E::to_float(st.s_row[row0 + k]);
+                            if (st.bias) v[k] += E::to_float(st.bias[row0 + k]);
+                        }
+                    }
+                    if (st.addend) {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            if (row0 + k >= seg.row_end) break;
+                            if (st.dep2 >= 0)
+                                v[k] += __builtin_bit_cast(float, __hip_atomic_load((const uint32_t*)st.addend + o + k, __ATOMIC_RELAXED,
+                                                                                    __HIP_MEMORY_SCOPE_AGENT));
+                            else
+                                v[k] += st.addend[o + k];
+                        }
+                    }
+                    if (!st.out_f32 && vec_rows && row0 + 3 < seg.row_end) {
+                        uint2 pk;
+                        pk.x = (uint32_t)E::from_float_clamped(v[0]) | ((uint32_t)E::from_float_clamped(v[1]) << 16);
+                        pk.y = (uint32_t)E::from_float_clamped(v[2]) | ((uint32_t)E::from_float_clamped(v[3]) << 16);
+                        *(uint2*)((uint16_t*)st.out + o) = pk;
+                        return;
+                    }
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        if (row0 + k >= seg.row_end) break;
+                        if (st.out_f32) {
+                            // fp32 results (h, partial sums over terms) may be read by other workgroups of this launch:
+                            // device-coherent store, completed before the counter of the slice is bumped
+                            if (st.signal) __hip_atomic_store((uint32_t*)st.out + o + k, __builtin_bit_cast(uint32_t, v[k]),
+                                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            else ((float*)st.out)[o + k] = v[k];
+                        } else {
+                            ((uint16_t*)st.out)[o + k] = E::from_float_clamped(v[k]);
+                        }
+                    }
+                };
+                // the q-th group of this wavefront is complete: acc[v] = sum for its row 4 g + v, batch row r16
+                auto store_group = [&](int q) __attribute__((always_inline)) {
+                    float4_t sum;
+                    if constexpr (kPow2Mfma) sum = pow2_combine(acc) * -2.f;      // signed sum = (sum of x) - 2 (sum of b x)
+                    else sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+                    if (r16 < BATCH) {
+                        const float xt = kPow2Mfma ? xtot[r16] : 0.f;
+                        const int row0 = seg.row_begin + 16 * (wave + kWaves * q) + 4 * g;
+                        if (row0 < seg.row_end) emit4(row0, r16, sum + xt);
+                    }
+                };
+                // one row of one batch row (the tail's epilogue; same order of operations as emit4)
+                auto emit1 = [&](int row, int b, float v) __attribute__((always_inline)) {
+                    if (st.s_row) v *= E::to_float(st.s_row[row]);
+                    if (st.bias) v += E::to_float(st.bias[row]);
+                    const size_t o = (size_t)b * st.out_stride + row;
+                    if (st.addend) {
+                        if (st.dep2 >= 0)
+                            v += __builtin_bit_cast(float, __hip_atomic_load((const uint32_t*)st.addend + o, __ATOMIC_RELAXED,
+                                                                             __HIP_MEMORY_SCOPE_AGENT));
+                        else
+                            v += st.addend[o];
+                    }
+                    if (st.out_f32) {
+                        if (st.signal) __hip_atomic_store((uint32_t*)st.out + o, __builtin_bit_cast(uint32_t, v),
+                                                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        else ((float*)st.out)[o] = v;
+                    } else {
+                        ((uint16_t*)st.out)[o] = E::from_float_clamped(v);
+                    }
+                };
+                // The groups [q_begin, q_end) of this wavefront times the unit groups of the staged chunk (c0, cu_n).
+                // Items = (row group, 4-unit group), unit group fastest.  Three item fetches (1 KB of packed words each) in
+                // flight, in three register sets that take turns, each refilled right after its use; a row group is
+                // walked in a multiple of three positions (the last ones may be empty), so the register sets keep their
+                // turns from group to group and the fetches run on into the next group while the current one is finished
+                // and stored.  A fetch past the last item loads nothing (offset past the end).  `complete`: the staged
+                // chunk is the last of the input.
+                auto run_items = [&](auto order_c, int q_begin, int q_end, int c0, int cu_n, bool complete) __attribute__((always_inline)) {
+                    constexpr int kOrder = decltype(order_c)::value;      // one copy of the loop per word order: see load_unit
+                    const int ngroups = (cu_n + 3) >> 2;
+                    const int positions = (ngroups + 2) / 3 * 3;
+                    const int nq = max(min(q_end, full_rounds) - q_begin, 0);
+                    int f_left = nq * positions, f_q = q_begin, f_j = 0;  // fetch cursor
+                    auto fetch = [&](uint4& w) {
+                        if constexpr (kOrder == 1) {
+                            // tile order: the item is one half (1 KB) of a 2 KB tile (slices begin at multiples of 16
+                            // rows, chunks at multiples of 4 units), 16 bytes per lane; rows and units past the end are
+                            // zero words
+                            const bool ok = f_left > 0 && f_j < ngroups;
+                            const int half = (seg.row_begin >> 4) + wave + kWaves * f_q;
+                            const int off = ((half >> 1) * bv.groups + (c0 >> 2) + f_j) * 2048 + (half & 1) * 1024;
+                            const uint32_t soff = ok ? (uint32_t)__builtin_amdgcn_readfirstlane(off) : 0u;
+                            const uint32_t voff = ok ? (uint32_t)lane * 16u : kPastEnd;
+                            const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(bv.rsrc, voff, soff, 2 /* nt */);
+                            w = make_uint4(a.x, a.y, a.z, a.w);
+                        } else {
+                            const int u = 4 * f_j + g;
+                            const int row = seg.row_begin + 16 * (wave + kWaves * f_q) + r16;
+                            w = load_unit<kOrder>(bv, min(row, st.rows - 1), c0 + u, f_left > 0 && u < cu_n);   // u < cu_n fails on empty positions as well
+                        }
+                        --f_left;
+                        if (++f_j == positions) { f_j = 0; ++f_q; }
+                    };
+                    auto work = [&](uint4& w, int j) {
+                        const int u = 4 * j + g;
+                        if constexpr (kOrder == 2) trim_unit(bv, w, c0 + u);   // tile order pads with zero words
+                        if constexpr (kPow2Mfma) unit_mfma_pow2<BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
+                        else unit_mfma<DT, BATCH>(w, xs, upad, u, u < cu_n, acc);
+                    };
+                    // A full wait ahead of the first fetches (what the staging loaded has been used) and after the stores
+                    // of a group: inside the loop the item fetches are the only accesses in flight and the compiler waits
+                    // for the oldest of them only, not for all.
+                    __builtin_amdgcn_s_waitcnt(0);
+                    uint4 w0, w1, w2;
+                    fetch(w0);
+                    fetch(w1);
+                    fetch(w2);
+#pragma unroll 1
+                    for (int q = q_begin; q < q_begin + nq; ++q) {
+#pragma unroll 1
+                        for (int j = 0; j < positions; j += 3) {
+                            work(w0, j);
+                            fetch(w0);
+                            if (j + 1 < ngroups) work(w1, j + 1);
+                            fetch(w1);
+                            if (j + 2 < ngroups) work(w2, j + 2);
+                            fetch(w2);
+                        }
+                        if (complete) {
+                            store_group(q);
+#pragma unroll
+                            for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
+                            __builtin_amdgcn_s_waitcnt(0);
+                        }
+                    }
+                };
+                // the tail's row sums are complete (a barrier has passed): all lanes share out its rows
+                auto tail_store = [&]() __attribute__((always_inline)) {
+                    const int rows = seg.row_end - tail_base;
+                    for (int i = tid; i < rows * BATCH; i += kStreamThreads) {
+                        const int rel = i / BATCH, b = i % BATCH;
+                        emit1(tail_base + rel, b, racc[tail_index<BATCH>(rel, b)] + (kPow2Mfma ? xtot[b] : 0.f));
+                    }
+                };
+                auto zero_tail = [&]() {
+                    for (int i = tid; i < kTailBytes / (int)sizeof(float); i += kStreamThreads) racc[i] = 0.f;
+                };
+                bool staged = false;                                      // a chunk is staged and may be in use
+                auto stage_chunk = [&](int c0, int cu_n, bool clear_tail) __attribute__((always_inline)) {
+                    if (staged) {
+                        lds_barrier();                                    // every wavefront is done with the staged chunk, the totals and the tail's sums
+                        if (kPow2Mfma && c0 == 0) {
+                            if (tid < kTotStride) xtot[tid] = 0.f;        // staged again from the first column: the totals start over
+                            lds_barrier();
+                        }
+                    }
+                    if (clear_tail) zero_tail();
+                    stage_units<DT, BATCH, kPow2Mfma>(xs, nullptr, sin, c0, cu_n, upad, kStreamThreads, kPow2Mfma ? xtot : nullptr);
+                    staged = true;
+                    lds_barrier();                                        // staged input, its totals and the cleared sums visible
+                };
+                auto owned = [&](int q_begin, int q_end, int c0, int cu_n, bool complete) __attribute__((always_inline)) {
+                    if (bv.groups) run_items(std::integral_constant<int, 1>{}, q_begin, q_end, c0, cu_n, complete);
+                    else run_items(std::integral_constant<int, 2>{}, q_begin, q_end, c0, cu_n, complete);
+                };
+                auto shared = [&](int c0, int cu_n) __attribute__((always_inline)) {
+                    if (bv.groups) stream_tail_items<DT, BATCH, THREADS, kPow2Mfma, 1>(bv, xs, racc, upad, st.rows, tail_base, seg.row_end - tail_base, tail_groups, c0, cu_n);
+                    else stream_tail_items<DT, BATCH, THREADS, kPow2Mfma, 2>(bv, xs, racc, upad, st.rows, tail_base, seg.row_end - tail_base, tail_groups, c0, cu_n);
+                };
+                // whole rounds: an input of one chunk is staged once and every wavefront walks all its groups in one go
+                const int staged_rounds = one_chunk ? min(full_rounds, 1) : full_rounds;
+#pragma unroll 1
+                for (int r = 0; r < staged_rounds; ++r) {
+#pragma unroll 1
+                    for (int c0 = 0; c0 < st.units; c0 += chunk_units) {
+                        const int cu_n = min(chunk_units, st.units - c0);
+                        stage_chunk(c0, cu_n, one_chunk && tail_groups > 0);
+                        owned(one_chunk ? 0 : r, one_chunk ? full_rounds : r + 1, c0, cu_n, c0 + chunk_units >= st.units);
+                    }
+                }
+                // the groups left over (fewer than 16: their row sums fit kTailBytes)
+                if (tail_groups > 0) {
+#pragma unroll 1
+                    for (int c0 = 0; c0 < st.units; c0 += chunk_units) {
+                        const int cu_n = min(chunk_units, st.units - c0);
+                        if (!one_chunk || !staged) stage_chunk(c0, cu_n, c0 == 0);
+                        shared(c0, cu_n);
+                    }
+                    lds_barrier();                                        // the tail's row sums are complete
+                    tail_store();
+                }
+              }
+            } else if (!aborted) {
                 bool staged = false;
 #pragma unroll 1
                 for (int rb = seg.row_begin; rb < seg.row_end; rb += kRowBlock) {
@@ -409,8 +731,6 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                                 lds_barrier();
                             }
                             if constexpr (kQ8) stage_units_q8<DT, BATCH, THREADS, DET>(xs, scl, xtot, sin, c0, cu_n, upad, ebmax);
-                            else stage_units<DT, BATCH, kPow2Mfma>(xs, nullptr, sin, c0, cu_n, upad, kStreamThreads,
-                                                                   kPow2Mfma ? xtot : nullptr);
                             staged = true;
                         }
                         lds_barrier();                           // xs / xsum / zeroed racc visible
@@ -530,54 +850,6 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                                     }
                                 }
                             }
-                        } else {
-                            // Items = (16-row group, 4-unit group), unit group fastest; every wavefront takes a
-                            // contiguous run of items, so it mostly stays on one row group and adds its
-                            // accumulator to the row sums only when the row group changes.
-                            const int lane = tid & 63, r16 = lane & 15, g = lane >> 4;
-                            const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar item arithmetic
-                            const int ngroups = (cu_n + 3) >> 2;
-                            const int nitems = ((nr + 15) >> 4) * ngroups;
-                            const int per = mfma_items_per_wave(nitems, kWaves);
-                            const int it_begin = wave * per, it_end = min(it_begin + per, nitems);
-                            constexpr int kAccs = kPow2Mfma ? kPow2Classes : kMfmaAccs;
-                            // (row group, unit group) of the current and of the next item, advanced without divisions
-                            int rg = 16 * (it_begin / ngroups), ub = it_begin % ngroups;
-                            int rg_n = rg, ub_n = ub + 1;
-                            if (ub_n == ngroups) { ub_n = 0; rg_n += 16; }
-                            uint4 w = wnext;                             // very first fetch of the slice
-                            if ((rb != seg.row_begin || c0 != 0) && it_begin < it_end)
-                                w = load_unit(bv, min(rb + rg + r16, st.rows - 1), c0 + 4 * ub + g, 4 * ub + g < cu_n);
-#pragma unroll 1
-                            for (int it = it_begin; it < it_end;) {
-                                // one run = the items of this wavefront that share a row group
-                                const int run = min(ngroups - ub, it_end - it);
-                                const int rg_run = rg;
-                                float4_t acc[kAccs];
-#pragma unroll
-                                for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
-#pragma unroll 1
-                                for (int k = 0; k < run; ++k, ++it) {
-                                    const int u = 4 * ub + g, un = 4 * ub_n + g;
-                                    const uint4 wpre = load_unit(bv, min(rb + rg_n + r16, st.rows - 1), c0 + un,
-                                                                 it + 1 < it_end && un < cu_n);
-                                    trim_unit(bv, w, c0 + u);
-                                    if constexpr (kPow2Mfma) unit_mfma_pow2<BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
-                                    else unit_mfma<DT, BATCH>(w, xs, upad, u, u < cu_n, acc);
-                                    w = wpre;
-                                    rg = rg_n; ub = ub_n;
-                                    if (++ub_n == ngroups) { ub_n = 0; rg_n += 16; }
-                                }
-                                // sum[v] = partial sum of row rg_run + 4*g + v for batch row r16
-                                float4_t sum;
-                                if constexpr (kPow2Mfma) sum = pow2_combine(acc) * -2.f;   // + sum of x at the end
-                                else sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
-                                if (r16 < BATCH) {
-#pragma unroll
-                                    for (int v = 0; v < 4; ++v)
-                                        if (rg_run + 4 * g + v < nr) atomicAdd(&racc[(rg_run + 4 * g + v) * BATCH + r16], sum[v]);
-                                }
-                            }
                         }
                         }
                     lds_barrier();                               // row sums complete
@@ -659,7 +931,7 @@ static void stream_lds_plan(int batch, int arith, int max_units, int* chunk_cap_
         return;
     }
     int chunk_cap = (kStreamLdsMax - racc_bytes - batch * (int)sizeof(uint4)) / (batch * 16 * (int)sizeof(uint4));
-    chunk_cap = (chunk_cap - 1) & ~1;
+    chunk_cap = (chunk_cap - 1) & ~3;   // whole 4-unit groups, and room for the odd pitch chunk_units | 1
     const int chunk_units = max_units < chunk_cap ? max_units : chunk_cap;
     *chunk_cap_out = chunk_cap;
     *lds_out = (size_t)racc_bytes + (size_t)xs_chunks(batch, chunk_units | 1) * sizeof(uint4);
@@ -843,7 +1115,7 @@ bool stream_needs_uniform_order(int dtype, int batch) {
 
 // Rows that one wave-load spans: slices of tile-order stages are cut at multiples of it.
 int stream_row_granule(int dtype, int batch) {
-#define NQ_GRAN(D, B) (StreamKernel<D, B>::kArith == 2 ? 32 : 16)
+#define NQ_GRAN(D, B) 32
     NQ_STREAM_DISPATCH(NQ_GRAN)
 #undef NQ_GRAN
     return 32;
