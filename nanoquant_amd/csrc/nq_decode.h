@@ -96,8 +96,30 @@ __device__ __forceinline__ void store_chunk(uint4* xs, int b, int i, int upad, i
     }
 }
 
+// The same with the 8 values as 4 packed pairs.
+template <bool PM>
+__device__ __forceinline__ void store_chunk_packed(uint4* xs, int b, int i, int upad, int cu, const uint32_t (&rp)[4]) {
+    if constexpr (PM) {
+        uint32_t* xd = (uint32_t*)xs;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) xd[xs_dword<true>(b, 4 * i + k, upad, cu)] = rp[k];
+    } else {
+        xs[xs_chunk(b, i, upad, cu)] = make_uint4(rp[0], rp[1], rp[2], rp[3]);
+    }
+}
+
 // Staging variants below: `xsum` (may be null) receives the per-unit sums, `xtot` (may be null) the sum over all staged units per batch row
 // (LDS float atomics; the caller zeroes it and puts a barrier before and after).
+
+// it / n for 0 <= it < 2^23 with rcp = 1.f / n: the float product is off by one at most (the compiler's exact 32-bit
+// division costs some 25 lane instructions, as much as the rest of a staged chunk).
+__device__ __forceinline__ int small_div(int it, int n, float rcp) {
+    int q = (int)((float)it * rcp);
+    const int r = it - q * n;
+    if (r >= n) ++q;
+    else if (r < 0) --q;
+    return q;
+}
 
 // Coherent fp32 input (the intermediate h written by other workgroups of this launch): 16-byte
 // device-coherent loads, kBurst per lane in flight before the first is consumed (a round trip to the
@@ -113,13 +135,16 @@ __device__ __forceinline__ void stage_units_coherent(uint4* xs, float* xsum, flo
     const int total = BATCH * nquads;
     const __amdgpu_buffer_rsrc_t rsrc =
         raw_buffer(st.in, (uint32_t)(((size_t)(BATCH - 1) * st.in_stride + st.K) * sizeof(float)));
+    const float rcp = 1.f / (float)nquads;
 #pragma unroll 1
     for (int it0 = threadIdx.x; it0 < total; it0 += nthreads * kBurst) {   // wave-uniform trip count: it0 - lane
         u32x4_t raw[kBurst];
+        int bq[kBurst];
 #pragma unroll
         for (int j = 0; j < kBurst; ++j) {
             const int it = it0 + j * nthreads;
-            const int b = it / nquads, q = it - b * nquads;
+            const int b = small_div(it, nquads, rcp), q = it - b * nquads;
+            bq[j] = b;
             const int col = c0 * 128 + 4 * q;
             const uint32_t off = (it < total && col < st.K) ? (uint32_t)(((size_t)b * st.in_stride + col) * sizeof(float)) : kPastEnd;
             raw[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, kCacheAgentCoherent);
@@ -127,7 +152,7 @@ __device__ __forceinline__ void stage_units_coherent(uint4* xs, float* xsum, flo
 #pragma unroll
         for (int j = 0; j < kBurst; ++j) {
             const int it = it0 + j * nthreads;
-            const int b = it / nquads, q = it - b * nquads;
+            const int b = bq[j], q = it - b * nquads;
             const uint16_t r0 = E::from_float(as_float(raw[j].x));
             const uint16_t r1 = E::from_float(as_float(raw[j].y));
             const uint16_t r2 = E::from_float(as_float(raw[j].z));
@@ -161,13 +186,16 @@ __device__ __forceinline__ void stage_units_vector(uint4* xs, float* xsum, float
     const __amdgpu_buffer_rsrc_t rin = raw_buffer(st.in, (uint32_t)(((size_t)(BATCH - 1) * st.in_stride + st.K) * esize));
     const bool scaled = !st.in_f32 && st.s_col != nullptr;
     const __amdgpu_buffer_rsrc_t rsc = raw_buffer(scaled ? (const void*)st.s_col : st.in, scaled ? (uint32_t)st.K * 2u : 0u);
+    const float rcp = 1.f / (float)nchunks;
 #pragma unroll 1
     for (int it0 = threadIdx.x; it0 < total; it0 += nthreads * kBurst) {
         u32x4_t raw_a[kBurst], raw_b[kBurst];
+        int bq[kBurst];
 #pragma unroll
         for (int j = 0; j < kBurst; ++j) {
             const int it = it0 + j * nthreads;
-            const int b = it / nchunks, q = it - b * nchunks;
+            const int b = small_div(it, nchunks, rcp), q = it - b * nchunks;
+            bq[j] = b;
             const int col = c0 * 128 + 8 * q;
             const bool live = it < total && col < st.K;
             const uint32_t off = live ? (uint32_t)(((size_t)b * st.in_stride + col) * esize) : kPastEnd;
@@ -181,7 +209,34 @@ __device__ __forceinline__ void stage_units_vector(uint4* xs, float* xsum, float
         for (int j = 0; j < kBurst; ++j) {
             if (wave_first + j * nthreads >= total) continue;
             const int it = it0 + j * nthreads;
-            const int b = it / nchunks, q = it - b * nchunks;
+            const int b = bq[j], q = it - b * nchunks;
+            if constexpr (DT == 0) {
+                if (!st.in_f32) {
+                    // fp16 input: packed products, rounded once to fp16 like the fp32 product below (the product of two
+                    // fp16 numbers is exact in fp32), and their sum with the packed dot product: 8 lane operations per
+                    // chunk instead of 50
+                    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+                    uint32_t rp[4];
+                    float tot = 0.f;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        half2_t xv = __builtin_bit_cast(half2_t, (uint32_t)raw_a[j][e]);
+                        if (scaled) xv = xv * __builtin_bit_cast(half2_t, (uint32_t)raw_b[j][e]);
+                        rp[e] = __builtin_bit_cast(uint32_t, xv);
+                        tot = __builtin_amdgcn_fdot2(xv, (half2_t){(_Float16)1.f, (_Float16)1.f}, tot, false);
+                    }
+                    tot = group_sum(tot, 16);
+                    if (it < total) {
+                        const int cu = q >> 4, i = q & 15;
+                        store_chunk_packed<PM>(xs, b, i, upad, cu, rp);
+                        if (i == 0) {
+                            if (xsum) xsum[b * upad + cu] = tot;
+                            if (xtot) atomicAdd(&xtot[b], tot);
+                        }
+                    }
+                    continue;
+                }
+            }
             float v[8];
             if (!st.in_f32) {
 #pragma unroll
