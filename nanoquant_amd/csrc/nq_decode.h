@@ -613,9 +613,11 @@ __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* scl, float* 
     const bool scaled = !st.in_f32 && st.s_col != nullptr;
     const __amdgpu_buffer_rsrc_t rsc = raw_buffer(scaled ? (const void*)st.s_col : st.in, scaled ? (uint32_t)st.K * 2u : 0u);
     const bool coherent = st.in_f32 && st.in_coherent;
+    const float rcp = 1.f / (float)nchunks;
+    auto batch_row = [&](int it) -> int { return BATCH == 1 ? 0 : small_div(it, nchunks, rcp); };
 
     auto issue = [&](int it, u32x4_t& ra, u32x4_t& rb) {
-        const int b = it / nchunks, q = it - b * nchunks;
+        const int b = batch_row(it), q = it - b * nchunks;
         const int col = c0 * 128 + 8 * q;
         const bool live = fast && it < total && col < st.K;
         const uint32_t off = live ? (uint32_t)(((size_t)b * st.in_stride + col) * esize) : kPastEnd;
@@ -647,7 +649,7 @@ __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* scl, float* 
             }
         } else {
             // element-wise fallback: odd K or rows that allow no 16-byte loads
-            const int b = it / nchunks, q = it - b * nchunks;
+            const int b = batch_row(it), q = it - b * nchunks;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const int c = c0 * 128 + 8 * q + e;
@@ -669,7 +671,7 @@ __device__ __forceinline__ void stage_units_q8(uint4* xq, uint32_t* scl, float* 
     };
     // chunk (b, q): unit scale, pieces into LDS, and the chunk's share of xtot
     auto quantize = [&](int it, float (&v)[8]) -> float {
-        const int b = it / nchunks, q = it - b * nchunks;
+        const int b = batch_row(it), q = it - b * nchunks;
         const int cu = q >> 4, t = (q >> 2) & 3, qq = q & 3;
         float m = 0.f;
 #pragma unroll
