@@ -247,6 +247,43 @@ def test_tiled_factors_give_the_same_layer(dev, batch, dtype):
                               atol=2e-4 * float(yr.float().abs().max()))
 
 
+@pytest.mark.parametrize("tiled", [False, True])
+@pytest.mark.parametrize("batch,dtype", [(16, torch.float16), (8, torch.float16), (16, torch.bfloat16)])
+def test_long_lists_on_the_16_bit_operands(dev, batch, dtype, tiled):
+    # Batch 8 and 16: a wavefront owns whole 16-row groups of a slice and keeps their row sums in registers, only the
+    # groups left over after the rounds of 16 are summed in LDS.  Short lists give every workgroup a few rows (all
+    # left-overs); here 64 linears with 2000 x 8192 first factors put about 500 rows of one stage on a workgroup (a
+    # whole round, a second one with rows missing, 15 groups left over in some) and make the input two chunks at batch 16.
+    m, n, r, count = 520, 8192, 2000, 64
+    checked = {0: 900, 31: 901, 63: 902}
+    to = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev).to(dtype)
+    f64 = lambda t: t.float().cpu().numpy().astype(np.float64)
+    words = (lambda w: packing.tile_words(w)) if tiled else (lambda w: w)
+    terms = {}
+    for seed in set(checked.values()) | {903}:
+        vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, seed)
+        dev_ops = (to(s_in), words(packing.binary_packer(torch.from_numpy(vt), "half2").to(dev)), to(s_mid),
+                   words(packing.binary_packer(torch.from_numpy(u), "half2").to(dev)), to(s_out))
+        terms[seed] = ((vt, u), dev_ops)
+    rl = DecodeRunList(batch, dtype, dev)
+    refs = {}
+    for i in range(count):
+        seed = checked.get(i, 903)
+        (vt, u), ops = terms[seed]
+        x = to(oracle.synth_x(batch, n, 950 + i))
+        rl.add(x, *ops, tiled=tiled)
+        if i in checked:
+            refs[i] = oracle.layer_forward(f64(x), vt, u, f64(ops[0]), f64(ops[2]), f64(ops[4]), dtype=np.float64)
+    print(f"long run list batch={batch} {dtype} tiled={tiled}", flush=True)
+    for rep in range(2):
+        ys = rl.run()
+        torch.cuda.synchronize()
+        assert rl.status() == 0
+        for i, ref in refs.items():
+            err = oracle.max_rel_err(ys[i].float().cpu().numpy(), ref)
+            assert err < (1e-2 if dtype == torch.bfloat16 else 2e-3), (i, rep, err)
+
+
 def test_tiled_factor_size_is_checked(dev):
     m, n, r = 64, 128, 32
     _, ops = _term(dev, m, n, r, seed=5)
