@@ -26,11 +26,10 @@
 
 namespace nq {
 
-// Rows whose sums a workgroup keeps in LDS at a time (then: barrier, scale, store, barrier): every block of a slice
-// ends with all wavefronts waiting for the slowest one, so few large blocks -- 1024 rows up to batch 4 (16 KiB of row
-// sums at batch 4; 256-row blocks cost the batch-4 stack 8.6 instead of 6.2 us per layer).  The 16-bit arithmetic
-// at batch 16 needs its LDS for the staged rows: 256 rows there (= 16 row groups, one per wavefront; 320, 384 and 512
-// measured no better), 1024 at batch 8 (stack 14.5 -> 13.9 us per layer against 512).
+// fp4 x fp8 arithmetic: rows whose sums a workgroup keeps in LDS at a time (then: barrier, scale, store, barrier).
+// Every block of a slice ends with all wavefronts waiting for the slowest one, so few large blocks: 1024 rows (16 KiB
+// of row sums at batch 4; 256-row blocks cost the batch-4 stack 8.6 instead of 6.2 us per layer).  The 16-bit
+// arithmetic (batch 8 and 16) keeps its row sums in registers and has no row blocks.
 __host__ __device__ constexpr int row_block(int batch) { return batch <= 8 ? 1024 : 256; }
 // Same-address device-scope atomics serialise at the memory side (tens of ns each), so completion
 // counts are spread over kSubCounters addresses per stage and kExitSubs addresses for the exit count,
@@ -114,8 +113,8 @@ __host__ __device__ constexpr size_t stream_head_bytes(int batch, int arith, boo
 // an MFMA result are 4 rows apart: 64 floats, the same bank), 8 after every 8 rows at batch 8.
 template <int BATCH>
 __device__ __forceinline__ int tail_index(int row, int b) {
-    static_assert(BATCH == 8 || BATCH == 16, "tail row sums are laid out for batch 8 and 16");
-    return row * BATCH + b + (BATCH == 16 ? 16 * (row >> 2) : 8 * (row >> 3));
+    static_assert(BATCH <= 16, "kTailBytes hold 256 rows of up to 16 batch rows with their padding");
+    return row * BATCH + b + (BATCH == 16 ? 16 * (row >> 2) : BATCH == 8 ? 8 * (row >> 3) : 0);
 }
 
 // Items of the MFMA path that each wavefront of a workgroup takes (contiguous runs).
