@@ -445,80 +445,54 @@ struct Mfma16<1> {
     }
 };
 
-// sign bits of `shifted` (bits 15 and 31) onto the pair (1.0, 1.0): one v_and_or_b32.  Plain C, not inline assembly:
-// the result feeds an MFMA and may be written into a register that the previous MFMA still reads, and the compiler
-// keeps the wait states between such instructions only for instructions it knows.
-__device__ __forceinline__ uint32_t sign_onto_one(uint32_t shifted, uint32_t one_pair) {
-    return (shifted & kSignPair) | one_pair;
-}
-
-// acc += signs(w: this lane's unit) x staged activations of unit `cu` (zero contribution when !valid).
-// xs row used by this lane: batch row min(lane & 15, BATCH-1); columns beyond BATCH are never read back.
-// Four accumulators in rotation: consecutive MFMAs do not depend on each other.
-constexpr int kMfmaAccs = 4;
+// The single-exponent-bit operand of the matmul-free loop as the MFMA weight operand.  A 16-bit pattern with only one
+// exponent bit set is itself a number of the type: fp16 bits 14..10 = 2^1, 2^-7, 2^-11, 2^-13, 2^-14 (five classes);
+// bf16 bits 14, 13, 12 = 2^1, 2^-63, 2^-95 (three classes: the lower exponent bits would put the products of small
+// activations below the fp32 normal range).  For a pair position j the four dwords `word_wi & mask` (wi = 0..3) ARE the
+// pairs c*(b_lo, b_hi) of pair j of the unit's four words with c the class constant of the mask bit: one AND per dword
+// instead of a shift and a bit-field insert (and no inline assembly ahead of an MFMA: for instructions it does not
+// know the compiler keeps no wait states, and a bit-field insert written that way gave wrong sums now and then).
+// Shifted copies of every word bring all 16 pair positions onto a class bit: pair j sits at bits (15-j, 31-j); pair 0
+// takes the copy >> 1 and class 0, pair j >= 1 the copy << C*((j-1)/C) and class (j-1) % C with C classes.  The
+// activation operand comes from the pair-major staging layout, whose chunk j holds exactly those 8 columns.  Each
+// class has its own accumulator; sum b*x = sum_c acc_c / c (pow2_combine), and the signed sum is
+// (sum of x) - 2 (sum b*x).  Zero words contribute nothing, so "no unit" is w = 0.
+template <int DT>
+struct Pow2 {
+    static constexpr int kClasses = DT == 0 ? 5 : 3;
+};
 
 template <int DT, int BATCH>
-__device__ __forceinline__ void unit_mfma(const uint4& w, const uint4* xs, int upad, int cu, bool valid,
-                                          float4_t (&acc)[kMfmaAccs]) {
-    using E = Elem<DT>;
+__device__ __forceinline__ void unit_mfma_pow2(const uint4& w, const uint4* xs, int upad, int cu,
+                                               float4_t (&acc)[Pow2<DT>::kClasses]) {
+    constexpr int C = Pow2<DT>::kClasses;
+    constexpr uint32_t M14 = 0x40004000u;
     const int nb = min((int)(threadIdx.x & 15), BATCH - 1);
-    const uint32_t one = E::kOnePair;
+    const uint4* xrow = xs + xs_chunk_pm(nb, 0, upad, cu);
+    {   // pair 0: bit 15 -> bit 14
+        const uint4 a = make_uint4((w.x >> 1) & M14, (w.y >> 1) & M14, (w.z >> 1) & M14, (w.w >> 1) & M14);
+        acc[0] = Mfma16<DT>::run(a, xrow[0], acc[0]);
+    }
 #pragma unroll
-    for (int wi = 0; wi < 4; ++wi) {
-        const uint32_t word = comp_d(w, wi);
+    for (int j0 = 1; j0 < 16; j0 += C) {
+        const int sh = j0 - 1;                            // C * ((j - 1) / C) for the pairs j0 .. j0 + C - 1
+        const uint32_t s0 = w.x << sh, s1 = w.y << sh, s2 = w.z << sh, s3 = w.w << sh;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            uint4 a;
-            a.x = sign_onto_one(word << (4 * q + 0), one);
-            a.y = sign_onto_one(word << (4 * q + 1), one);
-            a.z = sign_onto_one(word << (4 * q + 2), one);
-            a.w = sign_onto_one(word << (4 * q + 3), one);
-            uint4 b = make_uint4(0, 0, 0, 0);
-            if (valid) b = xs[xs_chunk(nb, 4 * wi + q, upad, cu)];
-            acc[q] = Mfma16<DT>::run(a, b, acc[q]);
+        for (int cls = 0; cls < C; ++cls) {
+            const int j = j0 + cls;
+            if (j > 15) break;
+            const uint32_t mask = M14 >> cls;
+            const uint4 a = make_uint4(s0 & mask, s1 & mask, s2 & mask, s3 & mask);
+            acc[cls] = Mfma16<DT>::run(a, xrow[j], acc[cls]);
         }
     }
 }
 
-// fp16 only: the single-exponent-bit operand of the matmul-free loop as the MFMA weight operand.  For a
-// pair position j the four dwords `word_wi & mask` (wi = 0..3) ARE the fp16 pairs c*(b_lo, b_hi) of pair
-// j of the unit's four words, with c = 2^1, 2^-7, 2^-11, 2^-13, 2^-14 for the mask bit 14..10: one AND
-// per dword instead of a shift and a bit-field insert.  Three shifted copies of every word (>>1, <<5,
-// <<10) bring all 16 pair positions onto an exponent bit.  The activation operand comes from the
-// pair-major staging layout, whose chunk j holds exactly those 8 columns.  Each class of c has its own
-// accumulator: acc[0..4] for bit 14..10; sum b*x = acc0/2 + 128 acc1 + 2048 acc2 + 8192 acc3 + 16384 acc4,
-// and the signed sum is (sum of x) - 2 (sum b*x).  Zero words contribute nothing, so "no unit" is w = 0.
-constexpr int kPow2Classes = 5;
-
-template <int BATCH>
-__device__ __forceinline__ void unit_mfma_pow2(const uint4& w, const uint4* xs, int upad, int cu,
-                                               float4_t (&acc)[kPow2Classes]) {
-    constexpr uint32_t M14 = 0x40004000u;
-    const int nb = min((int)(threadIdx.x & 15), BATCH - 1);
-    const uint4* xrow = xs + xs_chunk_pm(nb, 0, upad, cu);
-    uint32_t src[4][4];   // [copy][word]: copy 0 = >>1, 1 = as is, 2 = <<5, 3 = <<10
-#pragma unroll
-    for (int wi = 0; wi < 4; ++wi) {
-        const uint32_t w0 = comp_d(w, wi);
-        src[0][wi] = w0 >> 1; src[1][wi] = w0; src[2][wi] = w0 << 5; src[3][wi] = w0 << 10;
-    }
-#pragma unroll
-    for (int j = 0; j < 16; ++j) {
-        // pair j sits at bits (15-j, 31-j): j = 0 -> copy 0 bit 14; j = 1..5 -> copy 1 bits 14..10;
-        // j = 6..10 -> copy 2 bits 14..10; j = 11..15 -> copy 3 bits 14..10
-        const int copy = j == 0 ? 0 : (j + 4) / 5;
-        const int cls = j == 0 ? 0 : (j - 1) % 5;
-        const uint32_t mask = M14 >> cls;
-        uint4 a;
-        a.x = src[copy][0] & mask; a.y = src[copy][1] & mask; a.z = src[copy][2] & mask; a.w = src[copy][3] & mask;
-        const uint4 b = xrow[j];
-        acc[cls] = Mfma16<0>::run(a, b, acc[cls]);
-    }
-}
-
-// sum b*x per accumulator element from the five class accumulators (exact power-of-two rescaling)
-__device__ __forceinline__ float4_t pow2_combine(const float4_t (&acc)[kPow2Classes]) {
-    return acc[0] * 0.5f + acc[1] * 128.f + acc[2] * 2048.f + acc[3] * 8192.f + acc[4] * 16384.f;
+// sum b*x per accumulator element from the class accumulators (exact power-of-two rescaling)
+template <int DT>
+__device__ __forceinline__ float4_t pow2_combine(const float4_t (&acc)[Pow2<DT>::kClasses]) {
+    if constexpr (DT == 0) return acc[0] * 0.5f + acc[1] * 128.f + acc[2] * 2048.f + acc[3] * 8192.f + acc[4] * 16384.f;
+    else return acc[0] * 0.5f + acc[1] * 0x1p63f + acc[2] * 0x1p95f;
 }
 
 // ---- one-bit fp4 weights x fp8 pieces of the input (batch 1..4, fp16 and bf16 alike) ---------------

@@ -128,11 +128,11 @@ __host__ __device__ __forceinline__ int mfma_items_per_wave(int nitems, int wave
 // inlined: inside the kernel its loop shares the 128 registers of a 1024-lane workgroup with everything the slice keeps
 // alive and spills into the item loop.
 // ORDER: 1 = tile order, 2 = row-major (see load_unit).
-template <int DT, int BATCH, int THREADS, bool POW2, int ORDER>
+template <int DT, int BATCH, int THREADS, int ORDER>
 __device__ __attribute__((noinline)) void stream_tail_items(BitsView bv, const uint4* xs, float* racc, int upad, int st_rows,
                                                            int row_base, int left, int tn, int c0, int cu_n) {
     constexpr int kWaves = THREADS / kWave;
-    constexpr int kAccs = POW2 ? kPow2Classes : kMfmaAccs;
+    constexpr int kAccs = Pow2<DT>::kClasses;
     const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ngroups = (cu_n + 3) >> 2;
@@ -162,9 +162,7 @@ __device__ __attribute__((noinline)) void stream_tail_items(BitsView bv, const u
 #pragma unroll
     for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
     auto flush = [&]() {
-        float4_t sum;
-        if constexpr (POW2) sum = pow2_combine(acc) * -2.f;              // signed sum = (sum of x) - 2 (sum of b x)
-        else sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+        const float4_t sum = pow2_combine<DT>(acc) * -2.f;                // signed sum = (sum of x) - 2 (sum of b x)
         if (r16 < BATCH) {
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
@@ -182,8 +180,7 @@ __device__ __attribute__((noinline)) void stream_tail_items(BitsView bv, const u
         }
         const int u = 4 * ub + g;
         if constexpr (ORDER == 2) trim_unit(bv, w, c0 + u);              // tile order pads with zero words
-        if constexpr (POW2) unit_mfma_pow2<BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
-        else unit_mfma<DT, BATCH>(w, xs, upad, u, u < cu_n, acc);
+        unit_mfma_pow2<DT, BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
         if (++ub == ngroups) { ub = 0; ++rg; }
     };
     // A full wait ahead of the first fetches: from here on they are the only loads in flight and the compiler waits for
@@ -226,8 +223,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
     extern __shared__ uint4 lds_raw[];
     static_assert(ARITH == 1 || ARITH == 2, "unknown arithmetic");
     constexpr bool kQ8 = ARITH == 2;
-    constexpr bool kPow2Mfma = ARITH == 1 && DT == 0;           // fp16 MFMA path: single-bit operands, pair-major x
-    constexpr bool kTotals = kPow2Mfma || kQ8;                  // signed sum = (sum of x) - 2 (sum of b x)
+    constexpr bool kTotals = true;                              // both arithmetics: signed sum = (sum of x) - 2 (sum of b x)
     static_assert(!kQ8 || BATCH * kQ8Pieces <= 16, "pieces of all batch rows must fit the 16 operand columns");
     static_assert(!DET || kQ8, "reproducible sums exist for the fp4 x fp8 arithmetic only");
     constexpr int kRaccFloats = kQ8 ? kRowBlock * BATCH : kTailBytes / (int)sizeof(float);   // 16-bit arithmetic: the tail's row sums
@@ -488,7 +484,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                 // wavefront a contiguous run, and summed in LDS (stream_tail_items; kTailBytes hold 256 rows at batch 16).
                 const int lane = tid & 63, r16 = lane & 15, g = lane >> 4;
                 const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // scalar item arithmetic
-                constexpr int kAccs = kPow2Mfma ? kPow2Classes : kMfmaAccs;
+                constexpr int kAccs = Pow2<DT>::kClasses;
                 const int ngroups16 = (seg.row_end - seg.row_begin + 15) >> 4;
                 const int full_rounds = ngroups16 / kWaves;                       // the same for every wavefront
                 const int tail_groups = ngroups16 - full_rounds * kWaves;
@@ -556,11 +552,9 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                 };
                 // the q-th group of this wavefront is complete: acc[v] = sum for its row 4 g + v, batch row r16
                 auto store_group = [&](int q) __attribute__((always_inline)) {
-                    float4_t sum;
-                    if constexpr (kPow2Mfma) sum = pow2_combine(acc) * -2.f;      // signed sum = (sum of x) - 2 (sum of b x)
-                    else sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+                    const float4_t sum = pow2_combine<DT>(acc) * -2.f;            // signed sum = (sum of x) - 2 (sum of b x)
                     if (r16 < BATCH) {
-                        const float xt = kPow2Mfma ? xtot[r16] : 0.f;
+                        const float xt = xtot[r16];
                         const int row0 = seg.row_begin + 16 * (wave + kWaves * q) + 4 * g;
                         if (row0 < seg.row_end) emit4(row0, r16, sum + xt);
                     }
@@ -621,8 +615,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                     auto work = [&](uint4& w, int j) {
                         const int u = 4 * j + g;
                         if constexpr (kOrder == 2) trim_unit(bv, w, c0 + u);   // tile order pads with zero words
-                        if constexpr (kPow2Mfma) unit_mfma_pow2<BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
-                        else unit_mfma<DT, BATCH>(w, xs, upad, u, u < cu_n, acc);
+                        unit_mfma_pow2<DT, BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
                     };
                     // A full wait ahead of the first fetches (what the staging loaded has been used) and after the stores
                     // of a group: inside the loop the item fetches are the only accesses in flight and the compiler waits
@@ -656,7 +649,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                     const int rows = seg.row_end - tail_base;
                     for (int i = tid; i < rows * BATCH; i += kStreamThreads) {
                         const int rel = i / BATCH, b = i % BATCH;
-                        emit1(tail_base + rel, b, racc[tail_index<BATCH>(rel, b)] + (kPow2Mfma ? xtot[b] : 0.f));
+                        emit1(tail_base + rel, b, racc[tail_index<BATCH>(rel, b)] + xtot[b]);
                     }
                 };
                 auto zero_tail = [&]() {
@@ -666,13 +659,13 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                 auto stage_chunk = [&](int c0, int cu_n, bool clear_tail) __attribute__((always_inline)) {
                     if (staged) {
                         lds_barrier();                                    // every wavefront is done with the staged chunk, the totals and the tail's sums
-                        if (kPow2Mfma && c0 == 0) {
+                        if (c0 == 0) {
                             if (tid < kTotStride) xtot[tid] = 0.f;        // staged again from the first column: the totals start over
                             lds_barrier();
                         }
                     }
                     if (clear_tail) zero_tail();
-                    stage_units<DT, BATCH, kPow2Mfma>(xs, nullptr, sin, c0, cu_n, upad, kStreamThreads, kPow2Mfma ? xtot : nullptr);
+                    stage_units<DT, BATCH, true>(xs, nullptr, sin, c0, cu_n, upad, kStreamThreads, xtot);
                     staged = true;
                     lds_barrier();                                        // staged input, its totals and the cleared sums visible
                 };
@@ -681,8 +674,8 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                     else run_items(std::integral_constant<int, 2>{}, q_begin, q_end, c0, cu_n, complete);
                 };
                 auto shared = [&](int c0, int cu_n) __attribute__((always_inline)) {
-                    if (bv.groups) stream_tail_items<DT, BATCH, THREADS, kPow2Mfma, 1>(bv, xs, racc, upad, st.rows, tail_base, seg.row_end - tail_base, tail_groups, c0, cu_n);
-                    else stream_tail_items<DT, BATCH, THREADS, kPow2Mfma, 2>(bv, xs, racc, upad, st.rows, tail_base, seg.row_end - tail_base, tail_groups, c0, cu_n);
+                    if (bv.groups) stream_tail_items<DT, BATCH, THREADS, 1>(bv, xs, racc, upad, st.rows, tail_base, seg.row_end - tail_base, tail_groups, c0, cu_n);
+                    else stream_tail_items<DT, BATCH, THREADS, 2>(bv, xs, racc, upad, st.rows, tail_base, seg.row_end - tail_base, tail_groups, c0, cu_n);
                 };
                 // whole rounds: an input of one chunk is staged once and every wavefront walks all its groups in one go
                 const int staged_rounds = one_chunk ? min(full_rounds, 1) : full_rounds;
