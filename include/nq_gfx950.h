@@ -154,10 +154,12 @@ int nq_runlist_status(const void* workspace, int* status_out, void* stream);
 /* Reproducible sums for the launches of this plan, on (1) or off (0, as built).  The run-list kernel finishes a row
  * sum with additions from several wavefronts whose order differs from launch to launch, so outputs may differ in
  * the last bit between launches (the reference's reductions are ordered: kernel/cuda/gemv_kernel.cu:148-170,
- * shuffles inside one warp).  With this switch every launch of the plan gives bit-identical outputs: partial sums
- * are rounded to a grid on which their additions are exact.  The results stay within the same tolerance but lose up
- * to 16 bits below (columns x largest input value); available for batch 1, 2 and 4 (NQ_ERR_SHAPE otherwise).  Sets
- * bit 3 of plan->bound. */
+ * shuffles inside one warp).  With this switch every launch of the plan gives bit-identical outputs.  Batch 1, 2 and
+ * 4: partial sums are rounded to a grid on which their additions are exact; the results stay within the same
+ * tolerance but lose up to 16 bits below (columns x largest input value).  Batch 8 and 16: every row sum is formed by
+ * one wavefront (without the switch only the rows left over after a slice's rounds of 256 are summed by several),
+ * same arithmetic, slices of few rows run slower.  NQ_ERR_SHAPE for a batch size without a run-list kernel.  Sets bit 3
+ * of plan->bound. */
 int nq_runlist_set_deterministic(nq_runlist_plan* plan, int on);
 
 /* One matmul-free stage: out[b,row] = s_row[row] * sum_c sgn(bits[row,c]) * in[b,c] * s_col[c].

@@ -107,7 +107,7 @@ __device__ __forceinline__ void trim_unit(const BitsView& v, uint4& w, int unit)
 // atomic fall into different banks (tail_index).
 constexpr int kTailBytes = 20 * 1024;
 __host__ __device__ constexpr size_t stream_head_bytes(int batch, int arith, bool det = false) {
-    return (arith == 2 ? (size_t)row_block(batch) * batch * sizeof(float) * (det ? 2 : 1) : (size_t)kTailBytes) + (det ? 1024 : 128);
+    return arith == 2 ? (size_t)row_block(batch) * batch * sizeof(float) * (det ? 2 : 1) + (det ? 1024 : 128) : (size_t)kTailBytes + 128;
 }
 // Row sum (row, batch row b) of the tail: 16 floats of padding after every 4 rows at batch 16 (the four lane groups of
 // an MFMA result are 4 rows apart: 64 floats, the same bank), 8 after every 8 rows at batch 8.
@@ -203,7 +203,7 @@ __device__ __attribute__((noinline)) void stream_tail_items(BitsView bv, const u
 }
 
 // ARITH: 1 = MFMA with 16-bit operands, 2 = MFMA with one-bit fp4 weights and fp8 pieces of the input (batch <= 4).
-// DET (fp4 x fp8 arithmetic only): row sums that do not depend on the order in which the wavefronts of a workgroup add
+// DET, fp4 x fp8 arithmetic: row sums that do not depend on the order in which the wavefronts of a workgroup add
 // their partial sums.  Every partial sum is rounded to a grid fine enough (2^-22 of columns x largest staged value, a
 // bound on every sum of the chunk) that all additions into a row sum are exact; the input totals are kept per wavefront
 // and added in wavefront order; the row sums of successive input chunks (different grids) are added one chunk after
@@ -225,14 +225,13 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
     constexpr bool kQ8 = ARITH == 2;
     constexpr bool kTotals = true;                              // both arithmetics: signed sum = (sum of x) - 2 (sum of b x)
     static_assert(!kQ8 || BATCH * kQ8Pieces <= 16, "pieces of all batch rows must fit the 16 operand columns");
-    static_assert(!DET || kQ8, "reproducible sums exist for the fp4 x fp8 arithmetic only");
     constexpr int kRaccFloats = kQ8 ? kRowBlock * BATCH : kTailBytes / (int)sizeof(float);   // 16-bit arithmetic: the tail's row sums
     float* racc = (float*)lds_raw;                              // [kRowBlock][BATCH] row sums
     float* rtot = racc + kRaccFloats;                           // DET: the same, summed over the input chunks done so far
     // [2][16] sum of the staged input per batch row (DET: [2][16 wavefronts][4]); slices alternate between the two, so
     // that the one of the next slice is cleared a barrier ahead of its staging instead of costing a barrier of its own
-    constexpr int kTotStride = DET ? 64 : 16;
-    float* xtot_base = racc + kRaccFloats * (DET ? 2 : 1);
+    constexpr int kTotStride = (DET && kQ8) ? 64 : 16;
+    float* xtot_base = racc + kRaccFloats * (DET && kQ8 ? 2 : 1);
     uint32_t* ebmax_base = (uint32_t*)(xtot_base + 2 * kTotStride);   // DET: [2] largest unit exponent of the staged input
     uint4* xs_base = lds_raw + stream_head_bytes(BATCH, ARITH, DET) / sizeof(uint4);
     __shared__ int s_flag;
@@ -240,7 +239,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
     const int wg = blockIdx.x;
     if (tid == 0) s_flag = 0;
     if (tid < 2 * kTotStride) xtot_base[tid] = 0.f;
-    if (DET && tid < 2) ebmax_base[tid] = 0u;
+    if (DET && kQ8 && tid < 2) ebmax_base[tid] = 0u;
     int slice_count = 0;
 
     // Which launch of this run list is this?  Needed only by waiting slices; the load is issued now and
@@ -467,7 +466,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
             lds_barrier();                                       // s_flag; previous slice is done with xs / racc
             aborted = aborted || (s_flag != 0);
             if (tid < kTotStride) xtot_other[tid] = 0.f;         // every reader of it (the previous slice) is past the barrier
-            if (DET && tid == 0) ebmax_base[slice_count & 1] = 0u;   // slice_count was advanced: this is the other one
+            if (DET && kQ8 && tid == 0) ebmax_base[slice_count & 1] = 0u;   // slice_count was advanced: this is the other one
 
             if constexpr (!kQ8) {
               if (!aborted) {
@@ -486,8 +485,12 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                 const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // scalar item arithmetic
                 constexpr int kAccs = Pow2<DT>::kClasses;
                 const int ngroups16 = (seg.row_end - seg.row_begin + 15) >> 4;
-                const int full_rounds = ngroups16 / kWaves;                       // the same for every wavefront
-                const int tail_groups = ngroups16 - full_rounds * kWaves;
+                // DET (reproducible sums): the left-over groups make one more round, owned like the others (some
+                // wavefronts idle), instead of being summed by several wavefronts in hardware order; the input totals are
+                // added up unit by unit in a fixed order instead of with LDS atomics.
+                const int full_rounds = DET ? (ngroups16 + kWaves - 1) / kWaves : ngroups16 / kWaves;   // the same for every wavefront
+                const int tail_groups = DET ? 0 : ngroups16 - full_rounds * kWaves;
+                const int my_rounds = DET ? (ngroups16 > wave ? (ngroups16 - wave + kWaves - 1) / kWaves : 0) : full_rounds;
                 const int tail_base = seg.row_begin + 16 * full_rounds * kWaves;  // first row of the tail
                 float4_t acc[kAccs];
 #pragma unroll
@@ -590,7 +593,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                     constexpr int kOrder = decltype(order_c)::value;      // one copy of the loop per word order: see load_unit
                     const int ngroups = (cu_n + 3) >> 2;
                     const int positions = (ngroups + 2) / 3 * 3;
-                    const int nq = max(min(q_end, full_rounds) - q_begin, 0);
+                    const int nq = max(min(q_end, my_rounds) - q_begin, 0);
                     int f_left = nq * positions, f_q = q_begin, f_j = 0;  // fetch cursor
                     auto fetch = [&](uint4& w) {
                         if constexpr (kOrder == 1) {
@@ -665,7 +668,19 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                         }
                     }
                     if (clear_tail) zero_tail();
-                    stage_units<DT, BATCH, true>(xs, nullptr, sin, c0, cu_n, upad, kStreamThreads, xtot);
+                    if constexpr (DET) {
+                        // unit totals to LDS (the tail's row sums are not used in this mode), then one lane per batch row
+                        // adds them in unit order
+                        stage_units<DT, BATCH, true>(xs, racc, sin, c0, cu_n, upad, kStreamThreads, nullptr);
+                        lds_barrier();
+                        if (tid < BATCH) {
+                            float t = 0.f;
+                            for (int cu = 0; cu < cu_n; ++cu) t += racc[tid * upad + cu];
+                            xtot[tid] += t;
+                        }
+                    } else {
+                        stage_units<DT, BATCH, true>(xs, nullptr, sin, c0, cu_n, upad, kStreamThreads, xtot);
+                    }
                     staged = true;
                     lds_barrier();                                        // staged input, its totals and the cleared sums visible
                 };
@@ -956,8 +971,8 @@ struct StreamKernel {
     static constexpr auto fn = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, false>;
     static constexpr auto fn_tiled = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2>;
     static constexpr auto fn_single = gemv_stream_kernel<DT, BATCH, kArith, kThreads, true, false>;
-    // reproducible sums: fp4 x fp8 arithmetic only (elsewhere these name the ordinary kernels and are never launched)
-    static constexpr bool kHasDet = kArith == 2;
+    // reproducible sums
+    static constexpr bool kHasDet = true;
     static constexpr auto fn_det = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, false, kHasDet>;
     static constexpr auto fn_tiled_det = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2, kHasDet>;
 };
@@ -1113,7 +1128,7 @@ int stream_row_granule(int dtype, int batch) {
     return 32;
 }
 
-// Reproducible sums exist for the fp4 x fp8 arithmetic.
+// Reproducible sums exist for every batch size that has a run-list kernel.
 bool stream_has_deterministic(int dtype, int batch) {
 #define NQ_DET(D, B) (StreamKernel<D, B>::kHasDet)
     NQ_STREAM_DISPATCH(NQ_DET)

@@ -362,11 +362,11 @@ def test_outlier_channels_leave_the_other_contributions_intact(dev, dtype, batch
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("batch,tiled", [(1, True), (1, False), (2, True), (4, True), (4, False)])
+@pytest.mark.parametrize("batch,tiled", [(1, True), (1, False), (2, True), (4, True), (4, False), (8, True), (16, True), (16, False)])
 def test_deterministic_lists_repeat_bit_for_bit(dev, batch, tiled, dtype):
     """`deterministic=True`: every launch of a list gives the same bits (eager launches and graph replays alike), and
     the results still meet the tolerance.  The shapes make many wavefronts add into the same row sums (few rows per
-    workgroup), include an input of 16384 columns (more than one staged chunk at batch 4) and a ragged one, and
+    workgroup), include an input of 16384 columns (more than one staged chunk from batch 4 on) and a ragged one, and
     the second linear reads the first one's output, so a difference anywhere upstream would show."""
     shapes = [(1024, 4096, 512), (512, 16384, 736), (1376, 1000, 96)]
     rl = DecodeRunList(batch, dtype, dev, deterministic=True)
@@ -390,8 +390,10 @@ def test_deterministic_lists_repeat_bit_for_bit(dev, batch, tiled, dtype):
     first = [y.clone() for y in rl.run()]
     torch.cuda.synchronize()
     assert rl.status() == 0
+    # batch 8 and 16 round x * s_in and the intermediate vector to the activation type when staging
+    tol = 1e-2 if (batch >= 8 and dtype == torch.bfloat16) else 1e-3
     for y, ref in zip(first, refs):
-        assert oracle.max_rel_err(y.cpu().numpy(), ref) < 1e-3
+        assert oracle.max_rel_err(y.cpu().numpy(), ref) < tol
     for rep in range(20):
         for y in rl.outputs:
             y.fill_(float("nan"))
@@ -421,14 +423,6 @@ def test_deterministic_lists_repeat_bit_for_bit(dev, batch, tiled, dtype):
         torch.cuda.synchronize()
         differing += int(any(not torch.equal(y, e) for y, e in zip(ys, base)))
     print(f"  default mode: {differing} of 20 launches differ from the first in some bit", flush=True)
-
-
-def test_deterministic_mode_is_refused_where_it_does_not_exist(dev):
-    _, ops = _term(dev, 256, 512, 64, seed=650)
-    rl = DecodeRunList(8, torch.float16, dev, deterministic=True)
-    rl.add(torch.from_numpy(oracle.synth_x(8, 512, 651)).to(dev), *ops)
-    with pytest.raises(RuntimeError):
-        rl.build()
 
 
 def test_an_expired_wait_is_reported_and_the_list_stays_usable(dev):

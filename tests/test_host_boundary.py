@@ -275,8 +275,11 @@ def test_row_routing_and_run_list_options_need_no_gpu():
     assert rl.deterministic and rl.spin_limit == 0
     with pytest.raises(ValueError):
         DecodeRunList(3, torch.float16, "cpu")
-    plan = NqRunlistPlan(batch=8, dtype=_lib.NQ_F16)
-    assert _lib.lib().nq_runlist_set_deterministic(ctypes.byref(plan), 1) != 0      # no such kernel at batch 8
+    plan = NqRunlistPlan(batch=3, dtype=_lib.NQ_F16)
+    assert _lib.lib().nq_runlist_set_deterministic(ctypes.byref(plan), 1) != 0      # no run-list kernel for 3 rows
+    for b in (8, 16):
+        plan = NqRunlistPlan(batch=b, dtype=_lib.NQ_BF16)
+        assert _lib.lib().nq_runlist_set_deterministic(ctypes.byref(plan), 1) == 0 and plan.bound & 8
     plan = NqRunlistPlan(batch=4, dtype=_lib.NQ_F16)
     assert _lib.lib().nq_runlist_set_deterministic(ctypes.byref(plan), 1) == 0 and plan.bound & 8
     assert _lib.lib().nq_runlist_set_deterministic(ctypes.byref(plan), 0) == 0 and not plan.bound & 8
