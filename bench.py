@@ -81,16 +81,11 @@ class SynthLinear:
                 self.vt_bits = self.u_bits = None
         return self._tiled
 
-    def add_to(self, rl, x, keep_row_major=True, tiled=None, **kw):
-        """Tile order up to batch 4 and, from batch 8 on, in long lists (`tiled=True`: Llama-2-7B stack at batch 16
-        12.6 against 14.5 us per layer).  A list of one layer at batch 8 or 16 reads the row-major words: tile order is
-        cut into slices at multiples of 32 rows, which balances a few hundred rows per workgroup worse (60 against
-        54 us per layer at batch 16)."""
+    def add_to(self, rl, x, keep_row_major=True, **kw):
+        """Tile order at every batch size: the run-list kernels fetch an item with scalar address arithmetic there
+        (Llama-2-7B stack at batch 16 13.0 against 14.1 us per layer on row-major words, one launch per layer 47 against
+        53)."""
         s_in, s_mid, s_out = self.scales_as(x.dtype)
-        if tiled is None:
-            tiled = rl.batch <= 4
-        if not tiled:
-            return rl.add(x, s_in, self.vt_bits, s_mid, self.u_bits, s_out, **kw)
         vt, u = self.runlist_words(keep_row_major)
         return rl.add(x, s_in, vt, s_mid, u, s_out, tiled=True, **kw)
 
@@ -218,7 +213,7 @@ def main():
         rl = DecodeRunList(batch, dtype, dev, deterministic=deterministic)
         for layer in layers:
             for lin, x, y in zip(layer, xs, ys):
-                lin.add_to(rl, x, y=y, tiled=True)
+                lin.add_to(rl, x, y=y)
         rl.build()
         return rl
 
@@ -247,7 +242,7 @@ def main():
             rl = DecodeRunList(b, torch.float16, dev)
             for layer in stack70:
                 for lin in layer:
-                    lin.add_to(rl, x70[lin.n], tiled=True)
+                    lin.add_to(rl, x70[lin.n])
             rl.build()
             ms70 = timed([rl.run], 5, 1)
             if rl.status() != 0:

@@ -157,9 +157,8 @@ int nq_runlist_status(const void* workspace, int* status_out, void* stream);
  * shuffles inside one warp).  With this switch every launch of the plan gives bit-identical outputs.  Batch 1, 2 and
  * 4: partial sums are rounded to a grid on which their additions are exact; the results stay within the same
  * tolerance but lose up to 16 bits below (columns x largest input value).  Batch 8 and 16: every row sum is formed by
- * one wavefront (without the switch only the rows left over after a slice's rounds of 256 are summed by several),
- * same arithmetic, slices of few rows run slower.  NQ_ERR_SHAPE for a batch size without a run-list kernel.  Sets bit 3
- * of plan->bound. */
+ * one wavefront in a fixed order whether the switch is on or off; it is accepted and selects the same kernel.
+ * NQ_ERR_SHAPE for a batch size without a run-list kernel.  Sets bit 3 of plan->bound. */
 int nq_runlist_set_deterministic(nq_runlist_plan* plan, int on);
 
 /* One matmul-free stage: out[b,row] = s_row[row] * sum_c sgn(bits[row,c]) * in[b,c] * s_col[c].

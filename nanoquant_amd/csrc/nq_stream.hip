@@ -102,105 +102,15 @@ __device__ __forceinline__ void trim_unit(const BitsView& v, uint4& w, int unit)
 // Bytes of LDS in front of the staged input: row sums and two sets of input totals [2][16].  Reproducible sums (det):
 // a second set of row sums (what earlier input chunks of the row block added up to), two sets of per-wavefront input
 // totals [2][16][4] and two exponent words.
-// The 16-bit arithmetic keeps the row sums of whole rounds in registers and only those of the last, partial round of a
-// slice in LDS: kTailBytes for up to 128 / batch row pairs at a time, rows padded apart so that the lanes of one LDS
-// atomic fall into different banks (tail_index).
-constexpr int kTailBytes = 20 * 1024;
+// The 16-bit arithmetic keeps its row sums in registers; its LDS head holds the totals of the staged units
+// ([batch][units + 1] floats, added up in unit order: no LDS atomics, so the results do not depend on their order).
+constexpr int kUnitTotalsBytes = 4096;
 __host__ __device__ constexpr size_t stream_head_bytes(int batch, int arith, bool det = false) {
-    return arith == 2 ? (size_t)row_block(batch) * batch * sizeof(float) * (det ? 2 : 1) + (det ? 1024 : 128) : (size_t)kTailBytes + 128;
-}
-// Row sum (row, batch row b) of the tail: 16 floats of padding after every 4 rows at batch 16 (the four lane groups of
-// an MFMA result are 4 rows apart: 64 floats, the same bank), 8 after every 8 rows at batch 8.
-template <int BATCH>
-__device__ __forceinline__ int tail_index(int row, int b) {
-    static_assert(BATCH <= 16, "kTailBytes hold 256 rows of up to 16 batch rows with their padding");
-    return row * BATCH + b + (BATCH == 16 ? 16 * (row >> 2) : BATCH == 8 ? 8 * (row >> 3) : 0);
+    return arith == 2 ? (size_t)row_block(batch) * batch * sizeof(float) * (det ? 2 : 1) + (det ? 1024 : 128) : (size_t)kUnitTotalsBytes + 128;
 }
 
-// Items of the MFMA path that each wavefront of a workgroup takes (contiguous runs).
+// fp4 x fp8 arithmetic: items that each wavefront of a workgroup takes (contiguous runs).
 __host__ __device__ __forceinline__ int mfma_items_per_wave(int nitems, int waves) { return (nitems + waves - 1) / waves; }
-
-// 16-bit MFMA arithmetic, the row groups of a slice that are left over after the whole rounds (see the kernel): `tn`
-// groups of 16 rows from row `row_base` of the matrix (`left` rows of them belong to the slice) times the unit groups of
-// the staged chunk (c0, cu_n).  Items = (16-row group, 4-unit group), unit group fastest, every wavefront a contiguous run of them;
-// the partial sums of a run go to the tail's row sums `racc` (LDS float atomics) when the row group changes and at the
-// end.  Three item fetches (1 KB each) in flight, in three register sets that take turns.  A function of its own, not
-// inlined: inside the kernel its loop shares the 128 registers of a 1024-lane workgroup with everything the slice keeps
-// alive and spills into the item loop.
-// ORDER: 1 = tile order, 2 = row-major (see load_unit).
-template <int DT, int BATCH, int THREADS, int ORDER>
-__device__ __attribute__((noinline)) void stream_tail_items(BitsView bv, const uint4* xs, float* racc, int upad, int st_rows,
-                                                           int row_base, int left, int tn, int c0, int cu_n) {
-    constexpr int kWaves = THREADS / kWave;
-    constexpr int kAccs = Pow2<DT>::kClasses;
-    const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int ngroups = (cu_n + 3) >> 2;
-    const int nitems = tn * ngroups;
-    const int per = mfma_items_per_wave(nitems, kWaves);
-    const int it_begin = min(wave * per, nitems), it_end = min(it_begin + per, nitems);
-    int f_it = it_begin, f_rg = it_begin / ngroups, f_ub = it_begin - (it_begin / ngroups) * ngroups;   // fetch cursor
-    int rg = f_rg, ub = f_ub, rg_run = f_rg;                                                           // compute cursor (row group = 16 rows)
-    auto fetch = [&](uint4& w) {
-        if constexpr (ORDER == 1) {
-            // 1 KB = one half of a 2 KB tile (row_base is a multiple of 16)
-            const bool ok = f_it < it_end;
-            const int half = (row_base >> 4) + f_rg;
-            const int tile = (half >> 1) * bv.groups + (c0 >> 2) + f_ub;
-            const uint32_t soff = ok ? (uint32_t)__builtin_amdgcn_readfirstlane(tile * 2048 + (half & 1) * 1024) : 0u;
-            const uint32_t voff = ok ? (uint32_t)lane * 16u : kPastEnd;
-            const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(bv.rsrc, voff, soff, 2 /* nt */);
-            w = make_uint4(a.x, a.y, a.z, a.w);
-        } else {
-            const int u = 4 * f_ub + g;
-            w = load_unit<ORDER>(bv, min(row_base + 16 * f_rg + r16, st_rows - 1), c0 + u, f_it < it_end && u < cu_n);
-        }
-        ++f_it;
-        if (++f_ub == ngroups) { f_ub = 0; ++f_rg; }
-    };
-    float4_t acc[kAccs];
-#pragma unroll
-    for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
-    auto flush = [&]() {
-        const float4_t sum = pow2_combine<DT>(acc) * -2.f;                // signed sum = (sum of x) - 2 (sum of b x)
-        if (r16 < BATCH) {
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int rel = 16 * rg_run + 4 * g + v;
-                if (rel < left) atomicAdd(&racc[tail_index<BATCH>(rel, r16)], sum[v]);
-            }
-        }
-#pragma unroll
-        for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
-    };
-    auto work = [&](uint4& w) {
-        if (rg != rg_run) {
-            flush();
-            rg_run = rg;
-        }
-        const int u = 4 * ub + g;
-        if constexpr (ORDER == 2) trim_unit(bv, w, c0 + u);              // tile order pads with zero words
-        unit_mfma_pow2<DT, BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
-        if (++ub == ngroups) { ub = 0; ++rg; }
-    };
-    // A full wait ahead of the first fetches: from here on they are the only loads in flight and the compiler waits for
-    // the oldest of them only, not for all.
-    __builtin_amdgcn_s_waitcnt(0);
-    uint4 w0, w1, w2;
-    fetch(w0);
-    fetch(w1);
-    fetch(w2);
-    int it = it_begin;
-#pragma unroll 1
-    for (; it + 3 <= it_end; it += 3) {
-        work(w0); fetch(w0);
-        work(w1); fetch(w1);
-        work(w2); fetch(w2);
-    }
-    if (it < it_end) work(w0);
-    if (it + 1 < it_end) work(w1);
-    if (it_begin < it_end) flush();
-}
 
 // ARITH: 1 = MFMA with 16-bit operands, 2 = MFMA with one-bit fp4 weights and fp8 pieces of the input (batch <= 4).
 // DET, fp4 x fp8 arithmetic: row sums that do not depend on the order in which the wavefronts of a workgroup add
@@ -225,7 +135,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
     constexpr bool kQ8 = ARITH == 2;
     constexpr bool kTotals = true;                              // both arithmetics: signed sum = (sum of x) - 2 (sum of b x)
     static_assert(!kQ8 || BATCH * kQ8Pieces <= 16, "pieces of all batch rows must fit the 16 operand columns");
-    constexpr int kRaccFloats = kQ8 ? kRowBlock * BATCH : kTailBytes / (int)sizeof(float);   // 16-bit arithmetic: the tail's row sums
+    constexpr int kRaccFloats = kQ8 ? kRowBlock * BATCH : kUnitTotalsBytes / (int)sizeof(float);   // 16-bit arithmetic: the unit totals
     float* racc = (float*)lds_raw;                              // [kRowBlock][BATCH] row sums
     float* rtot = racc + kRaccFloats;                           // DET: the same, summed over the input chunks done so far
     // [2][16] sum of the staged input per batch row (DET: [2][16 wavefronts][4]); slices alternate between the two, so
@@ -474,24 +384,20 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                 // A group = 16 consecutive rows of the slice (the rows of one MFMA).  In a round, wavefront w takes group
                 // 16 * round + w and walks ALL columns of it, so a row sum lives in its MFMA accumulators from the first
                 // column to the last and goes from there straight to the output: no row sums in LDS, no LDS atomics (at
-                // batch 16 they cost more than the arithmetic), no barrier between rows.  With an input of one chunk the
-                // wavefronts of a workgroup meet once per slice (after the staging) and the item fetches of a wavefront
-                // run on from group to group; with a longer input the chunks are staged again for every round and the
-                // accumulators are kept across the chunks of a round.  The groups left over after the whole rounds
-                // (fewer than 16: a wavefront needs tens of microseconds for a group, so leaving wavefronts idle there
-                // costs a tenth of a long slice and most of a short one) are shared out item by item instead, every
-                // wavefront a contiguous run, and summed in LDS (stream_tail_items; kTailBytes hold 256 rows at batch 16).
+                // batch 16 they cost more than the arithmetic), no barrier between rows, and results that do not depend
+                // on any order left to the hardware.  With an input of one chunk the wavefronts of a workgroup meet once
+                // per slice (after the staging) and the item fetches of a wavefront run on from group to group; with a
+                // longer input the chunks are staged again for every round and the accumulators are kept across the
+                // chunks of a round.  In the last round of a slice some wavefronts have no group.  (Sharing that round
+                // out item by item, with LDS float atomics into 20 KB of row sums and an epilogue by all lanes, measured
+                // the same on long lists and slower on short ones: 58 against 47 us per Llama-2-7B layer and launch at
+                // batch 16.)
                 const int lane = tid & 63, r16 = lane & 15, g = lane >> 4;
                 const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // scalar item arithmetic
                 constexpr int kAccs = Pow2<DT>::kClasses;
                 const int ngroups16 = (seg.row_end - seg.row_begin + 15) >> 4;
-                // DET (reproducible sums): the left-over groups make one more round, owned like the others (some
-                // wavefronts idle), instead of being summed by several wavefronts in hardware order; the input totals are
-                // added up unit by unit in a fixed order instead of with LDS atomics.
-                const int full_rounds = DET ? (ngroups16 + kWaves - 1) / kWaves : ngroups16 / kWaves;   // the same for every wavefront
-                const int tail_groups = DET ? 0 : ngroups16 - full_rounds * kWaves;
-                const int my_rounds = DET ? (ngroups16 > wave ? (ngroups16 - wave + kWaves - 1) / kWaves : 0) : full_rounds;
-                const int tail_base = seg.row_begin + 16 * full_rounds * kWaves;  // first row of the tail
+                const int rounds = (ngroups16 + kWaves - 1) / kWaves;            // the same for every wavefront
+                const int my_rounds = ngroups16 > wave ? (ngroups16 - wave + kWaves - 1) / kWaves : 0;
                 float4_t acc[kAccs];
 #pragma unroll
                 for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
@@ -562,26 +468,6 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                         if (row0 < seg.row_end) emit4(row0, r16, sum + xt);
                     }
                 };
-                // one row of one batch row (the tail's epilogue; same order of operations as emit4)
-                auto emit1 = [&](int row, int b, float v) __attribute__((always_inline)) {
-                    if (st.s_row) v *= E::to_float(st.s_row[row]);
-                    if (st.bias) v += E::to_float(st.bias[row]);
-                    const size_t o = (size_t)b * st.out_stride + row;
-                    if (st.addend) {
-                        if (st.dep2 >= 0)
-                            v += __builtin_bit_cast(float, __hip_atomic_load((const uint32_t*)st.addend + o, __ATOMIC_RELAXED,
-                                                                             __HIP_MEMORY_SCOPE_AGENT));
-                        else
-                            v += st.addend[o];
-                    }
-                    if (st.out_f32) {
-                        if (st.signal) __hip_atomic_store((uint32_t*)st.out + o, __builtin_bit_cast(uint32_t, v),
-                                                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        else ((float*)st.out)[o] = v;
-                    } else {
-                        ((uint16_t*)st.out)[o] = E::from_float_clamped(v);
-                    }
-                };
                 // The groups [q_begin, q_end) of this wavefront times the unit groups of the staged chunk (c0, cu_n).
                 // Items = (row group, 4-unit group), unit group fastest.  Three item fetches (1 KB of packed words each) in
                 // flight, in three register sets that take turns, each refilled right after its use; a row group is
@@ -593,7 +479,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                     constexpr int kOrder = decltype(order_c)::value;      // one copy of the loop per word order: see load_unit
                     const int ngroups = (cu_n + 3) >> 2;
                     const int positions = (ngroups + 2) / 3 * 3;
-                    const int nq = max(min(q_end, my_rounds) - q_begin, 0);
+                    const int nq = max(min(q_end, my_rounds) - q_begin, 0);   // the last round has groups for some wavefronts only
                     int f_left = nq * positions, f_q = q_begin, f_j = 0;  // fetch cursor
                     auto fetch = [&](uint4& w) {
                         if constexpr (kOrder == 1) {
@@ -647,72 +533,41 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                         }
                     }
                 };
-                // the tail's row sums are complete (a barrier has passed): all lanes share out its rows
-                auto tail_store = [&]() __attribute__((always_inline)) {
-                    const int rows = seg.row_end - tail_base;
-                    for (int i = tid; i < rows * BATCH; i += kStreamThreads) {
-                        const int rel = i / BATCH, b = i % BATCH;
-                        emit1(tail_base + rel, b, racc[tail_index<BATCH>(rel, b)] + xtot[b]);
-                    }
-                };
-                auto zero_tail = [&]() {
-                    for (int i = tid; i < kTailBytes / (int)sizeof(float); i += kStreamThreads) racc[i] = 0.f;
-                };
                 bool staged = false;                                      // a chunk is staged and may be in use
-                auto stage_chunk = [&](int c0, int cu_n, bool clear_tail) __attribute__((always_inline)) {
+                float* unit_tot = racc;                                   // [BATCH][upad] totals of the staged units
+                auto stage_chunk = [&](int c0, int cu_n) __attribute__((always_inline)) {
                     if (staged) {
-                        lds_barrier();                                    // every wavefront is done with the staged chunk, the totals and the tail's sums
+                        lds_barrier();                                    // every wavefront is done with the staged chunk and the totals
                         if (c0 == 0) {
                             if (tid < kTotStride) xtot[tid] = 0.f;        // staged again from the first column: the totals start over
                             lds_barrier();
                         }
                     }
-                    if (clear_tail) zero_tail();
-                    if constexpr (DET) {
-                        // unit totals to LDS (the tail's row sums are not used in this mode), then one lane per batch row
-                        // adds them in unit order
-                        stage_units<DT, BATCH, true>(xs, racc, sin, c0, cu_n, upad, kStreamThreads, nullptr);
-                        lds_barrier();
-                        if (tid < BATCH) {
-                            float t = 0.f;
-                            for (int cu = 0; cu < cu_n; ++cu) t += racc[tid * upad + cu];
-                            xtot[tid] += t;
-                        }
-                    } else {
-                        stage_units<DT, BATCH, true>(xs, nullptr, sin, c0, cu_n, upad, kStreamThreads, xtot);
+                    // unit totals to LDS, then one lane per batch row adds them in unit order
+                    stage_units<DT, BATCH, true>(xs, unit_tot, sin, c0, cu_n, upad, kStreamThreads, nullptr);
+                    lds_barrier();
+                    if (tid < BATCH) {
+                        float t = 0.f;
+                        for (int cu = 0; cu < cu_n; ++cu) t += unit_tot[tid * upad + cu];
+                        xtot[tid] += t;
                     }
                     staged = true;
-                    lds_barrier();                                        // staged input, its totals and the cleared sums visible
+                    lds_barrier();                                        // staged input and its totals visible
                 };
                 auto owned = [&](int q_begin, int q_end, int c0, int cu_n, bool complete) __attribute__((always_inline)) {
                     if (bv.groups) run_items(std::integral_constant<int, 1>{}, q_begin, q_end, c0, cu_n, complete);
                     else run_items(std::integral_constant<int, 2>{}, q_begin, q_end, c0, cu_n, complete);
                 };
-                auto shared = [&](int c0, int cu_n) __attribute__((always_inline)) {
-                    if (bv.groups) stream_tail_items<DT, BATCH, THREADS, 1>(bv, xs, racc, upad, st.rows, tail_base, seg.row_end - tail_base, tail_groups, c0, cu_n);
-                    else stream_tail_items<DT, BATCH, THREADS, 2>(bv, xs, racc, upad, st.rows, tail_base, seg.row_end - tail_base, tail_groups, c0, cu_n);
-                };
-                // whole rounds: an input of one chunk is staged once and every wavefront walks all its groups in one go
-                const int staged_rounds = one_chunk ? min(full_rounds, 1) : full_rounds;
+                // an input of one chunk is staged once and every wavefront walks all its groups in one go
+                const int staged_rounds = one_chunk ? min(rounds, 1) : rounds;
 #pragma unroll 1
                 for (int r = 0; r < staged_rounds; ++r) {
 #pragma unroll 1
                     for (int c0 = 0; c0 < st.units; c0 += chunk_units) {
                         const int cu_n = min(chunk_units, st.units - c0);
-                        stage_chunk(c0, cu_n, one_chunk && tail_groups > 0);
-                        owned(one_chunk ? 0 : r, one_chunk ? full_rounds : r + 1, c0, cu_n, c0 + chunk_units >= st.units);
+                        stage_chunk(c0, cu_n);
+                        owned(one_chunk ? 0 : r, one_chunk ? rounds : r + 1, c0, cu_n, c0 + chunk_units >= st.units);
                     }
-                }
-                // the groups left over (fewer than 16: their row sums fit kTailBytes)
-                if (tail_groups > 0) {
-#pragma unroll 1
-                    for (int c0 = 0; c0 < st.units; c0 += chunk_units) {
-                        const int cu_n = min(chunk_units, st.units - c0);
-                        if (!one_chunk || !staged) stage_chunk(c0, cu_n, c0 == 0);
-                        shared(c0, cu_n);
-                    }
-                    lds_barrier();                                        // the tail's row sums are complete
-                    tail_store();
                 }
               }
             } else if (!aborted) {
@@ -972,9 +827,10 @@ struct StreamKernel {
     static constexpr auto fn_tiled = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2>;
     static constexpr auto fn_single = gemv_stream_kernel<DT, BATCH, kArith, kThreads, true, false>;
     // reproducible sums
+    // the 16-bit arithmetic is reproducible as it is: the same instance
     static constexpr bool kHasDet = true;
-    static constexpr auto fn_det = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, false, kHasDet>;
-    static constexpr auto fn_tiled_det = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2, kHasDet>;
+    static constexpr auto fn_det = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, false, kArith == 2>;
+    static constexpr auto fn_tiled_det = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2, kArith == 2>;
 };
 
 template <int DT, int BATCH>

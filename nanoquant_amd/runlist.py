@@ -42,10 +42,10 @@ class DecodeRunList:
     def __init__(self, batch: int, dtype: torch.dtype = torch.float16, device=None, interleave: int = 2,
                  deterministic: bool = False):
         """`deterministic=True`: every launch of the list gives bit-identical outputs.  Up to batch 4 partial sums are
-        rounded to a grid on which additions are exact, at a small cost in precision; at batch 8 and 16 every row sum
-        is formed by one wavefront, at a small cost in balance.  By default the order in which the wavefronts of a
-        workgroup add up a row sum (batch 8 and 16: the left-over rows of a slice) is left to the hardware and the
-        last bit may differ from launch to launch."""
+        rounded to a grid on which additions are exact, at a small cost in precision; without it the order in which
+        the wavefronts of a workgroup add up a row sum is left to the hardware and the last bit may differ from launch
+        to launch.  At batch 8 and 16 one wavefront forms every row sum in a fixed order: launches repeat bit for bit
+        either way and the switch changes nothing."""
         if batch not in self.BATCHES:
             raise ValueError(f"run-list batch must be one of {self.BATCHES}, got {batch}")
         if dtype not in (torch.float16, torch.bfloat16):

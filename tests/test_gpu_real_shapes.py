@@ -57,7 +57,7 @@ def test_cfg1_layer_run_list_as_benchmarked(dev, batch):
         x = oracle.synth_x(batch, n, 1100 + i)
         vt_bits = packing.binary_packer(torch.from_numpy(vt_p), "half2")
         u_bits = packing.binary_packer(torch.from_numpy(u_p), "half2")
-        tiled = batch <= 4                                             # bench.py: tile order up to batch 4
+        tiled = batch != 8                           # tile order as in bench.py; batch 8 keeps row-major words covered
         if tiled:
             vt_dev, u_dev = packing.tile_words(vt_bits.to(dev)), packing.tile_words(u_bits.to(dev))
         else:

@@ -250,10 +250,11 @@ def test_tiled_factors_give_the_same_layer(dev, batch, dtype):
 @pytest.mark.parametrize("tiled", [False, True])
 @pytest.mark.parametrize("batch,dtype", [(16, torch.float16), (8, torch.float16), (16, torch.bfloat16)])
 def test_long_lists_on_the_16_bit_operands(dev, batch, dtype, tiled):
-    # Batch 8 and 16: a wavefront owns whole 16-row groups of a slice and keeps their row sums in registers, only the
-    # groups left over after the rounds of 16 are summed in LDS.  Short lists give every workgroup a few rows (all
-    # left-overs); here 64 linears with 2000 x 8192 first factors put about 500 rows of one stage on a workgroup (a
-    # whole round, a second one with rows missing, 15 groups left over in some) and make the input two chunks at batch 16.
+    # Batch 8 and 16: a wavefront owns whole 16-row groups of a slice and keeps their row sums in registers; in round r
+    # wavefront w has group 16 r + w.  Short lists give every workgroup a few rows (one round, most wavefronts idle);
+    # here 64 linears with 2000 x 8192 first factors put about 500 rows of one stage on a workgroup (a whole round, a
+    # second one that only some wavefronts take part in, a last group with rows missing) and make the input two chunks
+    # at batch 16.
     m, n, r, count = 520, 8192, 2000, 64
     checked = {0: 900, 31: 901, 63: 902}
     to = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev).to(dtype)
