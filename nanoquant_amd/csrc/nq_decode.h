@@ -328,6 +328,120 @@ __device__ __forceinline__ void stage_units(uint4* xs, float* xsum, const StageI
     else stage_units_vector<DT, BATCH, PM>(xs, xsum, xtot, st, c0, cu_n, upad, nthreads);
 }
 
+// Staging for the run-list kernel's 16-bit arithmetic (pair-major layout, unit totals to unit_tot[b * upad + cu]):
+// one lane takes the 8 columns of one 16-byte chunk for kRows batch rows.  The column scale is loaded once for all of
+// them, every load of a lane is in flight before the first is used (an input of 4096 columns at batch 16 is one round
+// trip to the memory side for the workgroup instead of two or three), and no index is divided.  A wavefront's 64
+// chunks belong to one half of the batch rows (the chunk count is padded to a multiple of 64).  Requires 16-byte
+// aligned rows and K % 8 == 0; everything else goes through stage_units.
+template <int DT, int BATCH, int THREADS>
+__device__ __forceinline__ void stage_units_rows(uint4* xs, float* unit_tot, const StageInput& st, int c0, int cu_n,
+                                                 int upad) {
+    if (!st.vec_in || (st.K & 7)) {
+        stage_units<DT, BATCH, true>(xs, unit_tot, st, c0, cu_n, upad, THREADS, nullptr);
+        return;
+    }
+    using E = Elem<DT>;
+    constexpr int kParts = BATCH >= 8 ? 2 : 1;
+    constexpr int kRows = BATCH / kParts;                    // batch rows per lane
+    constexpr int kRowsF32 = kRows > 4 ? 4 : kRows;          // fp32 input: two loads per row, half as many rows in flight
+    const int lane = threadIdx.x & 63;
+    const int nchunks = cu_n * 16;
+    const int npad = ((cu_n + 3) & ~3) * 16;
+    const int nitems = kParts * npad;
+    const uint32_t esize = st.in_f32 ? 4u : 2u;
+    const __amdgpu_buffer_rsrc_t rin = raw_buffer(st.in, (uint32_t)(((size_t)(BATCH - 1) * st.in_stride + st.K) * esize));
+    const bool scaled = !st.in_f32 && st.s_col != nullptr;
+    const __amdgpu_buffer_rsrc_t rsc = raw_buffer(scaled ? (const void*)st.s_col : st.in, scaled ? (uint32_t)st.K * 2u : 0u);
+    const uint32_t row_bytes = (uint32_t)st.in_stride * esize;
+    // the 8 rounded values r of chunk (b, q) and their unit total
+    auto put = [&](int b, int q, const uint32_t (&rp)[4], float tot) {
+        tot = group_sum(tot, 16);                            // the 16 chunks of a unit sit in 16 consecutive lanes
+        if (q < nchunks) {
+            store_chunk_packed<true>(xs, b, q & 15, upad, q >> 4, rp);
+            if ((q & 15) == 0) unit_tot[b * upad + (q >> 4)] = tot;
+        }
+    };
+    auto round_and_put = [&](int b, int q, const float (&v)[8]) {
+        uint32_t rp[4];
+        float tot = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            rp[e] = (uint32_t)E::from_float(v[2 * e]) | ((uint32_t)E::from_float(v[2 * e + 1]) << 16);
+            tot = E::dot2(rp[e], E::kOnePair, tot);          // the sum of what the dot products will actually see
+        }
+        put(b, q, rp, tot);
+    };
+#pragma unroll 1
+    for (int item = threadIdx.x; item - lane < nitems; item += THREADS) {     // wave-uniform trip count
+        const int part = (kParts > 1 && item - lane >= npad) ? 1 : 0;           // wave-uniform
+        const int q = item - part * npad, b0 = part * kRows;
+        const int col = c0 * 128 + 8 * q;
+        const bool live = q < nchunks && col < st.K;
+        const uint32_t off0 = (uint32_t)b0 * row_bytes + (uint32_t)col * esize;
+        if (!st.in_f32) {
+            const u32x4_t sc = __builtin_amdgcn_raw_buffer_load_b128(rsc, live ? (uint32_t)col * 2u : kPastEnd, 0, kCacheDefault);
+            u32x4_t raw[kRows];
+#pragma unroll
+            for (int j = 0; j < kRows; ++j)
+                raw[j] = __builtin_amdgcn_raw_buffer_load_b128(rin, live ? off0 + (uint32_t)j * row_bytes : kPastEnd, 0, kCacheDefault);
+#pragma unroll
+            for (int j = 0; j < kRows; ++j) {
+                if constexpr (DT == 0) {
+                    // packed products, rounded once to fp16 (the product of two fp16 numbers is exact in fp32), and their
+                    // sum with the packed dot product
+                    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+                    uint32_t rp[4];
+                    float tot = 0.f;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        half2_t xv = __builtin_bit_cast(half2_t, (uint32_t)raw[j][e]);
+                        if (scaled) xv = xv * __builtin_bit_cast(half2_t, (uint32_t)sc[e]);
+                        rp[e] = __builtin_bit_cast(uint32_t, xv);
+                        tot = __builtin_amdgcn_fdot2(xv, (half2_t){(_Float16)1.f, (_Float16)1.f}, tot, false);
+                    }
+                    put(b0 + j, q, rp, tot);
+                } else {
+                    float v[8];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t xw = raw[j][e], sw = scaled ? sc[e] : E::kOnePair;
+                        v[2 * e] = E::to_float(xw & 0xFFFFu) * E::to_float(sw & 0xFFFFu);
+                        v[2 * e + 1] = E::to_float(xw >> 16) * E::to_float(sw >> 16);
+                    }
+                    round_and_put(b0 + j, q, v);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j0 = 0; j0 < kRows; j0 += kRowsF32) {
+                u32x4_t ra[kRowsF32], rb[kRowsF32];
+#pragma unroll
+                for (int j = 0; j < kRowsF32; ++j) {
+                    const uint32_t off = live ? off0 + (uint32_t)(j0 + j) * row_bytes : kPastEnd;
+                    if (st.in_coherent) {
+                        ra[j] = __builtin_amdgcn_raw_buffer_load_b128(rin, off, 0, kCacheAgentCoherent);
+                        rb[j] = __builtin_amdgcn_raw_buffer_load_b128(rin, live ? off + 16u : kPastEnd, 0, kCacheAgentCoherent);
+                    } else {
+                        ra[j] = __builtin_amdgcn_raw_buffer_load_b128(rin, off, 0, kCacheDefault);
+                        rb[j] = __builtin_amdgcn_raw_buffer_load_b128(rin, live ? off + 16u : kPastEnd, 0, kCacheDefault);
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < kRowsF32; ++j) {
+                    float v[8];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        v[e] = as_float(ra[j][e]);
+                        v[4 + e] = as_float(rb[j][e]);
+                    }
+                    round_and_put(b0 + j0 + j, q, v);
+                }
+            }
+        }
+    }
+}
+
 // Signed sum over one unit for BATCH rows: out[b] = sum_{c in unit} sgn(bit c) * x[b][c].
 template <int DT, int BATCH>
 struct UnitDot;

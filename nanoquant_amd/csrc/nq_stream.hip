@@ -41,6 +41,7 @@ constexpr int kCounterStride = 8;              // 64-bit words between sub-count
 // in [g*members_k, (g+1)*members_k) for as long as the reading workgroup itself has not left, so
 // g = value / members_k needs no reset between launches and no atomic that returns a value; stage s
 // is complete in launch g when its sub-counters add up to (g+1) * seg_count(s).
+constexpr size_t kStreamShareBytes = 15 * 1024; // column shares of the 16-bit arithmetic: (1024 / 64 - 1) wavefronts x 64 lanes x 16 bytes
 constexpr int kQ8Depth = 3;                    // items (2 KB of packed words each) in flight per wavefront, fp4 x fp8 path
 constexpr int kStreamLdsMax = 160 * 1024 - 512;   // staged activations + row accumulators: the LDS of a CU less the static variables
 
@@ -397,7 +398,16 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                 constexpr int kAccs = Pow2<DT>::kClasses;
                 const int ngroups16 = (seg.row_end - seg.row_begin + 15) >> 4;
                 const int rounds = (ngroups16 + kWaves - 1) / kWaves;            // the same for every wavefront
-                const int my_rounds = ngroups16 > wave ? (ngroups16 - wave + kWaves - 1) / kWaves : 0;
+                // Few row groups (a short list gives a workgroup some tens of rows): the wavefronts that would have no
+                // group take shares of the columns instead.  Wavefront w works on group w % groups, share w / groups of
+                // every staged chunk; the shares of a group are added in share order by its first wavefront, through the
+                // memory of the staged input once everybody is done with it.
+                const bool split = rounds == 1 && 2 * ngroups16 <= kWaves;
+                const int nshares = split ? kWaves / ngroups16 : 1;
+                const int grp = split ? wave % ngroups16 : wave;                 // group of this wavefront in round 0
+                const int share = split ? wave / ngroups16 : 0;                  // >= nshares: nothing to do
+                const int my_rounds = split ? (share < nshares ? 1 : 0)
+                                            : (ngroups16 > wave ? (ngroups16 - wave + kWaves - 1) / kWaves : 0);
                 float4_t acc[kAccs];
 #pragma unroll
                 for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
@@ -460,11 +470,11 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                     }
                 };
                 // the q-th group of this wavefront is complete: acc[v] = sum for its row 4 g + v, batch row r16
-                auto store_group = [&](int q) __attribute__((always_inline)) {
-                    const float4_t sum = pow2_combine<DT>(acc) * -2.f;            // signed sum = (sum of x) - 2 (sum of b x)
+                auto store_group = [&](int q, const float4_t& bsum) __attribute__((always_inline)) {
+                    const float4_t sum = bsum * -2.f;                             // signed sum = (sum of x) - 2 (sum of b x)
                     if (r16 < BATCH) {
                         const float xt = xtot[r16];
-                        const int row0 = seg.row_begin + 16 * (wave + kWaves * q) + 4 * g;
+                        const int row0 = seg.row_begin + 16 * (grp + kWaves * q) + 4 * g;
                         if (row0 < seg.row_end) emit4(row0, r16, sum + xt);
                     }
                 };
@@ -477,9 +487,12 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                 // chunk is the last of the input.
                 auto run_items = [&](auto order_c, int q_begin, int q_end, int c0, int cu_n, bool complete) __attribute__((always_inline)) {
                     constexpr int kOrder = decltype(order_c)::value;      // one copy of the loop per word order: see load_unit
-                    const int ngroups = (cu_n + 3) >> 2;
+                    const int ngroups_all = (cu_n + 3) >> 2;
+                    const int j_begin = split ? share * ngroups_all / nshares : 0;        // this wavefront's unit groups
+                    const int ngroups = (split ? (share + 1) * ngroups_all / nshares : ngroups_all) - j_begin;
                     const int positions = (ngroups + 2) / 3 * 3;
-                    const int nq = max(min(q_end, my_rounds) - q_begin, 0);   // the last round has groups for some wavefronts only
+                    // the last round has groups for some wavefronts only, and a chunk may have fewer unit groups than shares
+                    const int nq = ngroups > 0 ? max(min(q_end, my_rounds) - q_begin, 0) : 0;
                     int f_left = nq * positions, f_q = q_begin, f_j = 0;  // fetch cursor
                     auto fetch = [&](uint4& w) {
                         if constexpr (kOrder == 1) {
@@ -487,22 +500,22 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                             // rows, chunks at multiples of 4 units), 16 bytes per lane; rows and units past the end are
                             // zero words
                             const bool ok = f_left > 0 && f_j < ngroups;
-                            const int half = (seg.row_begin >> 4) + wave + kWaves * f_q;
-                            const int off = ((half >> 1) * bv.groups + (c0 >> 2) + f_j) * 2048 + (half & 1) * 1024;
+                            const int half = (seg.row_begin >> 4) + grp + kWaves * f_q;
+                            const int off = ((half >> 1) * bv.groups + (c0 >> 2) + j_begin + f_j) * 2048 + (half & 1) * 1024;
                             const uint32_t soff = ok ? (uint32_t)__builtin_amdgcn_readfirstlane(off) : 0u;
                             const uint32_t voff = ok ? (uint32_t)lane * 16u : kPastEnd;
                             const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(bv.rsrc, voff, soff, 2 /* nt */);
                             w = make_uint4(a.x, a.y, a.z, a.w);
                         } else {
-                            const int u = 4 * f_j + g;
-                            const int row = seg.row_begin + 16 * (wave + kWaves * f_q) + r16;
+                            const int u = 4 * (j_begin + f_j) + g;
+                            const int row = seg.row_begin + 16 * (grp + kWaves * f_q) + r16;
                             w = load_unit<kOrder>(bv, min(row, st.rows - 1), c0 + u, f_left > 0 && u < cu_n);   // u < cu_n fails on empty positions as well
                         }
                         --f_left;
                         if (++f_j == positions) { f_j = 0; ++f_q; }
                     };
                     auto work = [&](uint4& w, int j) {
-                        const int u = 4 * j + g;
+                        const int u = 4 * (j_begin + j) + g;
                         if constexpr (kOrder == 2) trim_unit(bv, w, c0 + u);   // tile order pads with zero words
                         unit_mfma_pow2<DT, BATCH>(w, xs, upad, min(u, cu_n - 1), acc);   // w = 0 beyond cu_n
                     };
@@ -525,8 +538,8 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                             if (j + 2 < ngroups) work(w2, j + 2);
                             fetch(w2);
                         }
-                        if (complete) {
-                            store_group(q);
+                        if (complete && !split) {
+                            store_group(q, pow2_combine<DT>(acc));
 #pragma unroll
                             for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
                             __builtin_amdgcn_s_waitcnt(0);
@@ -543,13 +556,15 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                             lds_barrier();
                         }
                     }
-                    // unit totals to LDS, then one lane per batch row adds them in unit order
-                    stage_units<DT, BATCH, true>(xs, unit_tot, sin, c0, cu_n, upad, kStreamThreads, nullptr);
+                    // unit totals to LDS, then 16 lanes per batch row add them in a fixed order
+                    stage_units_rows<DT, BATCH, kStreamThreads>(xs, unit_tot, sin, c0, cu_n, upad);
                     lds_barrier();
-                    if (tid < BATCH) {
+                    if (tid < BATCH * 16) {                               // whole wavefronts
+                        const int b = tid >> 4, k = tid & 15;
                         float t = 0.f;
-                        for (int cu = 0; cu < cu_n; ++cu) t += unit_tot[tid * upad + cu];
-                        xtot[tid] += t;
+                        for (int cu = k; cu < cu_n; cu += 16) t += unit_tot[b * upad + cu];
+                        t = group_sum(t, 16);
+                        if (k == 0) xtot[b] += t;
                     }
                     staged = true;
                     lds_barrier();                                        // staged input and its totals visible
@@ -557,6 +572,17 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                 auto owned = [&](int q_begin, int q_end, int c0, int cu_n, bool complete) __attribute__((always_inline)) {
                     if (bv.groups) run_items(std::integral_constant<int, 1>{}, q_begin, q_end, c0, cu_n, complete);
                     else run_items(std::integral_constant<int, 2>{}, q_begin, q_end, c0, cu_n, complete);
+                    if (split && complete) {
+                        float4_t mine = pow2_combine<DT>(acc);
+                        float4_t* shares = (float4_t*)xs;                 // (kWaves - 1) x 64 x 16 bytes
+                        lds_barrier();                                    // every wavefront is done with the staged input
+                        if (share > 0 && share < nshares) shares[(wave - ngroups16) * 64 + lane] = mine;
+                        lds_barrier();
+                        if (share == 0) {
+                            for (int t = 1; t < nshares; ++t) mine += shares[(grp + (t - 1) * ngroups16) * 64 + lane];
+                            store_group(0, mine);
+                        }
+                    }
                 };
                 // an input of one chunk is staged once and every wavefront walks all its groups in one go
                 const int staged_rounds = one_chunk ? min(rounds, 1) : rounds;
@@ -796,7 +822,10 @@ static void stream_lds_plan(int batch, int arith, int max_units, int* chunk_cap_
     chunk_cap = (chunk_cap - 1) & ~3;   // whole 4-unit groups, and room for the odd pitch chunk_units | 1
     const int chunk_units = max_units < chunk_cap ? max_units : chunk_cap;
     *chunk_cap_out = chunk_cap;
-    *lds_out = (size_t)racc_bytes + (size_t)xs_chunks(batch, chunk_units | 1) * sizeof(uint4);
+    // the staged input's memory also takes the column shares of a slice of few rows: 1 KB per wavefront but the first
+    size_t xs_bytes = (size_t)xs_chunks(batch, chunk_units | 1) * sizeof(uint4);
+    if (xs_bytes < kStreamShareBytes) xs_bytes = kStreamShareBytes;
+    *lds_out = (size_t)racc_bytes + xs_bytes;
 }
 
 // Which arithmetic, by batch (measured on Llama-2-7B layers with row-major words: one launch per layer / 26 layers
