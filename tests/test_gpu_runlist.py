@@ -285,6 +285,38 @@ def test_long_lists_on_the_16_bit_operands(dev, batch, dtype, tiled):
             assert err < (1e-2 if dtype == torch.bfloat16 else 2e-3), (i, rep, err)
 
 
+@pytest.mark.parametrize("tiled", [False, True])
+@pytest.mark.parametrize("batch,dtype", [(16, torch.float16), (8, torch.bfloat16)])
+def test_column_shares_of_short_slices(dev, batch, dtype, tiled):
+    # Batch 8 and 16, one linear per launch: a workgroup gets a few 16-row groups of a stage, and the wavefronts
+    # without a group of their own take shares of the columns (added in a fixed order through LDS).  Shapes: an input
+    # of three staged chunks at batch 16 (11008 columns) with 40 rows per workgroup and fewer unit groups in the last
+    # chunk than shares; a rank that leaves a last group of 8 rows; an input shorter than one unit group.
+    to = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev).to(dtype)
+    f64 = lambda t: t.float().cpu().numpy().astype(np.float64)
+    words = (lambda w: packing.tile_words(w)) if tiled else (lambda w: w)
+    for k, (m, n, r) in enumerate([(4096, 11008, 1000), (520, 4096, 40), (64, 96, 32)]):
+        vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, 7700 + k)
+        vt_p, u_p, mid_p = oracle.pad_rank(vt, u, s_mid, 32)
+        pack = lambda w: words(packing.binary_packer(torch.from_numpy(w), "half2").to(dev))
+        x = to(oracle.synth_x(batch, n, 7800 + k))
+        sc = (to(s_in), to(mid_p), to(s_out))
+        rl = DecodeRunList(batch, dtype, dev)
+        rl.add(x, sc[0], pack(vt_p), sc[1], pack(u_p), sc[2], tiled=tiled)
+        print(f"column shares: batch {batch} {dtype} tiled={tiled} m={m} n={n} r={r}", flush=True)
+        first = None
+        for rep in range(3):
+            y = rl.run()[0]
+            torch.cuda.synchronize()
+            assert rl.status() == 0
+            if first is None:
+                first = y.clone()
+            assert torch.equal(y, first), rep                            # fixed order of the shares: bit for bit
+        ref = oracle.layer_forward(f64(x), vt, u, f64(sc[0]), f64(to(s_mid)), f64(sc[2]), dtype=np.float64)
+        err = oracle.max_rel_err(first.float().cpu().numpy(), ref)
+        assert err < (2e-2 if dtype == torch.bfloat16 else (TIGHT if r >= 256 else 1e-2)), (m, n, r, err)
+
+
 def test_tiled_factor_size_is_checked(dev):
     m, n, r = 64, 128, 32
     _, ops = _term(dev, m, n, r, seed=5)
@@ -457,15 +489,15 @@ def test_an_expired_wait_is_reported_and_the_list_stays_usable(dev):
         assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < 1e-2   # rank 40: the fp16-output budget
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(16))
 def test_random_lists_match_the_oracle(dev, seed):
     """Seeded random lists: batch, type, word order, reproducible sums, 1 to 4 linears of ragged shapes, some fed by
     the linear before them."""
     rng = np.random.default_rng(4200 + seed)
     batch = int(rng.choice([1, 2, 4, 8, 16]))
     dtype = torch.float16 if rng.random() < 0.6 else torch.bfloat16
-    tiled = bool(rng.random() < 0.5) and batch <= 4
-    det = bool(rng.random() < 0.3) and batch <= 4
+    tiled = bool(rng.random() < 0.5)
+    det = bool(rng.random() < 0.3)
     rl = DecodeRunList(batch, dtype, dev, deterministic=det)
     to = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev).to(dtype)
     f64 = lambda t: t.float().cpu().numpy().astype(np.float64)
