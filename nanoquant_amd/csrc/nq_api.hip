@@ -396,6 +396,15 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         {
             const long long fixed = batch == 1 ? 8800 : batch == 2 ? 6600 : batch == 4 ? 4400 : 2200;
             auto gran = [&](size_t k) { return table[ids[k]].tiled ? granule : 1; };
+            // Batch 8 and 16: an input too long to be staged at once is staged again, chunk by chunk, for every 256 rows
+            // of a slice (three barriers and a round trip to memory per chunk): charged as 10 more units per chunk and
+            // row, from per-workgroup time accounts of the Llama-2-7B stack (down projection, 86 units in 3 chunks
+            // at batch 16: without the charge its workgroups end 20 % behind the others).
+            const long long chunk_cap_long = std::max(1, nq::stream_chunk_cap(dtype, batch, max_units));
+            auto restage = [&](long long units) -> long long {
+                const long long chunks = (units + chunk_cap_long - 1) / chunk_cap_long;
+                return batch >= 8 && chunks > 1 ? 10 * chunks : 0;
+            };
             // fills workgroups with budget T; returns how many it needs (emits the slices when `emit`)
             auto fill = [&](long long T, bool emit) -> long long {
                 long long w = 0, budget = T;
@@ -403,7 +412,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
                 int row = 0;
                 while (k < ids.size()) {
                     const nq::RunStage& stg = table[ids[k]];
-                    const long long u = stg.units;
+                    const long long u = stg.units + restage(stg.units);
                     const int left = stg.rows - row;
                     const int g = gran(k);
                     const long long least = fixed + u * std::min<long long>(left, std::max<long long>(g, fixed / (4 * u)));
@@ -426,7 +435,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
                 }
                 return w + 1;
             };
-            long long lo = total / nwg, hi = total + (long long)ids.size() * fixed + 1;
+            long long lo = total / nwg, hi = 2 * total + (long long)ids.size() * fixed + 1;   // restage() adds at most 10 to chunk_cap + 1 units
             while (lo < hi) {
                 const long long mid = lo + (hi - lo) / 2;
                 if (fill(mid, false) <= nwg) hi = mid; else lo = mid + 1;
