@@ -135,12 +135,15 @@ def test_mixture_through_addend(dev):
     assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < TIGHT
 
 
-def test_bf16_and_ragged_shapes(dev):
-    rl = DecodeRunList(1, torch.bfloat16, dev)
+@pytest.mark.parametrize("batch", [1, 8, 16])
+def test_bf16_and_ragged_shapes(dev, batch):
+    # ranks 70 and 2985 and 4100 columns: intermediate rows that allow no 16-byte loads (element-wise staging at every
+    # batch size), inputs that end inside a unit, row counts that end inside a 16-row group
+    rl = DecodeRunList(batch, torch.bfloat16, dev)
     refs = []
     for i, (m, n, r) in enumerate([(100, 1000, 70), (33, 4100, 2985), (300, 96, 32)]):
         vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, 200 + i)
-        x = oracle.synth_x(1, n, 200 + i)
+        x = oracle.synth_x(batch, n, 200 + i)
         bf = lambda a: torch.from_numpy(a.astype(np.float32)).to(torch.bfloat16)
         xt, si, sm, so = bf(x), bf(s_in), bf(s_mid), bf(s_out)
         rl.add(xt.to(dev), si.to(dev), packing.binary_packer(torch.from_numpy(vt), "half2").to(dev), sm.to(dev),
@@ -151,7 +154,7 @@ def test_bf16_and_ragged_shapes(dev):
     torch.cuda.synchronize()
     assert rl.status() == 0
     for y, ref in zip(ys, refs):
-        assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < 1e-2
+        assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < (1e-2 if batch == 1 else 2e-2)   # bf16 staging from 8 rows on
 
 
 def test_graph_replay_of_a_run_list(dev):
