@@ -134,7 +134,9 @@ typedef struct nq_runlist_plan {
     int nlinears, nstages, nphases, workgroups, max_units, batch, dtype, index_words;
     int bound;              /* bit 0: some x was NULL, bit 1: some y was NULL (nq_runlist_run_bound must supply them);
                                bit 2: the linears are in tile order (up to batch 4 all linears of a list must agree);
-                               bit 3: reproducible sums (nq_runlist_set_deterministic) */
+                               bit 3: reproducible sums (nq_runlist_set_deterministic);
+                               bit 4: set by the builder for a short fp16 list at batch 4, which runs on the arithmetic of
+                               batch 8 and 16 (16-bit operands; reproducible with or without bit 3) */
     int spin_limit;         /* polls after which a dependency wait gives up and sets the status word; 0 (as built) =
                                the default of 2^21 polls, about a second.  The caller may lower it, e.g. to exercise
                                its handling of an expired wait: every kernel still runs to its end */
@@ -156,8 +158,9 @@ int nq_runlist_status(const void* workspace, int* status_out, void* stream);
  * the last bit between launches (the reference's reductions are ordered: kernel/cuda/gemv_kernel.cu:148-170,
  * shuffles inside one warp).  With this switch every launch of the plan gives bit-identical outputs.  Batch 1, 2 and
  * 4: partial sums are rounded to a grid on which their additions are exact; the results stay within the same
- * tolerance but lose up to 16 bits below (columns x largest input value).  Batch 8 and 16: every row sum is formed by
- * one wavefront in a fixed order whether the switch is on or off; it is accepted and selects the same kernel.
+ * tolerance but lose up to 16 bits below (columns x largest input value).  Batch 8 and 16, and plans with bit 4 of
+ * `bound` set: every row sum is formed by one wavefront in a fixed order whether the switch is on or off; it is
+ * accepted and selects the same kernel.
  * NQ_ERR_SHAPE for a batch size without a run-list kernel.  Sets bit 3 of plan->bound. */
 int nq_runlist_set_deterministic(nq_runlist_plan* plan, int on);
 

@@ -277,8 +277,21 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
     }
 
     // ---- grid = what the device keeps resident; every workgroup gets an equal share of every phase ----
+    // Which arithmetic: at batch 4 (fp16) a list with little work per workgroup (up to two Llama-2-7B layers on 256
+    // workgroups: 14000 rows x 16-byte units each) runs on the 16-bit arithmetic of batch 8 and 16, whose staging costs a
+    // tenth of the quantising one; longer lists stream faster on the fp4 x fp8 arithmetic (crossover measured at 2.6
+    // layers: 24 against 31 us for one layer per launch, 9.6 against 6.3 us per layer for 16).
+    bool alt = false;
+    if (nq::stream_has_alt(dtype, batch)) {
+        long long work = 0;
+        for (const auto& st : table) work += (long long)st.rows * st.units;
+        const int usual = nq::stream_capacity(dtype, batch, max_units, false);
+        if (usual <= 0) return NQ_ERR_HIP;
+        alt = work / usual <= 14000;
+    }
+    const bool wide = batch >= 8 || alt;                 // the 16-bit arithmetic and its cost model
     const int granule = nq::stream_row_granule(dtype, batch);
-    int nwg = nq::stream_capacity(dtype, batch, max_units);
+    int nwg = nq::stream_capacity(dtype, batch, max_units, alt);
     if (nwg <= 0) return NQ_ERR_HIP;
     if (nwg > kMaxResidentWorkgroups) nwg = kMaxResidentWorkgroups;
     std::vector<std::vector<int>> by_phase((size_t)nphases);
@@ -310,9 +323,9 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
             // of an input too long to be staged at once costs the latency of one more staging round trip
             // (2 us, 700 row units there).  The workgroup counts n_s minimise the slowest slice,
             // max_s (units_s * rows_s / n_s + fixed_s).
-            const double overhead_rows = batch >= 16 ? 64.0 : batch >= 8 ? 48.0 : 12.0;
-            const double pass_cost = batch >= 8 ? 700.0 : 0.0;
-            const int chunk_cap = std::max(1, nq::stream_chunk_cap(dtype, batch, max_units));
+            const double overhead_rows = batch >= 16 ? 64.0 : wide ? 48.0 : 12.0;
+            const double pass_cost = wide ? 700.0 : 0.0;
+            const int chunk_cap = std::max(1, nq::stream_chunk_cap(dtype, batch, max_units, alt));
             std::vector<double> fixed(ids.size(), 0.0);
             for (size_t k = 0; k < ids.size(); ++k) {
                 const int u = table[ids[k]].units;
@@ -394,16 +407,16 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         // fill (never starting a slice that cannot hold a quarter of the fixed part in arithmetic) needs at most
         // the resident workgroups.
         {
-            const long long fixed = batch == 1 ? 8800 : batch == 2 ? 6600 : batch == 4 ? 4400 : 2200;
+            const long long fixed = wide ? 2200 : batch == 1 ? 8800 : batch == 2 ? 6600 : 4400;
             auto gran = [&](size_t k) { return table[ids[k]].tiled ? granule : 1; };
             // Batch 8 and 16: an input too long to be staged at once is staged again, chunk by chunk, for every 256 rows
             // of a slice (three barriers and a round trip to memory per chunk): charged as 10 more units per chunk and
             // row, from per-workgroup time accounts of the Llama-2-7B stack (down projection, 86 units in 3 chunks
             // at batch 16: without the charge its workgroups end 20 % behind the others).
-            const long long chunk_cap_long = std::max(1, nq::stream_chunk_cap(dtype, batch, max_units));
+            const long long chunk_cap_long = std::max(1, nq::stream_chunk_cap(dtype, batch, max_units, alt));
             auto restage = [&](long long units) -> long long {
                 const long long chunks = (units + chunk_cap_long - 1) / chunk_cap_long;
-                return batch >= 8 && chunks > 1 ? 10 * chunks : 0;
+                return wide && chunks > 1 ? 10 * chunks : 0;
             };
             // fills workgroups with budget T; returns how many it needs (emits the slices when `emit`)
             auto fill = [&](long long T, bool emit) -> long long {
@@ -493,6 +506,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
     plan_out->spin_limit = 0;
     for (int i = 0; i < nlinears; ++i) plan_out->bound |= (linears[i].x ? 0 : 1) | (linears[i].y ? 0 : 2);
     if (linears[0].tiled) plan_out->bound |= 4;
+    if (alt) plan_out->bound |= 16;
     return hip_status(hipStreamSynchronize(hs));   // the tables are host memory: finish before they die
 }
 
@@ -516,7 +530,7 @@ int nq_runlist_run_bound(const void* workspace, const nq_runlist_plan* plan, con
                                       (unsigned long long*)(base + 256),
                                       (unsigned*)base, plan->workgroups, plan->max_units, (hipStream_t)stream, x, y,
                                       (plan->bound & 4) != 0, (plan->bound & 8) != 0,
-                                      plan->spin_limit > 0 ? (unsigned)plan->spin_limit : 0u));
+                                      plan->spin_limit > 0 ? (unsigned)plan->spin_limit : 0u, (plan->bound & 16) != 0));
 }
 
 int nq_runlist_set_deterministic(nq_runlist_plan* plan, int on) {

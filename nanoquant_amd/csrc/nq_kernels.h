@@ -52,14 +52,17 @@ struct RunSlice {
     RunStage st;
 };
 size_t stream_counter_bytes(int nstages);
-int stream_capacity(int dtype, int batch, int max_units);
-int stream_chunk_cap(int dtype, int batch, int max_units);
+// alt: the 16-bit arithmetic instead of the batch size's usual one, where stream_has_alt(dtype, batch)
+int stream_capacity(int dtype, int batch, int max_units, bool alt = false);
+int stream_chunk_cap(int dtype, int batch, int max_units, bool alt = false);
 int stream_row_granule(int dtype, int batch);
 hipError_t gemv_stream(int dtype, int batch, int nstages, const RunSlice* slices, unsigned long long* counters,
                        unsigned* status, int nwg, int max_units, hipStream_t stream, const void* ext_in = nullptr,
-                       void* ext_out = nullptr, bool tiled = false, bool det = false, unsigned spin_limit = 0);
-bool stream_needs_uniform_order(int dtype, int batch);
+                       void* ext_out = nullptr, bool tiled = false, bool det = false, unsigned spin_limit = 0,
+                       bool alt = false);
+bool stream_needs_uniform_order(int dtype, int batch, bool alt = false);
 bool stream_has_deterministic(int dtype, int batch);
+bool stream_has_alt(int dtype, int batch);
 
 // One stage on its own through the run-list kernel (no tables, no counters); batch 16 only.
 hipError_t gemv_stream_single(int dtype, int batch, const RunStage& st, hipStream_t stream);

@@ -848,9 +848,17 @@ static void stream_lds_plan(int batch, int arith, int max_units, int* chunk_cap_
 #define NQ_STREAM_THREADS(DT, BATCH) 1024
 #endif
 
-template <int DT, int BATCH>
+// Short lists at batch 4 run faster on the 16-bit arithmetic (one Llama-2-7B layer per launch: 24 against 31 us; its
+// staging is a tenth of the quantising one), long ones on the fp4 x fp8 arithmetic (16 layers per launch: 6.3 against
+// 9.6 us per layer): the builder picks per list (`alt`).  At batch 1 and 2 the fp4 x fp8 arithmetic wins or ties
+// everywhere (19 against 22, 22.5 against 22.3 us for one layer).  fp16 only: the 16-bit arithmetic rounds x * s_in and
+// the intermediate vector to the activation type, which costs bf16 lists a factor of eight in accuracy (2.3e-3 against
+// 3e-4 of the output maximum) where the fp4 x fp8 pieces are as exact for bf16 as for fp16.
+constexpr bool stream_alt_exists(int dtype, int batch) { return dtype == 0 && batch == 4; }
+
+template <int DT, int BATCH, int ARITH = NQ_STREAM_ARITH(DT, BATCH)>
 struct StreamKernel {
-    static constexpr int kArith = NQ_STREAM_ARITH(DT, BATCH);
+    static constexpr int kArith = ARITH;
     static constexpr int kThreads = NQ_STREAM_THREADS(DT, BATCH);
     static constexpr auto fn = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, false>;
     static constexpr auto fn_tiled = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2>;
@@ -862,21 +870,22 @@ struct StreamKernel {
     static constexpr auto fn_tiled_det = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2, kArith == 2>;
 };
 
-template <int DT, int BATCH>
+template <int DT, int BATCH, int ARITH>
 static hipError_t prepare_kernel(size_t lds) {
+    using SK = StreamKernel<DT, BATCH, ARITH>;
     static PerDeviceFlag attr_done;              // per template instance and device
     const int dev = current_device();
     if (lds > 64 * 1024 && !attr_done.test(dev)) {
-        hipError_t e = hipFuncSetAttribute((const void*)StreamKernel<DT, BATCH>::fn,
+        hipError_t e = hipFuncSetAttribute((const void*)SK::fn,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
         if (e != hipSuccess) return e;
-        e = hipFuncSetAttribute((const void*)StreamKernel<DT, BATCH>::fn_tiled,
+        e = hipFuncSetAttribute((const void*)SK::fn_tiled,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
         if (e != hipSuccess) return e;
-        e = hipFuncSetAttribute((const void*)StreamKernel<DT, BATCH>::fn_det,
+        e = hipFuncSetAttribute((const void*)SK::fn_det,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
         if (e != hipSuccess) return e;
-        e = hipFuncSetAttribute((const void*)StreamKernel<DT, BATCH>::fn_tiled_det,
+        e = hipFuncSetAttribute((const void*)SK::fn_tiled_det,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
         if (e != hipSuccess) return e;
         attr_done.set(dev);
@@ -884,32 +893,32 @@ static hipError_t prepare_kernel(size_t lds) {
     return hipSuccess;
 }
 
-template <int DT, int BATCH>
+template <int DT, int BATCH, int ARITH>
 static int capacity_of(int max_units) {
+    using SK = StreamKernel<DT, BATCH, ARITH>;
     int chunk_cap;
     size_t lds;
-    stream_lds_plan(BATCH, StreamKernel<DT, BATCH>::kArith, max_units, &chunk_cap, &lds);
-    if (prepare_kernel<DT, BATCH>(lds) != hipSuccess) return 0;
+    stream_lds_plan(BATCH, ARITH, max_units, &chunk_cap, &lds);
+    if (prepare_kernel<DT, BATCH, ARITH>(lds) != hipSuccess) return 0;
     int per_cu = 0, dev = 0, cus = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)StreamKernel<DT, BATCH>::fn, StreamKernel<DT, BATCH>::kThreads,
-                                                     lds) != hipSuccess)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)SK::fn, SK::kThreads, lds) != hipSuccess)
         return 0;
     if (hipGetDevice(&dev) != hipSuccess) return 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
     return per_cu * cus;
 }
 
-template <int DT, int BATCH>
+template <int DT, int BATCH, int ARITH>
 static hipError_t launch_stream(int nstages, const RunSlice* slices, unsigned long long* counters, unsigned* status, int nwg,
                                 int max_units, hipStream_t stream, const void* ext_in, void* ext_out, bool tiled, bool det,
                                 unsigned spin_limit) {
-    using SK = StreamKernel<DT, BATCH>;
+    using SK = StreamKernel<DT, BATCH, ARITH>;
     if (spin_limit == 0) spin_limit = 1u << 21;                  // about a second of polling
     if (det && !SK::kHasDet) return hipErrorInvalidValue;
     int chunk_cap;
     size_t lds;
     stream_lds_plan(BATCH, SK::kArith, max_units, &chunk_cap, &lds, det);
-    hipError_t e = prepare_kernel<DT, BATCH>(lds);
+    hipError_t e = prepare_kernel<DT, BATCH, ARITH>(lds);
     if (e != hipSuccess) return e;
     if (det)
         hipLaunchKernelGGL((tiled ? SK::fn_tiled_det : SK::fn_det), dim3(nwg), dim3(SK::kThreads), lds, stream, nstages, slices,
@@ -969,37 +978,39 @@ hipError_t gemv_stream_single(int dtype, int batch, const RunStage& st, hipStrea
     return dtype == 0 ? launch_single<0, 16>(st, stream) : launch_single<1, 16>(st, stream);
 }
 
-#define NQ_STREAM_DISPATCH(CALL)                                          \
-    switch (batch) {                                                      \
-        case 1: return dtype == 0 ? CALL(0, 1) : CALL(1, 1);              \
-        case 2: return dtype == 0 ? CALL(0, 2) : CALL(1, 2);              \
-        case 4: return dtype == 0 ? CALL(0, 4) : CALL(1, 4);              \
-        case 8: return dtype == 0 ? CALL(0, 8) : CALL(1, 8);              \
-        case 16: return dtype == 0 ? CALL(0, 16) : CALL(1, 16);           \
-        default: break;                                                   \
+// CALL(dtype, batch, arithmetic); `alt` selects the 16-bit arithmetic where the batch size has both
+#define NQ_STREAM_DISPATCH(CALL)                                                                  \
+    if (alt && batch == 4 && dtype == 0) return CALL(0, 4, 1);                                    \
+    switch (batch) {                                                                              \
+        case 1: return dtype == 0 ? CALL(0, 1, NQ_STREAM_ARITH(0, 1)) : CALL(1, 1, NQ_STREAM_ARITH(1, 1));      \
+        case 2: return dtype == 0 ? CALL(0, 2, NQ_STREAM_ARITH(0, 2)) : CALL(1, 2, NQ_STREAM_ARITH(1, 2));      \
+        case 4: return dtype == 0 ? CALL(0, 4, NQ_STREAM_ARITH(0, 4)) : CALL(1, 4, NQ_STREAM_ARITH(1, 4));      \
+        case 8: return dtype == 0 ? CALL(0, 8, NQ_STREAM_ARITH(0, 8)) : CALL(1, 8, NQ_STREAM_ARITH(1, 8));      \
+        case 16: return dtype == 0 ? CALL(0, 16, NQ_STREAM_ARITH(0, 16)) : CALL(1, 16, NQ_STREAM_ARITH(1, 16)); \
+        default: break;                                                                           \
     }
 
 // Number of workgroups the device keeps resident for this kernel variant (0 on error).
-int stream_capacity(int dtype, int batch, int max_units) {
-#define NQ_CAP(D, B) capacity_of<D, B>(max_units)
+int stream_capacity(int dtype, int batch, int max_units, bool alt) {
+#define NQ_CAP(D, B, A) capacity_of<D, B, A>(max_units)
     NQ_STREAM_DISPATCH(NQ_CAP)
 #undef NQ_CAP
     return 0;
 }
 
 // Units of an input vector that are staged at once (longer inputs take several passes over the rows of a slice).
-int stream_chunk_cap(int dtype, int batch, int max_units) {
+int stream_chunk_cap(int dtype, int batch, int max_units, bool alt) {
     int cap = 0;
     size_t lds = 0;
-#define NQ_CHUNK(D, B) (stream_lds_plan(B, StreamKernel<D, B>::kArith, max_units, &cap, &lds), cap)
+#define NQ_CHUNK(D, B, A) (stream_lds_plan(B, A, max_units, &cap, &lds), cap)
     NQ_STREAM_DISPATCH(NQ_CHUNK)
 #undef NQ_CHUNK
     return 0;
 }
 
 // The fp4 x fp8 arithmetic has one kernel per word order: all stages of such a list must agree.
-bool stream_needs_uniform_order(int dtype, int batch) {
-#define NQ_UNI(D, B) (StreamKernel<D, B>::kArith == 2)
+bool stream_needs_uniform_order(int dtype, int batch, bool alt) {
+#define NQ_UNI(D, B, A) (A == 2)
     NQ_STREAM_DISPATCH(NQ_UNI)
 #undef NQ_UNI
     return false;
@@ -1007,7 +1018,8 @@ bool stream_needs_uniform_order(int dtype, int batch) {
 
 // Rows that one wave-load spans: slices of tile-order stages are cut at multiples of it.
 int stream_row_granule(int dtype, int batch) {
-#define NQ_GRAN(D, B) 32
+    const bool alt = false;
+#define NQ_GRAN(D, B, A) 32
     NQ_STREAM_DISPATCH(NQ_GRAN)
 #undef NQ_GRAN
     return 32;
@@ -1015,7 +1027,8 @@ int stream_row_granule(int dtype, int batch) {
 
 // Reproducible sums exist for every batch size that has a run-list kernel.
 bool stream_has_deterministic(int dtype, int batch) {
-#define NQ_DET(D, B) (StreamKernel<D, B>::kHasDet)
+    const bool alt = false;
+#define NQ_DET(D, B, A) (StreamKernel<D, B, A>::kHasDet)
     NQ_STREAM_DISPATCH(NQ_DET)
 #undef NQ_DET
     return false;
@@ -1023,11 +1036,13 @@ bool stream_has_deterministic(int dtype, int batch) {
 
 hipError_t gemv_stream(int dtype, int batch, int nstages, const RunSlice* slices, unsigned long long* counters,
                        unsigned* status, int nwg, int max_units, hipStream_t stream, const void* ext_in, void* ext_out,
-                       bool tiled, bool det, unsigned spin_limit) {
-#define NQ_RUN(D, B) launch_stream<D, B>(nstages, slices, counters, status, nwg, max_units, stream, ext_in, ext_out, tiled, det, spin_limit)
+                       bool tiled, bool det, unsigned spin_limit, bool alt) {
+#define NQ_RUN(D, B, A) launch_stream<D, B, A>(nstages, slices, counters, status, nwg, max_units, stream, ext_in, ext_out, tiled, det, spin_limit)
     NQ_STREAM_DISPATCH(NQ_RUN)
 #undef NQ_RUN
     return hipErrorInvalidValue;
 }
+
+bool stream_has_alt(int dtype, int batch) { return stream_alt_exists(dtype, batch); }
 
 }  // namespace nq

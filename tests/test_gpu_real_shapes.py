@@ -57,7 +57,7 @@ def test_cfg1_layer_run_list_as_benchmarked(dev, batch):
         x = oracle.synth_x(batch, n, 1100 + i)
         vt_bits = packing.binary_packer(torch.from_numpy(vt_p), "half2")
         u_bits = packing.binary_packer(torch.from_numpy(u_p), "half2")
-        tiled = batch != 8                           # tile order as in bench.py; batch 8 keeps row-major words covered
+        tiled = True                                                   # tile order, as in bench.py
         if tiled:
             vt_dev, u_dev = packing.tile_words(vt_bits.to(dev)), packing.tile_words(u_bits.to(dev))
         else:
@@ -76,9 +76,10 @@ def test_cfg1_layer_run_list_as_benchmarked(dev, batch):
             if rep == 0:
                 print(f"  {name}: max_rel_err {e:.2e}, element-wise (floor 0.1 rms) {ee:.2e}", flush=True)
             assert e < 1e-3, (name, batch, rep, e)
-            # fp16 outputs cost 2^-11 of the element by themselves; the 16-bit arithmetic (more than 4 rows) also rounds
-            # x * s_in and the intermediate vector to fp16, as the reference's kernels do
-            assert ee < (5e-3 if batch <= 4 else 5e-2), (name, batch, rep, ee)
+            # fp16 outputs cost 2^-11 of the element by themselves; the 16-bit arithmetic (more than 4 rows, and a list
+            # as short as this one at 4 rows) also rounds x * s_in and the intermediate vector to fp16, as the
+            # reference's kernels do
+            assert ee < (5e-3 if batch <= 2 else 5e-2), (name, batch, rep, ee)
 
 
 # ---- cfg2 --------------------------------------------------------------------------------------------

@@ -320,6 +320,36 @@ def test_column_shares_of_short_slices(dev, batch, dtype, tiled):
         assert err < (2e-2 if dtype == torch.bfloat16 else (TIGHT if r >= 256 else 1e-2)), (m, n, r, err)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_batch_4_lists_choose_their_arithmetic_by_length(dev, dtype):
+    # fp16 at batch 4: a list with little work per workgroup runs on the 16-bit arithmetic (bit 4 of the plan's flag
+    # word), a long one on the fp4 x fp8 arithmetic; bf16 lists always on the latter.  Both against the oracle.
+    to = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev).to(dtype)
+    f64 = lambda t: t.float().cpu().numpy().astype(np.float64)
+    m, n, r = 520, 8192, 2000
+    for count in (1, 64):
+        rl = DecodeRunList(4, dtype, dev)
+        checked = {}
+        for i in range(count):
+            vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, 8100 + (i if i in (0, count - 1) else 1))
+            vt_p, u_p, mid_p = oracle.pad_rank(vt, u, s_mid, 32)
+            pack = lambda w: packing.tile_words(packing.binary_packer(torch.from_numpy(w), "half2").to(dev))
+            x = to(oracle.synth_x(4, n, 8200 + i))
+            sc = (to(s_in), to(mid_p), to(s_out))
+            rl.add(x, sc[0], pack(vt_p), sc[1], pack(u_p), sc[2], tiled=True)
+            if i in (0, count - 1):
+                checked[i] = oracle.layer_forward(f64(x), vt, u, f64(sc[0]), f64(to(s_mid)), f64(sc[2]), dtype=np.float64)
+        ys = rl.run()
+        torch.cuda.synchronize()
+        assert rl.status() == 0
+        short = bool(rl._plan.bound & 16)
+        print(f"batch 4 {dtype} list of {count}: 16-bit arithmetic = {short}", flush=True)
+        assert short == (count == 1 and dtype == torch.float16)
+        for i, ref in checked.items():
+            err = oracle.max_rel_err(ys[i].float().cpu().numpy(), ref)
+            assert err < (1e-2 if dtype == torch.bfloat16 else TIGHT), (count, i, err)
+
+
 def test_tiled_factor_size_is_checked(dev):
     m, n, r = 64, 128, 32
     _, ops = _term(dev, m, n, r, seed=5)
