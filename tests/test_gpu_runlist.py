@@ -348,6 +348,21 @@ def test_batch_4_lists_choose_their_arithmetic_by_length(dev, dtype):
         for i, ref in checked.items():
             err = oracle.max_rel_err(ys[i].float().cpu().numpy(), ref)
             assert err < (1e-2 if dtype == torch.bfloat16 else TIGHT), (count, i, err)
+    # a short list whose input is longer than what is staged at once at 4 rows (28672 columns, two chunks on the 16-bit
+    # arithmetic) and whose rows end inside a 16-row group
+    m, n, r = 100, 28672, 256
+    vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, 8300)
+    x = to(oracle.synth_x(4, n, 8301))
+    sc = (to(s_in), to(s_mid), to(s_out))
+    pack = lambda w: packing.binary_packer(torch.from_numpy(w), "half2").to(dev)
+    rl = DecodeRunList(4, dtype, dev)
+    rl.add(x, sc[0], pack(vt), sc[1], pack(u), sc[2])
+    y = rl.run()[0]
+    torch.cuda.synchronize()
+    assert rl.status() == 0
+    ref = oracle.layer_forward(f64(x), vt, u, f64(sc[0]), f64(sc[1]), f64(sc[2]), dtype=np.float64)
+    err = oracle.max_rel_err(y.float().cpu().numpy(), ref)
+    assert err < (1e-2 if dtype == torch.bfloat16 else TIGHT), err
 
 
 def test_tiled_factor_size_is_checked(dev):
