@@ -290,6 +290,15 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         alt = work / usual <= 14000;
     }
     const bool wide = batch >= 8 || alt;                 // the 16-bit arithmetic and its cost model
+    // fp4 x fp8 arithmetic with wavefronts that own row pairs (tile order only; the launch falls back where it does not
+    // apply): always at batch 4, from about six Llama-2-7B layers per launch on at batch 2 (40000 rows x units per
+    // workgroup), where a slice has more row pairs than the workgroup has wavefronts
+    bool own = false;
+    if (!alt && (batch == 4 || batch == 2)) {
+        long long work = 0;
+        for (const auto& st : table) work += (long long)st.rows * st.units;
+        own = batch == 4 || work / std::max(1, nq::stream_capacity(dtype, batch, max_units, false)) >= 40000;
+    }
     const int granule = nq::stream_row_granule(dtype, batch);
     int nwg = nq::stream_capacity(dtype, batch, max_units, alt);
     if (nwg <= 0) return NQ_ERR_HIP;
@@ -507,6 +516,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
     for (int i = 0; i < nlinears; ++i) plan_out->bound |= (linears[i].x ? 0 : 1) | (linears[i].y ? 0 : 2);
     if (linears[0].tiled) plan_out->bound |= 4;
     if (alt) plan_out->bound |= 16;
+    if (own) plan_out->bound |= 32;
     return hip_status(hipStreamSynchronize(hs));   // the tables are host memory: finish before they die
 }
 
@@ -530,7 +540,8 @@ int nq_runlist_run_bound(const void* workspace, const nq_runlist_plan* plan, con
                                       (unsigned long long*)(base + 256),
                                       (unsigned*)base, plan->workgroups, plan->max_units, (hipStream_t)stream, x, y,
                                       (plan->bound & 4) != 0, (plan->bound & 8) != 0,
-                                      plan->spin_limit > 0 ? (unsigned)plan->spin_limit : 0u, (plan->bound & 16) != 0));
+                                      plan->spin_limit > 0 ? (unsigned)plan->spin_limit : 0u, (plan->bound & 16) != 0,
+                                      (plan->bound & 32) != 0));
 }
 
 int nq_runlist_set_deterministic(nq_runlist_plan* plan, int on) {

@@ -52,14 +52,16 @@ struct RunSlice {
     RunStage st;
 };
 size_t stream_counter_bytes(int nstages);
-// alt: the 16-bit arithmetic instead of the batch size's usual one, where stream_has_alt(dtype, batch)
+// alt: the 16-bit arithmetic instead of the batch size's usual one, where stream_has_alt(dtype, batch);
+// own: the fp4 x fp8 kernel whose wavefronts own row pairs, where it exists (tile order, batch 2 and 4, no reproducible
+// sums, every input staged in one chunk; ignored otherwise)
 int stream_capacity(int dtype, int batch, int max_units, bool alt = false);
 int stream_chunk_cap(int dtype, int batch, int max_units, bool alt = false);
 int stream_row_granule(int dtype, int batch);
 hipError_t gemv_stream(int dtype, int batch, int nstages, const RunSlice* slices, unsigned long long* counters,
                        unsigned* status, int nwg, int max_units, hipStream_t stream, const void* ext_in = nullptr,
                        void* ext_out = nullptr, bool tiled = false, bool det = false, unsigned spin_limit = 0,
-                       bool alt = false);
+                       bool alt = false, bool own = false);
 bool stream_needs_uniform_order(int dtype, int batch, bool alt = false);
 bool stream_has_deterministic(int dtype, int batch);
 bool stream_has_alt(int dtype, int batch);

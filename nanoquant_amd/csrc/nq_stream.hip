@@ -121,7 +121,12 @@ __host__ __device__ __forceinline__ int mfma_items_per_wave(int nitems, int wave
 // the other.  Costs up to 16 bits below that bound in precision, two barriers per chunk of a long input, 4 KiB of LDS.
 // TILED (fp4 x fp8 arithmetic only): every stage of the list has its words in tile order; the 16-bit arithmetic reads
 // either order, stage by stage.
-template <int DT, int BATCH, int ARITH, int THREADS, bool SINGLE, bool TILED, bool DET = false>
+// OWN (fp4 x fp8 arithmetic in tile order, every input staged in one chunk): a wavefront owns whole row pairs (32 rows)
+// of a slice and walks all their columns, so the row sums stay in its MFMA accumulators and go from there to the output:
+// no row sums in LDS, no LDS atomics, no barrier and no epilogue pass per row block.  The first pair of wavefront w is
+// pair w; every further one comes from a counter in LDS, so a wavefront that is served faster takes more pairs (the
+// four wavefronts of a SIMD are served oldest first; with equal shares the oldest waits 40 % of every pass).
+template <int DT, int BATCH, int ARITH, int THREADS, bool SINGLE, bool TILED, bool DET = false, bool OWN = false>
 __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const RunSlice* __restrict__ slices,
                                                                      unsigned long long* counters, unsigned* status,
                                                                      unsigned spin_limit, int chunk_cap,
@@ -134,6 +139,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
     extern __shared__ uint4 lds_raw[];
     static_assert(ARITH == 1 || ARITH == 2, "unknown arithmetic");
     constexpr bool kQ8 = ARITH == 2;
+    static_assert(!OWN || (kQ8 && TILED && !SINGLE && !DET), "owned row pairs exist for the tile-order fp4 x fp8 kernel only");
     constexpr bool kTotals = true;                              // both arithmetics: signed sum = (sum of x) - 2 (sum of b x)
     static_assert(!kQ8 || BATCH * kQ8Pieces <= 16, "pieces of all batch rows must fit the 16 operand columns");
     constexpr int kRaccFloats = kQ8 ? kRowBlock * BATCH : kUnitTotalsBytes / (int)sizeof(float);   // 16-bit arithmetic: the unit totals
@@ -146,6 +152,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
     uint32_t* ebmax_base = (uint32_t*)(xtot_base + 2 * kTotStride);   // DET: [2] largest unit exponent of the staged input
     uint4* xs_base = lds_raw + stream_head_bytes(BATCH, ARITH, DET) / sizeof(uint4);
     __shared__ int s_flag;
+    __shared__ int s_pair;                                      // OWN: the next row pair of the slice that nobody has taken
     const int tid = threadIdx.x;
     const int wg = blockIdx.x;
     if (tid == 0) s_flag = 0;
@@ -329,7 +336,9 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                 // dependency wait and the staging of the input (in tile order: unless the previous pass already did),
                 // and arrive while those run.  (Sending them out behind the first input loads of a slice that waits for
                 // nothing, so that the input does not queue behind them, gained 0.3 of 20 us per one-layer launch.)
-                if constexpr (TILED) {
+                if constexpr (OWN) {
+                    // the first fetches are sent out after the staging
+                } else if constexpr (TILED) {
                     if (!aborted) q_enter(seg.row_begin, 0);
                 } else {
                     q_setup(seg.row_begin, 0);
@@ -376,9 +385,70 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
             }
             lds_barrier();                                       // s_flag; previous slice is done with xs / racc
             aborted = aborted || (s_flag != 0);
+            // pairs 0 .. kWaves - 1 are the wavefronts' first ones; nobody takes a pair of the previous slice any more,
+            // and the barrier behind the staging comes before the first one of this slice is taken
+            if (OWN && tid == 0) s_pair = kWaves;
             if (tid < kTotStride) xtot_other[tid] = 0.f;         // every reader of it (the previous slice) is past the barrier
             if (DET && kQ8 && tid == 0) ebmax_base[slice_count & 1] = 0u;   // slice_count was advanced: this is the other one
 
+            // rows row0 .. row0 + 3 of batch row b: row scale, bias, addend, store (as the epilogue of the row-block
+            // loop).  The four rows of a lane are consecutive: 8-byte accesses where the alignment allows them.
+            const bool vec_rows = (seg.row_begin & 3) == 0 && (st.out_stride & 3) == 0 &&
+                                  ((((uintptr_t)st.s_row) | ((uintptr_t)st.bias) | ((uintptr_t)st.out)) & 7u) == 0;
+            auto emit4 = [&](int row0, int b, float4_t v4) __attribute__((always_inline)) {
+                float v[4] = {v4[0], v4[1], v4[2], v4[3]};   // scalars: a device-scope atomic store of a vector element stored element 0 four times
+                const size_t o = (size_t)b * st.out_stride + row0;
+                if (vec_rows && row0 + 3 < seg.row_end) {
+                    if (st.s_row) {
+                        const uint2 sw = *(const uint2*)(st.s_row + row0);
+                        v[0] *= E::to_float((uint16_t)(sw.x & 0xFFFFu)); v[1] *= E::to_float((uint16_t)(sw.x >> 16));
+                        v[2] *= E::to_float((uint16_t)(sw.y & 0xFFFFu)); v[3] *= E::to_float((uint16_t)(sw.y >> 16));
+                    }
+                    if (st.bias) {
+                        const uint2 bw = *(const uint2*)(st.bias + row0);
+                        v[0] += E::to_float((uint16_t)(bw.x & 0xFFFFu)); v[1] += E::to_float((uint16_t)(bw.x >> 16));
+                        v[2] += E::to_float((uint16_t)(bw.y & 0xFFFFu)); v[3] += E::to_float((uint16_t)(bw.y >> 16));
+                    }
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        if (row0 + k >= seg.row_end) break;
+                        if (st.s_row) v[k] *= E::to_float(st.s_row[row0 + k]);
+                        if (st.bias) v[k] += E::to_float(st.bias[row0 + k]);
+                    }
+                }
+                if (st.addend) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        if (row0 + k >= seg.row_end) break;
+                        if (st.dep2 >= 0)
+                            v[k] += __builtin_bit_cast(float, __hip_atomic_load((const uint32_t*)st.addend + o + k, __ATOMIC_RELAXED,
+                                                                                __HIP_MEMORY_SCOPE_AGENT));
+                        else
+                            v[k] += st.addend[o + k];
+                    }
+                }
+                if (!st.out_f32 && vec_rows && row0 + 3 < seg.row_end) {
+                    uint2 pk;
+                    pk.x = (uint32_t)E::from_float_clamped(v[0]) | ((uint32_t)E::from_float_clamped(v[1]) << 16);
+                    pk.y = (uint32_t)E::from_float_clamped(v[2]) | ((uint32_t)E::from_float_clamped(v[3]) << 16);
+                    *(uint2*)((uint16_t*)st.out + o) = pk;
+                    return;
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    if (row0 + k >= seg.row_end) break;
+                    if (st.out_f32) {
+                        // fp32 results (h, partial sums over terms) may be read by other workgroups of this launch:
+                        // device-coherent store, completed before the counter of the slice is bumped
+                        if (st.signal) __hip_atomic_store((uint32_t*)st.out + o + k, __builtin_bit_cast(uint32_t, v[k]),
+                                                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        else ((float*)st.out)[o + k] = v[k];
+                    } else {
+                        ((uint16_t*)st.out)[o + k] = E::from_float_clamped(v[k]);
+                    }
+                }
+            };
             if constexpr (!kQ8) {
               if (!aborted) {
                 // ---- 16-bit MFMA arithmetic (batch 8 and 16): wavefronts own whole row groups ----
@@ -411,64 +481,6 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                 float4_t acc[kAccs];
 #pragma unroll
                 for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
-                // rows row0 .. row0 + 3 of batch row b: row scale, bias, addend, store (as the epilogue of the row-block
-                // loop).  The four rows of a lane are consecutive: 8-byte accesses where the alignment allows them.
-                const bool vec_rows = (seg.row_begin & 3) == 0 && (st.out_stride & 3) == 0 &&
-                                      ((((uintptr_t)st.s_row) | ((uintptr_t)st.bias) | ((uintptr_t)st.out)) & 7u) == 0;
-                auto emit4 = [&](int row0, int b, float4_t v4) __attribute__((always_inline)) {
-                    float v[4] = {v4[0], v4[1], v4[2], v4[3]};   // scalars: a device-scope atomic store of a vector element stored element 0 four times
-                    const size_t o = (size_t)b * st.out_stride + row0;
-                    if (vec_rows && row0 + 3 < seg.row_end) {
-                        if (st.s_row) {
-                            const uint2 sw = *(const uint2*)(st.s_row + row0);
-                            v[0] *= E::to_float((uint16_t)(sw.x & 0xFFFFu)); v[1] *= E::to_float((uint16_t)(sw.x >> 16));
-                            v[2] *= E::to_float((uint16_t)(sw.y & 0xFFFFu)); v[3] *= E::to_float((uint16_t)(sw.y >> 16));
-                        }
-                        if (st.bias) {
-                            const uint2 bw = *(const uint2*)(st.bias + row0);
-                            v[0] += E::to_float((uint16_t)(bw.x & 0xFFFFu)); v[1] += E::to_float((uint16_t)(bw.x >> 16));
-                            v[2] += E::to_float((uint16_t)(bw.y & 0xFFFFu)); v[3] += E::to_float((uint16_t)(bw.y >> 16));
-                        }
-                    } else {
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) {
-                            if (row0 + k >= seg.row_end) break;
-                            if (st.s_row) v[k] *= E::to_float(st.s_row[row0 + k]);
-                            if (st.bias) v[k] += E::to_float(st.bias[row0 + k]);
-                        }
-                    }
-                    if (st.addend) {
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) {
-                            if (row0 + k >= seg.row_end) break;
-                            if (st.dep2 >= 0)
-                                v[k] += __builtin_bit_cast(float, __hip_atomic_load((const uint32_t*)st.addend + o + k, __ATOMIC_RELAXED,
-                                                                                    __HIP_MEMORY_SCOPE_AGENT));
-                            else
-                                v[k] += st.addend[o + k];
-                        }
-                    }
-                    if (!st.out_f32 && vec_rows && row0 + 3 < seg.row_end) {
-                        uint2 pk;
-                        pk.x = (uint32_t)E::from_float_clamped(v[0]) | ((uint32_t)E::from_float_clamped(v[1]) << 16);
-                        pk.y = (uint32_t)E::from_float_clamped(v[2]) | ((uint32_t)E::from_float_clamped(v[3]) << 16);
-                        *(uint2*)((uint16_t*)st.out + o) = pk;
-                        return;
-                    }
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        if (row0 + k >= seg.row_end) break;
-                        if (st.out_f32) {
-                            // fp32 results (h, partial sums over terms) may be read by other workgroups of this launch:
-                            // device-coherent store, completed before the counter of the slice is bumped
-                            if (st.signal) __hip_atomic_store((uint32_t*)st.out + o + k, __builtin_bit_cast(uint32_t, v[k]),
-                                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                            else ((float*)st.out)[o + k] = v[k];
-                        } else {
-                            ((uint16_t*)st.out)[o + k] = E::from_float_clamped(v[k]);
-                        }
-                    }
-                };
                 // the q-th group of this wavefront is complete: acc[v] = sum for its row 4 g + v, batch row r16
                 auto store_group = [&](int q, const float4_t& bsum) __attribute__((always_inline)) {
                     const float4_t sum = bsum * -2.f;                             // signed sum = (sum of x) - 2 (sum of b x)
@@ -596,6 +608,95 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                     }
                 }
               }
+            } else if (OWN && !aborted) {
+                // ---- fp4 x fp8 arithmetic, wavefronts own row pairs (every input is one chunk) ----
+                if constexpr (OWN) {
+                    const int cu_n = st.units;
+                    stage_units_q8<DT, BATCH, THREADS, false>(xs, scl, xtot, sin, 0, cu_n, upad, nullptr);
+                    lds_barrier();                               // staged input and its totals visible
+                    const int r16 = qlane & 15, g = qlane >> 4;
+                    const int npairs = (seg.row_end - seg.row_begin + 31) >> 5;
+                    const int ngroups = (cu_n + 3) >> 2;
+                    const int positions = (ngroups + 2) / 3 * 3;       // the three register pairs keep their turns from pair to pair
+                    const int groups_all = (st.words + 15) >> 4;      // tiles per row pair in memory
+                    const uint32_t bits_bytes = (uint32_t)((size_t)((st.rows + 31) >> 5) * groups_all * 2048);
+                    const __amdgpu_buffer_rsrc_t rs = raw_buffer(st.bits, bits_bytes);
+                    const int tile0 = (seg.row_begin >> 5) * groups_all;
+                    // operand column of this lane (batch row, piece), as in the row-block loop below
+                    const bool qlive = r16 < BATCH * kQ8Pieces;
+                    const int qcol = min(r16, BATCH * kQ8Pieces - 1);
+                    const uint4* qbase = xs + (size_t)qcol * upad + 8 * (g >> 1) + (g & 1);
+                    const uint32_t* qscl = scl + (qcol / kQ8Pieces) * ((upad - 1) >> 3) + g;
+                    const bool qlast = qlive && r16 % kQ8Pieces == kQ8Pieces - 1;
+                    // Pairs: the one being worked on, and up to two that the fetches have already moved on to.
+                    int c_pair = qwave, f_pair = qwave, f_j = 0;
+                    int next_a = 0, next_b = 0, queued = 0;
+                    auto take_pair = [&]() -> int {
+                        int p = 0;
+                        if (qlane == 0) p = atomicAdd(&s_pair, 1);
+                        return __builtin_amdgcn_readfirstlane(p);
+                    };
+                    auto fetch = [&](uint4& wa, uint4& wb) __attribute__((always_inline)) {
+                        const bool live = f_pair < npairs && f_j < ngroups;
+                        const int tile = tile0 + f_pair * groups_all + f_j;
+                        const uint32_t soff = live ? (uint32_t)__builtin_amdgcn_readfirstlane(tile) * 2048u : 0u;
+                        const uint32_t voff = live ? (uint32_t)qlane * 16u : kPastEnd;
+                        const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, soff, 2 /* nt */);
+                        const u32x4_t b = __builtin_amdgcn_raw_buffer_load_b128(rs, voff + 1024u, soff, 2 /* nt */);
+                        wa = make_uint4(a.x, a.y, a.z, a.w);
+                        wb = make_uint4(b.x, b.y, b.z, b.w);
+                        if (++f_j == positions) {
+                            f_j = 0;
+                            f_pair = f_pair < npairs ? take_pair() : npairs;
+                            if (queued == 0) next_a = f_pair; else next_b = f_pair;
+                            ++queued;
+                        }
+                    };
+                    Q8Operand opnd = {};
+                    int qscale = 0x7F7F7F7F;
+                    float4_t acc_a = {0.f, 0.f, 0.f, 0.f}, acc_b = {0.f, 0.f, 0.f, 0.f};
+                    auto work = [&](uint4& wa, uint4& wb, int ub) __attribute__((always_inline)) {
+                        if (qlive) {
+                            q8_read_operand(opnd, qbase + 32 * ub);
+                            qscale = (int)qscl[4 * ub];
+                        }
+                        unit_mfma_q8_pair(wa, wb, opnd, qscale, acc_a, acc_b);
+                    };
+                    __builtin_amdgcn_s_waitcnt(0);               // what the staging loaded has been used: see the tile-order loop below
+                    fetch(wa0, wb0); fetch(wa1, wb1); fetch(wa2, wb2);
+#pragma unroll 1
+                    while (c_pair < npairs) {
+#pragma unroll 1
+                        for (int j = 0; j < positions; j += 3) {
+                            work(wa0, wb0, j);
+                            fetch(wa0, wb0);
+                            if (j + 1 < ngroups) work(wa1, wb1, j + 1);
+                            fetch(wa1, wb1);
+                            if (j + 2 < ngroups) work(wa2, wb2, j + 2);
+                            fetch(wa2, wb2);
+                        }
+                        // acc_a[v]: row 32 pair + 4 g + v (acc_b: 16 rows further), column r16; the sum over the pieces of a
+                        // batch row is valid in the lane of its last piece
+                        float4_t sa, sb;
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) {
+                            sa[v] = q8_piece_sum(acc_a[v]);
+                            sb[v] = q8_piece_sum(acc_b[v]);
+                        }
+                        if (qlast) {
+                            const int b = qcol / kQ8Pieces;
+                            const float xt = xtot[b];
+                            const int row0 = seg.row_begin + 32 * c_pair + 4 * g;
+                            if (row0 < seg.row_end) emit4(row0, b, sa + xt);
+                            if (row0 + 16 < seg.row_end) emit4(row0 + 16, b, sb + xt);
+                        }
+                        acc_a = acc_b = (float4_t){0.f, 0.f, 0.f, 0.f};
+                        __builtin_amdgcn_s_waitcnt(0);           // the stores are out: only fetches in flight inside the loop
+                        c_pair = next_a;
+                        next_a = next_b;
+                        --queued;
+                    }
+                }
             } else if (!aborted) {
                 bool staged = false;
 #pragma unroll 1
@@ -862,6 +963,15 @@ struct StreamKernel {
     static constexpr int kThreads = NQ_STREAM_THREADS(DT, BATCH);
     static constexpr auto fn = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, false>;
     static constexpr auto fn_tiled = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2>;
+    // tile order, fp4 x fp8 arithmetic, wavefronts own row pairs: for lists whose longest input is staged in one chunk.
+    // Measured against the row-block form on Llama-2-7B stacks (us per layer, 1 / 2 / 4 / 8 / 32 layers per launch):
+    // batch 4  31.3 / 16.7 / 9.9 / 6.5 / 5.9 against 31.1 / 17.5 / 10.8 / 7.5 / 6.8 (no LDS atomics: four batch rows cost
+    // four times the flushes); batch 2  25.4 / 13.6 / 8.3 / 6.1 / 5.25 against 23.0 / 12.9 / 8.4 / 6.2 / 5.5 (a short
+    // slice has fewer row pairs than wavefronts); batch 1  32 layers 1.8 % slower, one layer 21.0 against 18.9 (the
+    // stores of a pair stop its fetches, and one batch row has little to flush): the builder asks for it at batch 4
+    // and, for long lists, at batch 2.
+    static constexpr bool kHasOwn = kArith == 2 && (BATCH == 2 || BATCH == 4);
+    static constexpr auto fn_tiled_own = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2, false, kHasOwn>;
     static constexpr auto fn_single = gemv_stream_kernel<DT, BATCH, kArith, kThreads, true, false>;
     // reproducible sums
     // the 16-bit arithmetic is reproducible as it is: the same instance
@@ -888,6 +998,9 @@ static hipError_t prepare_kernel(size_t lds) {
         e = hipFuncSetAttribute((const void*)SK::fn_tiled_det,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
         if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute((const void*)SK::fn_tiled_own,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
+        if (e != hipSuccess) return e;
         attr_done.set(dev);
     }
     return hipSuccess;
@@ -911,7 +1024,7 @@ static int capacity_of(int max_units) {
 template <int DT, int BATCH, int ARITH>
 static hipError_t launch_stream(int nstages, const RunSlice* slices, unsigned long long* counters, unsigned* status, int nwg,
                                 int max_units, hipStream_t stream, const void* ext_in, void* ext_out, bool tiled, bool det,
-                                unsigned spin_limit) {
+                                unsigned spin_limit, bool own) {
     using SK = StreamKernel<DT, BATCH, ARITH>;
     if (spin_limit == 0) spin_limit = 1u << 21;                  // about a second of polling
     if (det && !SK::kHasDet) return hipErrorInvalidValue;
@@ -920,7 +1033,10 @@ static hipError_t launch_stream(int nstages, const RunSlice* slices, unsigned lo
     stream_lds_plan(BATCH, SK::kArith, max_units, &chunk_cap, &lds, det);
     hipError_t e = prepare_kernel<DT, BATCH, ARITH>(lds);
     if (e != hipSuccess) return e;
-    if (det)
+    if (SK::kHasOwn && own && tiled && !det && max_units <= chunk_cap)
+        hipLaunchKernelGGL((SK::fn_tiled_own), dim3(nwg), dim3(SK::kThreads), lds, stream, nstages, slices, counters, status,
+                           spin_limit, chunk_cap, RunStage{}, 0, ext_in, ext_out);
+    else if (det)
         hipLaunchKernelGGL((tiled ? SK::fn_tiled_det : SK::fn_det), dim3(nwg), dim3(SK::kThreads), lds, stream, nstages, slices,
                            counters, status, spin_limit, chunk_cap, RunStage{}, 0, ext_in, ext_out);
     else if (tiled && SK::kArith == 2)
@@ -1036,8 +1152,8 @@ bool stream_has_deterministic(int dtype, int batch) {
 
 hipError_t gemv_stream(int dtype, int batch, int nstages, const RunSlice* slices, unsigned long long* counters,
                        unsigned* status, int nwg, int max_units, hipStream_t stream, const void* ext_in, void* ext_out,
-                       bool tiled, bool det, unsigned spin_limit, bool alt) {
-#define NQ_RUN(D, B, A) launch_stream<D, B, A>(nstages, slices, counters, status, nwg, max_units, stream, ext_in, ext_out, tiled, det, spin_limit)
+                       bool tiled, bool det, unsigned spin_limit, bool alt, bool own) {
+#define NQ_RUN(D, B, A) launch_stream<D, B, A>(nstages, slices, counters, status, nwg, max_units, stream, ext_in, ext_out, tiled, det, spin_limit, own)
     NQ_STREAM_DISPATCH(NQ_RUN)
 #undef NQ_RUN
     return hipErrorInvalidValue;

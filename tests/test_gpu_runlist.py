@@ -323,18 +323,20 @@ def test_column_shares_of_short_slices(dev, batch, dtype, tiled):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_batch_4_lists_choose_their_arithmetic_by_length(dev, dtype):
     # fp16 at batch 4: a list with little work per workgroup runs on the 16-bit arithmetic (bit 4 of the plan's flag
-    # word), a long one on the fp4 x fp8 arithmetic; bf16 lists always on the latter.  Both against the oracle.
+    # word), a long one on the fp4 x fp8 arithmetic; bf16 lists always on the latter.  The fp4 x fp8 kernel whose
+    # wavefronts own whole row pairs (bit 5) takes every tile-order list at batch 4 and long ones at batch 2.  All
+    # against the oracle.
     to = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev).to(dtype)
     f64 = lambda t: t.float().cpu().numpy().astype(np.float64)
     m, n, r = 520, 8192, 2000
-    for count in (1, 64):
-        rl = DecodeRunList(4, dtype, dev)
+    for batch, count in ((4, 1), (4, 64), (2, 1), (2, 96)):
+        rl = DecodeRunList(batch, dtype, dev)
         checked = {}
         for i in range(count):
             vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, 8100 + (i if i in (0, count - 1) else 1))
             vt_p, u_p, mid_p = oracle.pad_rank(vt, u, s_mid, 32)
             pack = lambda w: packing.tile_words(packing.binary_packer(torch.from_numpy(w), "half2").to(dev))
-            x = to(oracle.synth_x(4, n, 8200 + i))
+            x = to(oracle.synth_x(batch, n, 8200 + i))
             sc = (to(s_in), to(mid_p), to(s_out))
             rl.add(x, sc[0], pack(vt_p), sc[1], pack(u_p), sc[2], tiled=True)
             if i in (0, count - 1):
@@ -342,12 +344,13 @@ def test_batch_4_lists_choose_their_arithmetic_by_length(dev, dtype):
         ys = rl.run()
         torch.cuda.synchronize()
         assert rl.status() == 0
-        short = bool(rl._plan.bound & 16)
-        print(f"batch 4 {dtype} list of {count}: 16-bit arithmetic = {short}", flush=True)
-        assert short == (count == 1 and dtype == torch.float16)
+        short, own = bool(rl._plan.bound & 16), bool(rl._plan.bound & 32)
+        print(f"batch {batch} {dtype} list of {count}: 16-bit arithmetic = {short}, owned row pairs = {own}", flush=True)
+        assert short == (batch == 4 and count == 1 and dtype == torch.float16)
+        assert own == (not short and (batch == 4 or count == 96))
         for i, ref in checked.items():
             err = oracle.max_rel_err(ys[i].float().cpu().numpy(), ref)
-            assert err < (1e-2 if dtype == torch.bfloat16 else TIGHT), (count, i, err)
+            assert err < (1e-2 if dtype == torch.bfloat16 else TIGHT), (batch, count, i, err)
     # a short list whose input is longer than what is staged at once at 4 rows (28672 columns, two chunks on the 16-bit
     # arithmetic) and whose rows end inside a 16-row group
     m, n, r = 100, 28672, 256
