@@ -170,16 +170,19 @@ def test_bf16_and_ragged_shapes(dev, batch):
         assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < (1e-2 if batch == 1 else 2e-2)   # bf16 staging from 8 rows on
 
 
-def test_graph_replay_of_a_run_list(dev):
-    # the launch allocates nothing and can be replayed; replays must equal the eager result
-    batch = 1
-    rl = DecodeRunList(batch, torch.float16, dev, interleave=2)
+@pytest.mark.parametrize("batch,dtype,tiled", [(1, torch.float16, False), (4, torch.bfloat16, True), (4, torch.float16, True),
+                                               (16, torch.float16, True)])
+def test_graph_replay_of_a_run_list(dev, batch, dtype, tiled):
+    # the launch allocates nothing and can be replayed; replays must equal the eager result.  Batch 4: bf16 in tile order
+    # runs the kernel whose wavefronts take row pairs from a counter in LDS, the short fp16 list the 16-bit arithmetic.
+    rl = DecodeRunList(batch, dtype, dev, interleave=2)
     xs = []
     for i, (m, n, r) in enumerate([(1024, 1024, 512), (1024, 2048, 512), (2048, 1024, 512)]):
         _, ops = _term(dev, m, n, r, seed=300 + i)
-        x = torch.from_numpy(oracle.synth_x(batch, n, 300 + i)).to(dev)
+        ops = tuple(o.to(dtype) if o.dtype == torch.float16 else (packing.tile_words(o) if tiled else o) for o in ops)
+        x = torch.from_numpy(oracle.synth_x(batch, n, 300 + i)).to(dev).to(dtype)
         xs.append(x)
-        rl.add(x, *ops)
+        rl.add(x, *ops, tiled=tiled)
     eager = [y.clone() for y in rl.run()]
     torch.cuda.synchronize()
     side = torch.cuda.Stream()
