@@ -160,9 +160,10 @@ int nq_runlist_status(const void* workspace, int* status_out, void* stream);
  * the last bit between launches (the reference's reductions are ordered: kernel/cuda/gemv_kernel.cu:148-170,
  * shuffles inside one warp).  With this switch every launch of the plan gives bit-identical outputs.  Batch 1, 2 and
  * 4: partial sums are rounded to a grid on which their additions are exact; the results stay within the same
- * tolerance but lose up to 16 bits below (columns x largest input value).  Batch 8 and 16, and plans with bit 4 of
- * `bound` set: every row sum is formed by one wavefront in a fixed order whether the switch is on or off; it is
- * accepted and selects the same kernel.
+ * tolerance but lose up to 16 bits below (columns x largest input value); plans with bit 5 of `bound` set in tile
+ * order form every row sum in one wavefront and lose nothing (the switch only fixes the order in which the input totals
+ * are added).  Batch 8 and 16, and plans with bit 4 of `bound` set: every row sum is formed by one wavefront in a fixed
+ * order whether the switch is on or off; it is accepted and selects the same kernel.
  * NQ_ERR_SHAPE for a batch size without a run-list kernel.  Sets bit 3 of plan->bound. */
 int nq_runlist_set_deterministic(nq_runlist_plan* plan, int on);
 

@@ -106,8 +106,10 @@ __device__ __forceinline__ void trim_unit(const BitsView& v, uint4& w, int unit)
 // The 16-bit arithmetic keeps its row sums in registers; its LDS head holds the totals of the staged units
 // ([batch][units + 1] floats, added up in unit order: no LDS atomics, so the results do not depend on their order).
 constexpr int kUnitTotalsBytes = 4096;
-__host__ __device__ constexpr size_t stream_head_bytes(int batch, int arith, bool det = false) {
-    return arith == 2 ? (size_t)row_block(batch) * batch * sizeof(float) * (det ? 2 : 1) + (det ? 1024 : 128) : (size_t)kUnitTotalsBytes + 128;
+// own: the fp4 x fp8 variant whose wavefronts own row pairs keeps no row sums in LDS.
+__host__ __device__ constexpr size_t stream_head_bytes(int batch, int arith, bool det = false, bool own = false) {
+    return arith == 2 ? (own ? 0 : (size_t)row_block(batch) * batch * sizeof(float) * (det ? 2 : 1)) + (det ? 1024 : 128)
+                      : (size_t)kUnitTotalsBytes + 128;
 }
 
 // fp4 x fp8 arithmetic: items that each wavefront of a workgroup takes (contiguous runs).
@@ -139,10 +141,10 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
     extern __shared__ uint4 lds_raw[];
     static_assert(ARITH == 1 || ARITH == 2, "unknown arithmetic");
     constexpr bool kQ8 = ARITH == 2;
-    static_assert(!OWN || (kQ8 && TILED && !SINGLE && !DET), "owned row pairs exist for the tile-order fp4 x fp8 kernel only");
+    static_assert(!OWN || (kQ8 && TILED && !SINGLE), "owned row pairs exist for the tile-order fp4 x fp8 kernel only");
     constexpr bool kTotals = true;                              // both arithmetics: signed sum = (sum of x) - 2 (sum of b x)
     static_assert(!kQ8 || BATCH * kQ8Pieces <= 16, "pieces of all batch rows must fit the 16 operand columns");
-    constexpr int kRaccFloats = kQ8 ? kRowBlock * BATCH : kUnitTotalsBytes / (int)sizeof(float);   // 16-bit arithmetic: the unit totals
+    constexpr int kRaccFloats = kQ8 ? (OWN ? 0 : kRowBlock * BATCH) : kUnitTotalsBytes / (int)sizeof(float);   // 16-bit arithmetic: the unit totals
     float* racc = (float*)lds_raw;                              // [kRowBlock][BATCH] row sums
     float* rtot = racc + kRaccFloats;                           // DET: the same, summed over the input chunks done so far
     // [2][16] sum of the staged input per batch row (DET: [2][16 wavefronts][4]); slices alternate between the two, so
@@ -150,7 +152,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
     constexpr int kTotStride = (DET && kQ8) ? 64 : 16;
     float* xtot_base = racc + kRaccFloats * (DET && kQ8 ? 2 : 1);
     uint32_t* ebmax_base = (uint32_t*)(xtot_base + 2 * kTotStride);   // DET: [2] largest unit exponent of the staged input
-    uint4* xs_base = lds_raw + stream_head_bytes(BATCH, ARITH, DET) / sizeof(uint4);
+    uint4* xs_base = lds_raw + stream_head_bytes(BATCH, ARITH, DET, OWN) / sizeof(uint4);
     __shared__ int s_flag;
     __shared__ int s_pair;                                      // OWN: the next row pair of the slice that nobody has taken
     const int tid = threadIdx.x;
@@ -612,7 +614,10 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                 // ---- fp4 x fp8 arithmetic, wavefronts own row pairs (every input is one chunk) ----
                 if constexpr (OWN) {
                     const int cu_n = st.units;
-                    stage_units_q8<DT, BATCH, THREADS, false>(xs, scl, xtot, sin, 0, cu_n, upad, nullptr);
+                    // DET: the input totals are kept per wavefront and added in wavefront order below; the row sums are
+                    // formed by one wavefront in a fixed order whichever wavefront takes the pair, so nothing is rounded
+                    // to a grid here
+                    stage_units_q8<DT, BATCH, THREADS, DET>(xs, scl, xtot, sin, 0, cu_n, upad, ebmax);
                     lds_barrier();                               // staged input and its totals visible
                     const int r16 = qlane & 15, g = qlane >> 4;
                     const int npairs = (seg.row_end - seg.row_begin + 31) >> 5;
@@ -685,7 +690,13 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                         }
                         if (qlast) {
                             const int b = qcol / kQ8Pieces;
-                            const float xt = xtot[b];
+                            float xt = 0.f;
+                            if constexpr (DET) {
+#pragma unroll
+                                for (int w = 0; w < kWaves; ++w) xt += xtot[4 * w + b];
+                            } else {
+                                xt = xtot[b];
+                            }
                             const int row0 = seg.row_begin + 32 * c_pair + 4 * g;
                             if (row0 < seg.row_end) emit4(row0, b, sa + xt);
                             if (row0 + 16 < seg.row_end) emit4(row0 + 16, b, sb + xt);
@@ -907,8 +918,9 @@ size_t stream_counter_bytes(int nstages) {
 }
 
 // ---- host side --------------------------------------------------------------------------------
-static void stream_lds_plan(int batch, int arith, int max_units, int* chunk_cap_out, size_t* lds_out, bool det = false) {
-    const int racc_bytes = (int)stream_head_bytes(batch, arith, det && arith == 2);
+static void stream_lds_plan(int batch, int arith, int max_units, int* chunk_cap_out, size_t* lds_out, bool det = false,
+                            bool own = false) {
+    const int racc_bytes = (int)stream_head_bytes(batch, arith, det && arith == 2, own && arith == 2);
     if (arith == 2) {
         // kQ8Pieces bytes per column and batch row, staged in whole groups of four units
         // plus one scale dword per batch row and unit
@@ -972,6 +984,7 @@ struct StreamKernel {
     // and, for long lists, at batch 2.
     static constexpr bool kHasOwn = kArith == 2 && (BATCH == 2 || BATCH == 4);
     static constexpr auto fn_tiled_own = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2, false, kHasOwn>;
+    static constexpr auto fn_tiled_own_det = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2, kHasOwn, kHasOwn>;
     static constexpr auto fn_single = gemv_stream_kernel<DT, BATCH, kArith, kThreads, true, false>;
     // reproducible sums
     // the 16-bit arithmetic is reproducible as it is: the same instance
@@ -999,6 +1012,9 @@ static hipError_t prepare_kernel(size_t lds) {
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
         if (e != hipSuccess) return e;
         e = hipFuncSetAttribute((const void*)SK::fn_tiled_own,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute((const void*)SK::fn_tiled_own_det,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLdsMax);
         if (e != hipSuccess) return e;
         attr_done.set(dev);
@@ -1030,12 +1046,19 @@ static hipError_t launch_stream(int nstages, const RunSlice* slices, unsigned lo
     if (det && !SK::kHasDet) return hipErrorInvalidValue;
     int chunk_cap;
     size_t lds;
-    stream_lds_plan(BATCH, SK::kArith, max_units, &chunk_cap, &lds, det);
+    // the variant whose wavefronts own row pairs, where the plan asks for it and the longest input is one chunk of its
+    // (larger) staging area
+    own = SK::kHasOwn && own && tiled;
+    if (own) {
+        stream_lds_plan(BATCH, SK::kArith, max_units, &chunk_cap, &lds, det, true);
+        own = max_units <= chunk_cap;
+    }
+    if (!own) stream_lds_plan(BATCH, SK::kArith, max_units, &chunk_cap, &lds, det);
     hipError_t e = prepare_kernel<DT, BATCH, ARITH>(lds);
     if (e != hipSuccess) return e;
-    if (SK::kHasOwn && own && tiled && !det && max_units <= chunk_cap)
-        hipLaunchKernelGGL((SK::fn_tiled_own), dim3(nwg), dim3(SK::kThreads), lds, stream, nstages, slices, counters, status,
-                           spin_limit, chunk_cap, RunStage{}, 0, ext_in, ext_out);
+    if (own)
+        hipLaunchKernelGGL((det ? SK::fn_tiled_own_det : SK::fn_tiled_own), dim3(nwg), dim3(SK::kThreads), lds, stream, nstages,
+                           slices, counters, status, spin_limit, chunk_cap, RunStage{}, 0, ext_in, ext_out);
     else if (det)
         hipLaunchKernelGGL((tiled ? SK::fn_tiled_det : SK::fn_det), dim3(nwg), dim3(SK::kThreads), lds, stream, nstages, slices,
                            counters, status, spin_limit, chunk_cap, RunStage{}, 0, ext_in, ext_out);
