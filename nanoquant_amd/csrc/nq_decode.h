@@ -42,10 +42,12 @@ struct StageInput {
 };
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 // By value on purpose: __builtin_bit_cast applied directly to a vector element (v.y, v[e]) reads
 // element 0 with this compiler.
 __device__ __forceinline__ float as_float(uint32_t bits) { return __builtin_bit_cast(float, bits); }
+__device__ __forceinline__ uint32_t as_bits(float v) { return __builtin_bit_cast(uint32_t, v); }
 
 // Raw buffer view (gfx9 resource words) of `bytes` bytes at p: loads past the end return zeros, so a
 // lane whose columns lie beyond K is pointed past the end instead of being branched around.

@@ -620,9 +620,14 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                     stage_units_q8<DT, BATCH, THREADS, DET>(xs, scl, xtot, sin, 0, cu_n, upad, ebmax);
                     lds_barrier();                               // staged input and its totals visible
                     const int r16 = qlane & 15, g = qlane >> 4;
-                    const int npairs = (seg.row_end - seg.row_begin + 31) >> 5;
+                    const int nrows = seg.row_end - seg.row_begin;
+                    const int npairs = (nrows + 31) >> 5;
                     const int ngroups = (cu_n + 3) >> 2;
                     const int positions = (ngroups + 2) / 3 * 3;       // the three register pairs keep their turns from pair to pair
+                    // results that need only their row scale go out as buffer stores (see the end of a pair)
+                    const size_t out_elems = (size_t)(BATCH - 1) * st.out_stride + st.rows;
+                    const bool plain_out = vec_rows && st.s_row && !st.bias && !st.addend && out_elems < (1u << 28);
+                    const __amdgpu_buffer_rsrc_t rout = raw_buffer(st.out, (uint32_t)(out_elems * (st.out_f32 ? 4u : 2u)));
                     const int groups_all = (st.words + 15) >> 4;      // tiles per row pair in memory
                     const uint32_t bits_bytes = (uint32_t)((size_t)((st.rows + 31) >> 5) * groups_all * 2048);
                     const __amdgpu_buffer_rsrc_t rs = raw_buffer(st.bits, bits_bytes);
@@ -688,21 +693,70 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                             sa[v] = q8_piece_sum(acc_a[v]);
                             sb[v] = q8_piece_sum(acc_b[v]);
                         }
-                        if (qlast) {
-                            const int b = qcol / kQ8Pieces;
-                            float xt = 0.f;
-                            if constexpr (DET) {
+                        const int b = qcol / kQ8Pieces;
+                        float xt = 0.f;
+                        if constexpr (DET) {
 #pragma unroll
-                                for (int w = 0; w < kWaves; ++w) xt += xtot[4 * w + b];
-                            } else {
-                                xt = xtot[b];
+                            for (int w = 0; w < kWaves; ++w) xt += xtot[4 * w + b];
+                        } else {
+                            xt = xtot[b];
+                        }
+                        sa += xt;
+                        sb += xt;
+                        if (plain_out && 32 * (c_pair + 1) <= nrows) {
+                            // A whole pair with nothing but row scales on the way out.  The scales come through the
+                            // scalar cache (64 bytes per pair, the same for every lane group) and the results leave as
+                            // two buffer stores per lane, past the end of the buffer for the lanes that hold no sum:
+                            // a fixed number of stores and no load among the lane memory operations, so the item
+                            // fetches that are in flight stay in flight (a load here would have to wait for all of
+                            // them, a varying number of stores likewise).
+                            typedef const uint32_t __attribute__((address_space(4)))* scalar_words_t;
+                            const int prow = seg.row_begin + 32 * __builtin_amdgcn_readfirstlane(c_pair);
+                            const scalar_words_t sp = (scalar_words_t)(uintptr_t)(st.s_row + prow);
+                            uint32_t sw[16];
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) {
+                                sw[i] = sp[i];
+                                asm volatile("" : "+s"(sw[i]));          // kept in scalar registers: one scalar load each
                             }
-                            const int row0 = seg.row_begin + 32 * c_pair + 4 * g;
-                            if (row0 < seg.row_end) emit4(row0, b, sa + xt);
-                            if (row0 + 16 < seg.row_end) emit4(row0 + 16, b, sb + xt);
+                            uint32_t s0 = sw[0], s1 = sw[1], s2 = sw[8], s3 = sw[9];   // rows 4g .. 4g + 3, 16 + 4g .. 16 + 4g + 3
+#pragma unroll
+                            for (int q = 1; q < 4; ++q) {
+                                s0 = g == q ? sw[2 * q] : s0;
+                                s1 = g == q ? sw[2 * q + 1] : s1;
+                                s2 = g == q ? sw[8 + 2 * q] : s2;
+                                s3 = g == q ? sw[9 + 2 * q] : s3;
+                            }
+                            sa[0] *= E::to_float((uint16_t)(s0 & 0xFFFFu)); sa[1] *= E::to_float((uint16_t)(s0 >> 16));
+                            sa[2] *= E::to_float((uint16_t)(s1 & 0xFFFFu)); sa[3] *= E::to_float((uint16_t)(s1 >> 16));
+                            sb[0] *= E::to_float((uint16_t)(s2 & 0xFFFFu)); sb[1] *= E::to_float((uint16_t)(s2 >> 16));
+                            sb[2] *= E::to_float((uint16_t)(s3 & 0xFFFFu)); sb[3] *= E::to_float((uint16_t)(s3 >> 16));
+                            const uint32_t elem = (uint32_t)b * (uint32_t)st.out_stride + (uint32_t)(prow + 4 * g);
+                            if (st.out_f32) {
+                                // fp32 results may be read by other workgroups of this launch: device-coherent stores
+                                const uint32_t off = qlast ? elem * 4u : kPastEnd;
+                                const u32x4_t ua = {as_bits(sa[0]), as_bits(sa[1]), as_bits(sa[2]), as_bits(sa[3])};
+                                const u32x4_t ub = {as_bits(sb[0]), as_bits(sb[1]), as_bits(sb[2]), as_bits(sb[3])};
+                                __builtin_amdgcn_raw_buffer_store_b128(ua, rout, off, 0, kCacheAgentCoherent);
+                                __builtin_amdgcn_raw_buffer_store_b128(ub, rout, off + 64u, 0, kCacheAgentCoherent);
+                            } else {
+                                const uint32_t off = qlast ? elem * 2u : kPastEnd;
+                                const u32x2_t ua = {(uint32_t)E::from_float_clamped(sa[0]) | ((uint32_t)E::from_float_clamped(sa[1]) << 16),
+                                                    (uint32_t)E::from_float_clamped(sa[2]) | ((uint32_t)E::from_float_clamped(sa[3]) << 16)};
+                                const u32x2_t ub = {(uint32_t)E::from_float_clamped(sb[0]) | ((uint32_t)E::from_float_clamped(sb[1]) << 16),
+                                                    (uint32_t)E::from_float_clamped(sb[2]) | ((uint32_t)E::from_float_clamped(sb[3]) << 16)};
+                                __builtin_amdgcn_raw_buffer_store_b64(ua, rout, off, 0, kCacheDefault);
+                                __builtin_amdgcn_raw_buffer_store_b64(ub, rout, off + 32u, 0, kCacheDefault);
+                            }
+                        } else {
+                            if (qlast) {
+                                const int row0 = seg.row_begin + 32 * c_pair + 4 * g;
+                                if (row0 < seg.row_end) emit4(row0, b, sa);
+                                if (row0 + 16 < seg.row_end) emit4(row0 + 16, b, sb);
+                            }
+                            __builtin_amdgcn_s_waitcnt(0);       // loads and a varying number of stores: start over with only fetches in flight
                         }
                         acc_a = acc_b = (float4_t){0.f, 0.f, 0.f, 0.f};
-                        __builtin_amdgcn_s_waitcnt(0);           // the stores are out: only fetches in flight inside the loop
                         c_pair = next_a;
                         next_a = next_b;
                         --queued;
