@@ -138,7 +138,7 @@ typedef struct nq_runlist_plan {
                                bit 4: set by the builder for a short fp16 list at batch 4, which runs on the arithmetic of
                                batch 8 and 16 (16-bit operands; reproducible with or without bit 3);
                                bit 5: set by the builder where the kernel variant whose wavefronts own whole row pairs
-                               is the faster one (batch 4, long lists at batch 2; used for tile order without bit 3) */
+                               is the faster one (batch 4, long lists at batch 1 and 2; used for tile order) */
     int spin_limit;         /* polls after which a dependency wait gives up and sets the status word; 0 (as built) =
                                the default of 2^21 polls, about a second.  The caller may lower it, e.g. to exercise
                                its handling of an expired wait: every kernel still runs to its end */

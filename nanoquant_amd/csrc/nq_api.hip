@@ -291,10 +291,10 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
     }
     const bool wide = batch >= 8 || alt;                 // the 16-bit arithmetic and its cost model
     // fp4 x fp8 arithmetic with wavefronts that own row pairs (tile order only; the launch falls back where it does not
-    // apply): always at batch 4, from about six Llama-2-7B layers per launch on at batch 2 (40000 rows x units per
+    // apply): always at batch 4, from about six Llama-2-7B layers per launch on at batch 1 and 2 (40000 rows x units per
     // workgroup), where a slice has more row pairs than the workgroup has wavefronts
     bool own = false;
-    if (!alt && (batch == 4 || batch == 2)) {
+    if (!alt && batch <= 4) {
         long long work = 0;
         for (const auto& st : table) work += (long long)st.rows * st.units;
         own = batch == 4 || work / std::max(1, nq::stream_capacity(dtype, batch, max_units, false)) >= 40000;

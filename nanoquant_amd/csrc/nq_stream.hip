@@ -626,7 +626,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                     const int positions = (ngroups + 2) / 3 * 3;       // the three register pairs keep their turns from pair to pair
                     // results that need only their row scale go out as buffer stores (see the end of a pair)
                     const size_t out_elems = (size_t)(BATCH - 1) * st.out_stride + st.rows;
-                    const bool plain_out = vec_rows && st.s_row && !st.bias && !st.addend && out_elems < (1u << 28);
+                    const bool plain_out = vec_rows && (nrows & 31) == 0 && st.s_row && !st.bias && !st.addend && out_elems < (1u << 28);
                     const __amdgpu_buffer_rsrc_t rout = raw_buffer(st.out, (uint32_t)(out_elems * (st.out_f32 ? 4u : 2u)));
                     const int groups_all = (st.words + 15) >> 4;      // tiles per row pair in memory
                     const uint32_t bits_bytes = (uint32_t)((size_t)((st.rows + 31) >> 5) * groups_all * 2048);
@@ -672,95 +672,110 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                         }
                         unit_mfma_q8_pair(wa, wb, opnd, qscale, acc_a, acc_b);
                     };
-                    __builtin_amdgcn_s_waitcnt(0);               // what the staging loaded has been used: see the tile-order loop below
-                    fetch(wa0, wb0); fetch(wa1, wb1); fetch(wa2, wb2);
+                    auto three_items = [&](int j) __attribute__((always_inline)) {
+                        work(wa0, wb0, j);
+                        fetch(wa0, wb0);
+                        if (j + 1 < ngroups) work(wa1, wb1, j + 1);
+                        fetch(wa1, wb1);
+                        if (j + 2 < ngroups) work(wa2, wb2, j + 2);
+                        fetch(wa2, wb2);
+                    };
+                    // PLAIN: every pair of the slice is whole and nothing but the row scale is applied on the way out.
+                    // The scales then come through the scalar cache (64 bytes per pair, the same for every lane) and the
+                    // results leave as four buffer stores per lane (two per output type, past the end of the buffer for
+                    // the other type and for the lanes that hold no sum): no load among the lane memory operations of
+                    // the loop but the item fetches, and a fixed number of stores on every way through it, so the
+                    // compiler, which counts the lane memory operations behind a fetch to know how long to wait for it,
+                    // lets the fetches in flight stay in flight from pair to pair.  (A load at the end of a pair waits
+                    // for all of them, and so does every step of the loop behind a varying number of stores.)  For the
+                    // same reason the first three items of a pair are code of their own, reached only with four stores
+                    // behind the three fetches: from the end of a pair and from the start of the slice.
+                    // (That holds at batch 4.  At one and two batch rows the same loop without the code of its own, where
+                    // the first items of a pair wait for a fetch more than they need, measures 5 % faster and equal.)
+                    constexpr bool kOwnExactWaits = BATCH >= 4;
+                    auto run_pairs = [&](auto plain_tag) __attribute__((always_inline)) {
+                        constexpr bool PLAIN = decltype(plain_tag)::value;
+                        const uint32_t past32 = st.out_f32 ? 0u : kPastEnd, past16 = st.out_f32 ? kPastEnd : 0u;
+                        auto store_pair = [&](uint32_t elem, bool live, float4_t va, float4_t vb) __attribute__((always_inline)) {
+                            const uint32_t o32 = live ? (elem * 4u) | past32 : kPastEnd;
+                            const uint32_t o16 = live ? (elem * 2u) | past16 : kPastEnd;
+                            // fp32 results may be read by other workgroups of this launch: device-coherent stores
+                            const u32x4_t fa = {as_bits(va[0]), as_bits(va[1]), as_bits(va[2]), as_bits(va[3])};
+                            const u32x4_t fb = {as_bits(vb[0]), as_bits(vb[1]), as_bits(vb[2]), as_bits(vb[3])};
+                            __builtin_amdgcn_raw_buffer_store_b128(fa, rout, o32, 0, kCacheAgentCoherent);
+                            __builtin_amdgcn_raw_buffer_store_b128(fb, rout, o32 + 64u, 0, kCacheAgentCoherent);
+                            const u32x2_t ha = {(uint32_t)E::from_float_clamped(va[0]) | ((uint32_t)E::from_float_clamped(va[1]) << 16),
+                                                (uint32_t)E::from_float_clamped(va[2]) | ((uint32_t)E::from_float_clamped(va[3]) << 16)};
+                            const u32x2_t hb = {(uint32_t)E::from_float_clamped(vb[0]) | ((uint32_t)E::from_float_clamped(vb[1]) << 16),
+                                                (uint32_t)E::from_float_clamped(vb[2]) | ((uint32_t)E::from_float_clamped(vb[3]) << 16)};
+                            __builtin_amdgcn_raw_buffer_store_b64(ha, rout, o16, 0, kCacheDefault);
+                            __builtin_amdgcn_raw_buffer_store_b64(hb, rout, o16 + 32u, 0, kCacheDefault);
+                        };
+                        __builtin_amdgcn_s_waitcnt(0);           // what the staging loaded has been used: see the tile-order loop below
+                        fetch(wa0, wb0); fetch(wa1, wb1); fetch(wa2, wb2);
+                        if constexpr (PLAIN) store_pair(0u, false, acc_a, acc_b);
 #pragma unroll 1
-                    while (c_pair < npairs) {
+                        while (c_pair < npairs) {
+                            if constexpr (PLAIN && kOwnExactWaits) three_items(0);
 #pragma unroll 1
-                        for (int j = 0; j < positions; j += 3) {
-                            work(wa0, wb0, j);
-                            fetch(wa0, wb0);
-                            if (j + 1 < ngroups) work(wa1, wb1, j + 1);
-                            fetch(wa1, wb1);
-                            if (j + 2 < ngroups) work(wa2, wb2, j + 2);
-                            fetch(wa2, wb2);
-                        }
-                        // acc_a[v]: row 32 pair + 4 g + v (acc_b: 16 rows further), column r16; the sum over the pieces of a
-                        // batch row is valid in the lane of its last piece
-                        float4_t sa, sb;
+                            for (int j = PLAIN && kOwnExactWaits ? 3 : 0; j < positions; j += 3) three_items(j);
+                            // acc_a[v]: row 32 pair + 4 g + v (acc_b: 16 rows further), column r16; the sum over the pieces
+                            // of a batch row is valid in the lane of its last piece
+                            float4_t sa, sb;
 #pragma unroll
-                        for (int v = 0; v < 4; ++v) {
-                            sa[v] = q8_piece_sum(acc_a[v]);
-                            sb[v] = q8_piece_sum(acc_b[v]);
-                        }
-                        const int b = qcol / kQ8Pieces;
-                        float xt = 0.f;
-                        if constexpr (DET) {
-#pragma unroll
-                            for (int w = 0; w < kWaves; ++w) xt += xtot[4 * w + b];
-                        } else {
-                            xt = xtot[b];
-                        }
-                        sa += xt;
-                        sb += xt;
-                        if (plain_out && 32 * (c_pair + 1) <= nrows) {
-                            // A whole pair with nothing but row scales on the way out.  The scales come through the
-                            // scalar cache (64 bytes per pair, the same for every lane group) and the results leave as
-                            // two buffer stores per lane, past the end of the buffer for the lanes that hold no sum:
-                            // a fixed number of stores and no load among the lane memory operations, so the item
-                            // fetches that are in flight stay in flight (a load here would have to wait for all of
-                            // them, a varying number of stores likewise).
-                            typedef const uint32_t __attribute__((address_space(4)))* scalar_words_t;
-                            const int prow = seg.row_begin + 32 * __builtin_amdgcn_readfirstlane(c_pair);
-                            const scalar_words_t sp = (scalar_words_t)(uintptr_t)(st.s_row + prow);
-                            uint32_t sw[16];
-#pragma unroll
-                            for (int i = 0; i < 16; ++i) {
-                                sw[i] = sp[i];
-                                asm volatile("" : "+s"(sw[i]));          // kept in scalar registers: one scalar load each
+                            for (int v = 0; v < 4; ++v) {
+                                sa[v] = q8_piece_sum(acc_a[v]);
+                                sb[v] = q8_piece_sum(acc_b[v]);
                             }
-                            uint32_t s0 = sw[0], s1 = sw[1], s2 = sw[8], s3 = sw[9];   // rows 4g .. 4g + 3, 16 + 4g .. 16 + 4g + 3
+                            const int b = qcol / kQ8Pieces;
+                            float xt = 0.f;
+                            if constexpr (DET) {
 #pragma unroll
-                            for (int q = 1; q < 4; ++q) {
-                                s0 = g == q ? sw[2 * q] : s0;
-                                s1 = g == q ? sw[2 * q + 1] : s1;
-                                s2 = g == q ? sw[8 + 2 * q] : s2;
-                                s3 = g == q ? sw[9 + 2 * q] : s3;
-                            }
-                            sa[0] *= E::to_float((uint16_t)(s0 & 0xFFFFu)); sa[1] *= E::to_float((uint16_t)(s0 >> 16));
-                            sa[2] *= E::to_float((uint16_t)(s1 & 0xFFFFu)); sa[3] *= E::to_float((uint16_t)(s1 >> 16));
-                            sb[0] *= E::to_float((uint16_t)(s2 & 0xFFFFu)); sb[1] *= E::to_float((uint16_t)(s2 >> 16));
-                            sb[2] *= E::to_float((uint16_t)(s3 & 0xFFFFu)); sb[3] *= E::to_float((uint16_t)(s3 >> 16));
-                            const uint32_t elem = (uint32_t)b * (uint32_t)st.out_stride + (uint32_t)(prow + 4 * g);
-                            if (st.out_f32) {
-                                // fp32 results may be read by other workgroups of this launch: device-coherent stores
-                                const uint32_t off = qlast ? elem * 4u : kPastEnd;
-                                const u32x4_t ua = {as_bits(sa[0]), as_bits(sa[1]), as_bits(sa[2]), as_bits(sa[3])};
-                                const u32x4_t ub = {as_bits(sb[0]), as_bits(sb[1]), as_bits(sb[2]), as_bits(sb[3])};
-                                __builtin_amdgcn_raw_buffer_store_b128(ua, rout, off, 0, kCacheAgentCoherent);
-                                __builtin_amdgcn_raw_buffer_store_b128(ub, rout, off + 64u, 0, kCacheAgentCoherent);
+                                for (int w = 0; w < kWaves; ++w) xt += xtot[4 * w + b];
                             } else {
-                                const uint32_t off = qlast ? elem * 2u : kPastEnd;
-                                const u32x2_t ua = {(uint32_t)E::from_float_clamped(sa[0]) | ((uint32_t)E::from_float_clamped(sa[1]) << 16),
-                                                    (uint32_t)E::from_float_clamped(sa[2]) | ((uint32_t)E::from_float_clamped(sa[3]) << 16)};
-                                const u32x2_t ub = {(uint32_t)E::from_float_clamped(sb[0]) | ((uint32_t)E::from_float_clamped(sb[1]) << 16),
-                                                    (uint32_t)E::from_float_clamped(sb[2]) | ((uint32_t)E::from_float_clamped(sb[3]) << 16)};
-                                __builtin_amdgcn_raw_buffer_store_b64(ua, rout, off, 0, kCacheDefault);
-                                __builtin_amdgcn_raw_buffer_store_b64(ub, rout, off + 32u, 0, kCacheDefault);
+                                xt = xtot[b];
                             }
-                        } else {
-                            if (qlast) {
-                                const int row0 = seg.row_begin + 32 * c_pair + 4 * g;
-                                if (row0 < seg.row_end) emit4(row0, b, sa);
-                                if (row0 + 16 < seg.row_end) emit4(row0 + 16, b, sb);
+                            sa += xt;
+                            sb += xt;
+                            if constexpr (PLAIN) {
+                                typedef const uint32_t __attribute__((address_space(4)))* scalar_words_t;
+                                const int prow = seg.row_begin + 32 * __builtin_amdgcn_readfirstlane(c_pair);
+                                const scalar_words_t sp = (scalar_words_t)(uintptr_t)(st.s_row + prow);
+                                uint32_t sw[16];
+#pragma unroll
+                                for (int i = 0; i < 16; ++i) {
+                                    sw[i] = sp[i];
+                                    asm volatile("" : "+s"(sw[i]));      // kept in scalar registers: one scalar load each
+                                }
+                                uint32_t s0 = sw[0], s1 = sw[1], s2 = sw[8], s3 = sw[9];   // rows 4g .. 4g + 3, 16 + 4g .. 16 + 4g + 3
+#pragma unroll
+                                for (int q = 1; q < 4; ++q) {
+                                    s0 = g == q ? sw[2 * q] : s0;
+                                    s1 = g == q ? sw[2 * q + 1] : s1;
+                                    s2 = g == q ? sw[8 + 2 * q] : s2;
+                                    s3 = g == q ? sw[9 + 2 * q] : s3;
+                                }
+                                sa[0] *= E::to_float((uint16_t)(s0 & 0xFFFFu)); sa[1] *= E::to_float((uint16_t)(s0 >> 16));
+                                sa[2] *= E::to_float((uint16_t)(s1 & 0xFFFFu)); sa[3] *= E::to_float((uint16_t)(s1 >> 16));
+                                sb[0] *= E::to_float((uint16_t)(s2 & 0xFFFFu)); sb[1] *= E::to_float((uint16_t)(s2 >> 16));
+                                sb[2] *= E::to_float((uint16_t)(s3 & 0xFFFFu)); sb[3] *= E::to_float((uint16_t)(s3 >> 16));
+                                store_pair((uint32_t)b * (uint32_t)st.out_stride + (uint32_t)(prow + 4 * g), qlast, sa, sb);
+                            } else {
+                                if (qlast) {
+                                    const int row0 = seg.row_begin + 32 * c_pair + 4 * g;
+                                    if (row0 < seg.row_end) emit4(row0, b, sa);
+                                    if (row0 + 16 < seg.row_end) emit4(row0 + 16, b, sb);
+                                }
+                                __builtin_amdgcn_s_waitcnt(0);   // loads and a varying number of stores: start over with only fetches in flight
                             }
-                            __builtin_amdgcn_s_waitcnt(0);       // loads and a varying number of stores: start over with only fetches in flight
+                            acc_a = acc_b = (float4_t){0.f, 0.f, 0.f, 0.f};
+                            c_pair = next_a;
+                            next_a = next_b;
+                            --queued;
                         }
-                        acc_a = acc_b = (float4_t){0.f, 0.f, 0.f, 0.f};
-                        c_pair = next_a;
-                        next_a = next_b;
-                        --queued;
-                    }
+                    };
+                    if (plain_out) run_pairs(std::true_type{});
+                    else run_pairs(std::false_type{});
                 }
             } else if (!aborted) {
                 bool staged = false;
@@ -1036,7 +1051,7 @@ struct StreamKernel {
     // slice has fewer row pairs than wavefronts); batch 1  32 layers 1.8 % slower, one layer 21.0 against 18.9 (the
     // stores of a pair stop its fetches, and one batch row has little to flush): the builder asks for it at batch 4
     // and, for long lists, at batch 2.
-    static constexpr bool kHasOwn = kArith == 2 && (BATCH == 2 || BATCH == 4);
+    static constexpr bool kHasOwn = kArith == 2 && BATCH <= 4;
     static constexpr auto fn_tiled_own = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2, false, kHasOwn>;
     static constexpr auto fn_tiled_own_det = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2, kHasOwn, kHasOwn>;
     static constexpr auto fn_single = gemv_stream_kernel<DT, BATCH, kArith, kThreads, true, false>;

@@ -340,12 +340,12 @@ def test_column_shares_of_short_slices(dev, batch, dtype, tiled):
 def test_batch_4_lists_choose_their_arithmetic_by_length(dev, dtype):
     # fp16 at batch 4: a list with little work per workgroup runs on the 16-bit arithmetic (bit 4 of the plan's flag
     # word), a long one on the fp4 x fp8 arithmetic; bf16 lists always on the latter.  The fp4 x fp8 kernel whose
-    # wavefronts own whole row pairs (bit 5) takes every tile-order list at batch 4 and long ones at batch 2.  All
+    # wavefronts own whole row pairs (bit 5) takes every tile-order list at batch 4 and long ones at batch 1 and 2.  All
     # against the oracle.
     to = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev).to(dtype)
     f64 = lambda t: t.float().cpu().numpy().astype(np.float64)
     m, n, r = 520, 8192, 2000
-    for batch, count in ((4, 1), (4, 64), (2, 1), (2, 96)):
+    for batch, count in ((4, 1), (4, 64), (2, 1), (2, 96), (1, 1), (1, 96)):
         rl = DecodeRunList(batch, dtype, dev)
         checked = {}
         for i in range(count):
