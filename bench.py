@@ -29,7 +29,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the headline kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
 # copy kernel of known size (profiles/gemv_stream_llama2_7b_stack_b1.md); valid for the default workload only.
-MEASURED_TRAFFIC_BYTES = 840352768
+MEASURED_TRAFFIC_BYTES = 843630592
 # The same for the two launches of the 128-token grouped layer (profiles/gemm_group_llama2_7b_layer_prefill.md):
 # (18776 + 27306) KiB x 2.000 fetched + (4352 + 10624) KiB written.
 MEASURED_PREFILL_TRAFFIC_BYTES = (18776 + 27306) * 2 * 1024 + (4352 + 10624) * 1024
@@ -299,7 +299,7 @@ def main():
         "us_per_layer": round(ms * 1e3 / nlayers, 3),
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_stream_kernel<fp16, batch 1, fp4 x fp8 MFMA, 1024 lanes, tile order> (one launch per token step: "
+            "kernel": "gemv_stream_kernel<fp16, batch 1, fp4 x fp8 MFMA, 1024 lanes, tile order, owned row pairs> (one launch per token step: "
                       "%d stages in 2 phases, 256 resident workgroups)" % (14 * nlayers),
             "achieved": round(gbs, 2),
             "peak": HBM_PEAK_GBS,
@@ -370,8 +370,9 @@ def main():
         ms_det = timed_launches(st_det.run, 10, 2) / len(layers)
         extra["batch1_deterministic"] = {"us_per_layer": round(ms_det * 1e3, 3),
                                          "GBps": round(bytes1 / (ms_det * 1e-3) / 1e9, 2),
-                                         "note": "DecodeRunList(deterministic=True): partial sums rounded to a grid on which "
-                                                 "additions are exact"}
+                                         "note": "DecodeRunList(deterministic=True): every sum formed in a fixed order (long tile-order "
+                                                 "lists: one wavefront per row pair; otherwise partial sums rounded to a "
+                                                 "grid on which additions are exact)"}
         del st_det
         # the same layer as ONE launch per layer (14 stages in 2 phases), rotating over the weight copies: what a
         # caller gets who launches layer by layer; bound by the serial latencies inside a launch, not by HBM
