@@ -623,7 +623,8 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                     const int nrows = seg.row_end - seg.row_begin;
                     const int npairs = (nrows + 31) >> 5;
                     const int ngroups = (cu_n + 3) >> 2;
-                    const int positions = (ngroups + 2) / 3 * 3;       // the three register pairs keep their turns from pair to pair
+                    constexpr int kOwnDepth = 3;                       // item fetches in flight per wavefront (2 or 3; 2 measures the same at batch 1, -1.5 % at batch 2, +1.4 % at batch 4)
+                    const int positions = (ngroups + kOwnDepth - 1) / kOwnDepth * kOwnDepth;   // the register pairs keep their turns from pair to pair
                     // results that need only their row scale go out as buffer stores (see the end of a pair)
                     const size_t out_elems = (size_t)(BATCH - 1) * st.out_stride + st.rows;
                     const bool plain_out = vec_rows && (nrows & 31) == 0 && st.s_row && !st.bias && !st.addend && out_elems < (1u << 28);
@@ -677,8 +678,10 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                         fetch(wa0, wb0);
                         if (j + 1 < ngroups) work(wa1, wb1, j + 1);
                         fetch(wa1, wb1);
-                        if (j + 2 < ngroups) work(wa2, wb2, j + 2);
-                        fetch(wa2, wb2);
+                        if constexpr (kOwnDepth == 3) {
+                            if (j + 2 < ngroups) work(wa2, wb2, j + 2);
+                            fetch(wa2, wb2);
+                        }
                     };
                     // PLAIN: every pair of the slice is whole and nothing but the row scale is applied on the way out.
                     // The scales then come through the scalar cache (64 bytes per pair, the same for every lane) and the
@@ -712,13 +715,14 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                             __builtin_amdgcn_raw_buffer_store_b64(hb, rout, o16 + 32u, 0, kCacheDefault);
                         };
                         __builtin_amdgcn_s_waitcnt(0);           // what the staging loaded has been used: see the tile-order loop below
-                        fetch(wa0, wb0); fetch(wa1, wb1); fetch(wa2, wb2);
+                        fetch(wa0, wb0); fetch(wa1, wb1);
+                        if constexpr (kOwnDepth == 3) fetch(wa2, wb2);
                         if constexpr (PLAIN) store_pair(0u, false, acc_a, acc_b);
 #pragma unroll 1
                         while (c_pair < npairs) {
                             if constexpr (PLAIN && kOwnExactWaits) three_items(0);
 #pragma unroll 1
-                            for (int j = PLAIN && kOwnExactWaits ? 3 : 0; j < positions; j += 3) three_items(j);
+                            for (int j = PLAIN && kOwnExactWaits ? kOwnDepth : 0; j < positions; j += kOwnDepth) three_items(j);
                             // acc_a[v]: row 32 pair + 4 g + v (acc_b: 16 rows further), column r16; the sum over the pieces
                             // of a batch row is valid in the lane of its last piece
                             float4_t sa, sb;
