@@ -492,6 +492,45 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                         if (row0 < seg.row_end) emit4(row0, r16, sum + xt);
                     }
                 };
+                // The same for a whole group whose results need nothing but their row scale (no bias, no addend, 8-byte
+                // aligned rows), without a load or a varying number of stores among the lane memory operations, so that
+                // the item fetches in flight need not be waited for: the 16 scales come through the scalar cache, the
+                // results leave as two buffer stores per lane, one per output type, past the end of the buffer for the
+                // other type and for the lanes that hold no batch row.
+                const int nrows16 = seg.row_end - seg.row_begin;
+                const size_t out_elems = (size_t)(BATCH - 1) * st.out_stride + st.rows;
+                const bool plain_out = vec_rows && st.s_row && !st.bias && !st.addend && out_elems < (1u << 28);
+                const __amdgpu_buffer_rsrc_t rout = raw_buffer(st.out, (uint32_t)(out_elems * (st.out_f32 ? 4u : 2u)));
+                const uint32_t past32 = st.out_f32 ? 0u : kPastEnd, past16 = st.out_f32 ? kPastEnd : 0u;
+                auto store_group_plain = [&](int grow, const float4_t& bsum) __attribute__((always_inline)) {
+                    typedef const uint32_t __attribute__((address_space(4)))* scalar_words_t;
+                    const int prow = seg.row_begin + __builtin_amdgcn_readfirstlane(grow);
+                    const scalar_words_t sp = (scalar_words_t)(uintptr_t)(st.s_row + prow);
+                    uint32_t sw[8];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        sw[i] = sp[i];
+                        asm volatile("" : "+s"(sw[i]));                  // kept in scalar registers: one scalar load each
+                    }
+                    uint32_t s0 = sw[0], s1 = sw[1];                     // rows 4g .. 4g + 3
+#pragma unroll
+                    for (int q = 1; q < 4; ++q) {
+                        s0 = g == q ? sw[2 * q] : s0;
+                        s1 = g == q ? sw[2 * q + 1] : s1;
+                    }
+                    float4_t v = bsum * -2.f + xtot[min(r16, BATCH - 1)];
+                    v[0] *= E::to_float((uint16_t)(s0 & 0xFFFFu)); v[1] *= E::to_float((uint16_t)(s0 >> 16));
+                    v[2] *= E::to_float((uint16_t)(s1 & 0xFFFFu)); v[3] *= E::to_float((uint16_t)(s1 >> 16));
+                    const bool live = r16 < BATCH;
+                    const uint32_t elem = (uint32_t)min(r16, BATCH - 1) * (uint32_t)st.out_stride + (uint32_t)(prow + 4 * g);
+                    const uint32_t o32 = live ? (elem * 4u) | past32 : kPastEnd;
+                    const uint32_t o16 = live ? (elem * 2u) | past16 : kPastEnd;
+                    const u32x4_t f = {as_bits(v[0]), as_bits(v[1]), as_bits(v[2]), as_bits(v[3])};
+                    __builtin_amdgcn_raw_buffer_store_b128(f, rout, o32, 0, kCacheAgentCoherent);   // fp32: read by other workgroups
+                    const u32x2_t h = {(uint32_t)E::from_float_clamped(v[0]) | ((uint32_t)E::from_float_clamped(v[1]) << 16),
+                                       (uint32_t)E::from_float_clamped(v[2]) | ((uint32_t)E::from_float_clamped(v[3]) << 16)};
+                    __builtin_amdgcn_raw_buffer_store_b64(h, rout, o16, 0, kCacheDefault);
+                };
                 // The groups [q_begin, q_end) of this wavefront times the unit groups of the staged chunk (c0, cu_n).
                 // Items = (row group, 4-unit group), unit group fastest.  Three item fetches (1 KB of packed words each) in
                 // flight, in three register sets that take turns, each refilled right after its use; a row group is
@@ -553,10 +592,15 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                             fetch(w2);
                         }
                         if (complete && !split) {
-                            store_group(q, pow2_combine<DT>(acc));
+                            const int grow = 16 * (grp + kWaves * q);
+                            if (plain_out && grow + 16 <= nrows16) {
+                                store_group_plain(grow, pow2_combine<DT>(acc));
+                            } else {
+                                store_group(q, pow2_combine<DT>(acc));
+                                __builtin_amdgcn_s_waitcnt(0);           // loads and a varying number of stores behind the fetches
+                            }
 #pragma unroll
                             for (int k = 0; k < kAccs; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
-                            __builtin_amdgcn_s_waitcnt(0);
                         }
                     }
                 };
