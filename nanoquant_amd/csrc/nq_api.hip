@@ -417,8 +417,9 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         // the resident workgroups.
         {
             // (the variant whose wavefronts own row pairs starts every slice without fetches in flight: 16000, from
-            // sweeps of the Llama-2-7B stack at batch 4 and 2: 5.8 against 5.95 and 5.3 against 5.45 us per layer)
-            const long long fixed = own ? 16000 : wide ? 2200 : batch == 1 ? 8800 : batch == 2 ? 6600 : 4400;
+            // sweeps of the Llama-2-7B stack at batch 4 and 2: 5.8 against 5.95 and 5.3 against 5.45 us per layer;
+            // at batch 1 6000 / 10000 / 16000 / 24000 / 40000 give 6120 / 6149 / 6085 / 5990 / 5709 GB/s on that stack)
+            const long long fixed = own ? (batch == 1 ? 10000 : 16000) : wide ? 2200 : batch == 1 ? 8800 : batch == 2 ? 6600 : 4400;
             auto gran = [&](size_t k) { return table[ids[k]].tiled ? granule : 1; };
             // Batch 8 and 16: an input too long to be staged at once is staged again, chunk by chunk, for every 256 rows
             // of a slice (three barriers and a round trip to memory per chunk): charged as 10 more units per chunk and
