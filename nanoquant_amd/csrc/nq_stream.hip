@@ -667,7 +667,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                     const int nrows = seg.row_end - seg.row_begin;
                     const int npairs = (nrows + 31) >> 5;
                     const int ngroups = (cu_n + 3) >> 2;
-                    constexpr int kOwnDepth = 3;                       // item fetches in flight per wavefront (2 or 3; 2 measures the same at batch 1, -1.5 % at batch 2, +1.4 % at batch 4)
+                    constexpr int kOwnDepth = 3;                       // item fetches in flight per wavefront (2 against 3: within +-1.5 % at batch 1, 2 and 4)
                     const int positions = (ngroups + kOwnDepth - 1) / kOwnDepth * kOwnDepth;   // the register pairs keep their turns from pair to pair
                     // results that need only their row scale go out as buffer stores (see the end of a pair)
                     const size_t out_elems = (size_t)(BATCH - 1) * st.out_stride + st.rows;
