@@ -230,6 +230,27 @@ int nq_gemm_group_max(void);
 int nq_gemm_nanoquant_group(const nq_gemm_term* terms, int count, int tokens, int dtype, void* scratch,
                             size_t scratch_bytes, void* stream);
 
+/* The same with a workspace for the panel launches.  Around 128 tokens (96..128) a group that gives every compute
+ * unit a few k steps of work runs each of its two stages as ONE persistent launch over panels of 128 tokens x 256
+ * rows whose k ranges are shared out evenly over the compute units (what the reference's stream-k stripes do,
+ * kernel/cuda/gemm_kernel.cu:335-400, :594-640): panels cut by a share boundary hand their partial fp32 tiles to
+ * the workgroup that finishes them through `panel_ws`.
+ *   panel_ws: nq_gemm_panel_workspace_bytes() bytes of device memory, 256-byte aligned, ZERO when first used and
+ *   left to these launches from then on (it holds partial tiles, hand-over flags and a count of finished
+ *   workgroups from which every launch derives its own flag value, so nothing is cleared between launches or graph
+ *   replays).  It must not be `scratch` and launches that share it must not overlap in time.
+ *   panel_mode: NQ_PANEL_AUTO picks per stage (other token counts and small groups take the launches of
+ *   nq_gemm_nanoquant_group), NQ_PANEL_ALWAYS forces the panel launch for any token count, NQ_PANEL_NEVER (or
+ *   panel_ws NULL) never takes it.
+ * The waits of a finishing workgroup are bounded; nq_gemm_panel_status copies the workspace's status word back
+ * (synchronises) and clears it: 0 ok, 1 = a wait expired in some launch since the last call (that launch's outputs
+ * are invalid; the workspace stays usable). */
+enum { NQ_PANEL_AUTO = 0, NQ_PANEL_ALWAYS = 1, NQ_PANEL_NEVER = 2 };
+size_t nq_gemm_panel_workspace_bytes(void);
+int nq_gemm_nanoquant_group_ws(const nq_gemm_term* terms, int count, int tokens, int dtype, void* scratch,
+                               size_t scratch_bytes, void* panel_ws, size_t panel_ws_bytes, int panel_mode, void* stream);
+int nq_gemm_panel_status(const void* panel_ws, int* status_out, void* stream);
+
 /* Word-order conversion on the device, in place allowed (dst == src): the checkpoint format
  * ("lsb_first", modules/linear.py:298) to the kernel format ("half2", modules/linear.py:171-172)
  * without the dense round trip of utils/load_utils.py:269-293.  order ids: nq_word_order. */

@@ -41,6 +41,9 @@ _SIGNATURES = {
     "nq_repack_words": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
     "nq_gemm_group_max": (_i, []),
     "nq_gemm_nanoquant_group": (_i, [_vp, _i, _i, _i, _vp, _sz, _vp]),
+    "nq_gemm_panel_workspace_bytes": (_sz, []),
+    "nq_gemm_nanoquant_group_ws": (_i, [_vp, _i, _i, _i, _vp, _sz, _vp, _sz, _i, _vp]),
+    "nq_gemm_panel_status": (_i, [_vp, ctypes.POINTER(_i), _vp]),
     "nq_pack_gemm_tiles": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "nq_tiled_words": (_sz, [_i, _i]),
     "nq_tile_words": (_i, [_vp, _vp, _i, _i, _i, _vp]),

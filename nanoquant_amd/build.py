@@ -10,7 +10,7 @@ from concurrent.futures import ThreadPoolExecutor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libnq_gfx950.so")
-SOURCES = ("nq_gemv.hip", "nq_stream.hip", "nq_gemm.hip", "nq_util.hip", "nq_api.hip")
+SOURCES = ("nq_gemv.hip", "nq_stream.hip", "nq_gemm.hip", "nq_panel.hip", "nq_util.hip", "nq_api.hip")
 # -packed-fp32-ops off: hipcc may otherwise fuse scalar float code into packed-fp32 instructions.
 FLAGS = ("--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-munsafe-fp-atomics",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops")

@@ -41,7 +41,7 @@ const char* nq_status_string(int status) {
 
 int nq_last_hip_error(void) { return g_last_hip_error; }
 
-int nq_abi_version(void) { return 7; }
+int nq_abi_version(void) { return 8; }
 
 int nq_device_query(int attr, int* value) {
     if (!value) return NQ_ERR_NULL;
@@ -612,8 +612,31 @@ int nq_gemm_group_max(void) { return nq::gemm_group_max(); }
 
 int nq_gemm_nanoquant_group(const nq_gemm_term* terms, int count, int tokens, int dtype, void* scratch,
                             size_t scratch_bytes, void* stream) {
+    return nq_gemm_nanoquant_group_ws(terms, count, tokens, dtype, scratch, scratch_bytes, nullptr, 0, NQ_PANEL_NEVER, stream);
+}
+
+size_t nq_gemm_panel_workspace_bytes(void) { return nq::panel_workspace_bytes(); }
+
+int nq_gemm_panel_status(const void* panel_ws, int* status_out, void* stream) {
+    if (!panel_ws || !status_out) return NQ_ERR_NULL;
+    unsigned v = 0;
+    const char* word = (const char*)panel_ws + 64;
+    hipError_t e = hipMemcpyAsync(&v, word, sizeof(v), hipMemcpyDeviceToHost, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_status(e);
+    e = hipStreamSynchronize((hipStream_t)stream);
+    *status_out = (int)v;
+    if (e == hipSuccess && v != 0) {                 // read and clear
+        e = hipMemsetAsync(const_cast<char*>(word), 0, sizeof(v), (hipStream_t)stream);
+        if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
+    }
+    return hip_status(e);
+}
+
+int nq_gemm_nanoquant_group_ws(const nq_gemm_term* terms, int count, int tokens, int dtype, void* scratch,
+                               size_t scratch_bytes, void* panel_ws, size_t panel_ws_bytes, int panel_mode, void* stream) {
     if (dtype != NQ_F16 && dtype != NQ_BF16) return NQ_ERR_DTYPE;
     if (count < 0 || tokens < 0) return NQ_ERR_SHAPE;
+    if (panel_mode != NQ_PANEL_AUTO && panel_mode != NQ_PANEL_ALWAYS && panel_mode != NQ_PANEL_NEVER) return NQ_ERR_SHAPE;
     if (count == 0 || tokens == 0) return NQ_OK;
     if (!terms) return NQ_ERR_NULL;
     if (count > nq::gemm_group_max()) return NQ_ERR_SHAPE;
@@ -644,17 +667,29 @@ int nq_gemm_nanoquant_group(const nq_gemm_term* terms, int count, int tokens, in
     const void* x[kMax]; const uint32_t* w[kMax]; const void* si[kMax]; const void* so[kMax]; const void* bs[kMax]; void* out[kMax];
     int K[kMax], R[kMax];
     if (count > kMax) return NQ_ERR_SHAPE;
+    const bool have_ws = panel_ws && panel_mode != NQ_PANEL_NEVER;
+    if (have_ws) {
+        if (((uintptr_t)panel_ws) & 255u) return NQ_ERR_ALIGN;
+        const size_t need = nq::panel_workspace_bytes();
+        if (need == 0 || panel_ws_bytes < need) return NQ_ERR_WORKSPACE;
+    }
+    // one stage: the panel launch where a workspace was given and the shapes make it the faster one
+    auto stage = [&]() -> hipError_t {
+        if (have_ws && (panel_mode == NQ_PANEL_ALWAYS || nq::panel_applies(count, tokens, K, R)))
+            return nq::gemm_panel_group(dtype, count, x, w, si, so, bs, out, tokens, K, R, panel_ws, 0u, (hipStream_t)stream);
+        return nq::gemm_onebit_group(dtype, count, x, w, si, so, bs, out, tokens, K, R, (hipStream_t)stream);
+    };
     for (int i = 0; i < count; ++i) {
         const nq_gemm_term& t = terms[i];
         x[i] = t.x; w[i] = t.vt_tiles; si[i] = t.s_in; so[i] = t.s_mid; bs[i] = nullptr; out[i] = t.h; K[i] = t.n; R[i] = t.r;
     }
-    hipError_t e = nq::gemm_onebit_group(dtype, count, x, w, si, so, bs, out, tokens, K, R, (hipStream_t)stream);
+    hipError_t e = stage();
     if (e != hipSuccess) return hip_status(e);
     for (int i = 0; i < count; ++i) {
         const nq_gemm_term& t = terms[i];
         x[i] = t.h; w[i] = t.u_tiles; si[i] = nullptr; so[i] = t.s_out; bs[i] = t.bias; out[i] = t.y; K[i] = t.r; R[i] = t.m;
     }
-    return hip_status(nq::gemm_onebit_group(dtype, count, x, w, si, so, bs, out, tokens, K, R, (hipStream_t)stream));
+    return hip_status(stage());
 }
 
 size_t nq_tiled_words(int rows, int words) {

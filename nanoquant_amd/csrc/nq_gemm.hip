@@ -20,6 +20,7 @@
 // and converts (and re-zeroes the scratch, which must be zero on entry).
 #include "nq_common.h"
 #include "nq_kernels.h"
+#include "nq_mfma.h"
 
 namespace nq {
 
@@ -36,34 +37,6 @@ struct GemmArgs {
     int ktiles_per_split;
     int xcd_gx;             // > 0: flat grid, token blocks dealt to the 8 XCDs; value = row blocks
 };
-
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-
-constexpr int kTileK = 256;  // k extent of one packed weight tile (and the granularity of k-splits)
-
-// LDS row pitch in 16-bit elements for a slab of KS k-values: 16 bytes of padding make the 128-bit
-// fragment reads of 32 consecutive rows conflict-free.
-template <int KS>
-constexpr int slab_pitch() { return KS + 8; }
-
-template <int DT>
-struct Mfma;
-template <>
-struct Mfma<0> {
-    static __device__ __forceinline__ float16_t run(uint4 a, uint4 b, float16_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
-    }
-};
-template <>
-struct Mfma<1> {
-    static __device__ __forceinline__ float16_t run(uint4 a, uint4 b, float16_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf168_t, a), __builtin_bit_cast(bf168_t, b), c, 0, 0, 0);
-    }
-};
-
-__device__ __forceinline__ uint32_t comp4(const uint4& v, int i) {
-    return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
-}
 
 // Issues the global loads of one activation slab [32*TT tokens][KS k] starting at k0 (and its KS input
 // scales) into registers; nothing waits on them here.

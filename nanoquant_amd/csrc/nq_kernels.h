@@ -83,6 +83,15 @@ hipError_t gemm_onebit_group(int dtype, int count, const void* const* x, const u
                              const void* const* s_in, const void* const* s_out, const void* const* bias, void* const* y,
                              int T, const int* K, const int* R, hipStream_t stream);
 
+// nq_panel.hip: the same GEMMs at about 128 tokens as one persistent launch over 128-token x 256-row panels
+// (see the file header).  workspace: panel_workspace_bytes() bytes, zero when first used.
+size_t panel_workspace_bytes();
+int panel_max_tokens();
+bool panel_applies(int count, int T, const int* K, const int* R);
+hipError_t gemm_panel_group(int dtype, int count, const void* const* x, const uint32_t* const* tiles,
+                            const void* const* s_in, const void* const* s_out, const void* const* bias, void* const* y,
+                            int T, const int* K, const int* R, void* workspace, unsigned spin_limit, hipStream_t stream);
+
 // nq_util.hip
 hipError_t stream_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);
 hipError_t repack_words(const uint32_t* src, uint32_t* dst, size_t nwords, int src_order, int dst_order,

@@ -226,6 +226,39 @@ def _scratch(nbytes, device):
     return buf
 
 
+# Workspace of the panel launches (partial tiles, hand-over flags, the count of finished workgroups): zero when
+# first used, then owned by the launches; one per (device, stream) so that launches sharing it are stream-ordered.
+_panel_ws_cache = {}
+PANEL_MODES = {"auto": 0, "always": 1, "never": 2}
+
+
+def _panel_workspace(device):
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    buf = _panel_ws_cache.get(key)
+    if buf is None:
+        with torch.cuda.device(device):
+            nbytes = int(_lib.lib().nq_gemm_panel_workspace_bytes())
+        if nbytes == 0:
+            raise RuntimeError("nq_gemm_panel_workspace_bytes() returned 0: no usable device")
+        buf = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        _panel_ws_cache[key] = buf
+    return buf
+
+
+def panel_status(device=None) -> int:
+    """Status word of the current stream's panel workspace (synchronises; reads and clears): 0 ok, 1 = a bounded
+    wait of a panel launch expired since the last call and that launch's outputs are invalid."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    buf = _panel_ws_cache.get(key)
+    if buf is None:
+        return 0
+    out = ctypes.c_int(0)
+    with torch.cuda.device(device):
+        _lib.check(_lib.lib().nq_gemm_panel_status(_ptr(buf), ctypes.byref(out), _stream(device)))
+    return int(out.value)
+
+
 def marlin_onebit_forward(x, weight, scale_g, scale_h, workspace):
     """C[m, n] = s_out[n] * sum_k (x[m, k] * s_in[k]) * sgn(weight)[n, k]; weight from marlin_onebit_packer."""
     dt = _gemm_dtype(x)
@@ -308,12 +341,14 @@ class NqGemmTerm(ctypes.Structure):
                 ("n", ctypes.c_int), ("r", ctypes.c_int), ("m", ctypes.c_int)]
 
 
-def gemm_group_forward(xs, terms, biases=None, outs=None):
+def gemm_group_forward(xs, terms, biases=None, outs=None, panel="auto"):
     """Several `marlin_nanoquant_forward` calls on the same number of tokens in two launches instead of two per
     call: `terms` is a list of argument tuples (weight_u, weight_v, scale_g, scale_l, scale_h, workspace) as that
     op takes them after x; `xs` is one tensor [tokens, n] read by every term or a list of one tensor per term;
     `biases` an optional list of [m] tensors / None; `outs` an optional list of contiguous [tokens, m] tensors of
-    the activation type to write into (allocated here when absent).  Returns the list of outputs.  The terms share
+    the activation type to write into (allocated here when absent); `panel` ("auto", "always", "never") says whether
+    the stages may run as persistent panel launches (around 128 tokens, see include/nq_gfx950.h).  Returns the list of
+    outputs.  The terms share
     launches (a single linear leaves most of the device idle up to some hundred tokens): few-token tiles up to 160
     tokens, 64-token block tiles without k-split above.  The
     reference launches every linear by itself (modules/linear.py:131-133)."""
@@ -360,11 +395,14 @@ def gemm_group_forward(xs, terms, biases=None, outs=None):
     device = xs[0].device
     group_max = int(lib.nq_gemm_group_max())
     scratch = _scratch(nbytes, device)
+    mode = PANEL_MODES[panel]
+    ws = None if mode == 2 else _panel_workspace(device)
     with torch.cuda.device(device):
         for lo in range(0, count, group_max):
             part = arr_items[lo:lo + group_max]
             arr = (NqGemmTerm * len(part))(*part)
-            _lib.check(lib.nq_gemm_nanoquant_group(arr, len(part), tokens, dt, _ptr(scratch), nbytes, _stream(device)))
+            _lib.check(lib.nq_gemm_nanoquant_group_ws(arr, len(part), tokens, dt, _ptr(scratch), nbytes, _ptr(ws),
+                                                      0 if ws is None else ws.numel(), mode, _stream(device)))
     return outs
 
 
