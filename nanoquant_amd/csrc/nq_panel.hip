@@ -55,8 +55,8 @@ struct PanelArgs {
     PanelProblem p[kPanelMax];
     int T, tblocks, total_units;
     unsigned spin_limit;
-    float* partials;                 // [G][kPanelSlotFloats]
-    unsigned* flags;                 // [G][kPanelFlagStride]
+    float* partials;                 // [2 G][kPanelSlotFloats]: slot 2 w for the first segment of workgroup w, 2 w + 1 for its last
+    unsigned* flags;                 // [2 G][kPanelFlagStride]
     unsigned long long* exit_count;  // workgroup exits of all launches on this workspace
     unsigned* status;
 };
@@ -172,6 +172,7 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
             arb = 0;
             ++ap;
         };
+        if (u + 1 < u_end) advance(p1, rb1, tb1, kt1);
         // The MFMAs of one unit; with `fetch_next` the loads of the next unit's slab and weight tiles are issued
         // between the first k steps, one instruction per step, so that no wavefront queues behind a burst of loads.
         auto compute = [&](const uint16_t* slab, const u32x4_t (&w)[2], bool fetch_next, const SlabFetch& nf) {
@@ -229,9 +230,10 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
         // Accumulator element v of lane l of tile (r, tt): token 64 th + 32 tt + 8 (v >> 2) + 4 (l >> 5) + (v & 3),
         // row 32 (8 rb + 2 rq + r) + (l & 31).  A tile is scaled, converted and turned round in the wavefront's
         // staging area (rows of one token next to each other), then leaves as 16-byte stores: lane l stores rows
-        // 8 (l & 3) .. + 7 of token (l >> 2) and of token 16 + (l >> 2).  Always 8 store instructions per wavefront:
-        // tokens beyond T and row tiles beyond R are pointed past the end of the buffer and dropped.
-        auto epilogue = [&](int ep, int erb, int etb) {
+        // 8 (l & 3) .. + 7 of token (l >> 2) and of token 16 + (l >> 2).  With all four tiles in `tile_mask` always 8
+        // store instructions per wavefront: tokens beyond T and row tiles beyond R are pointed past the end of the
+        // buffer and dropped.
+        auto epilogue = [&](int ep, int erb, int etb, unsigned tile_mask) {
             const PanelProblem& P = g.p[ep];
             uint16_t* stage = panel_lds + 2 * kPanelBufHalves + wave * kPanelStageHalves;
             const uint32_t row_bytes = (uint32_t)P.R * 2u;
@@ -245,6 +247,7 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
                 if (live && P.bias) bs = E::to_float(P.bias[row0 + (lane & 31)]);
 #pragma unroll
                 for (int tt = 0; tt < 2; ++tt) {
+                    if (!((tile_mask >> (2 * r + tt)) & 1u)) continue;        // finished by another workgroup
 #pragma unroll
                     for (int v = 0; v < 16; ++v)
                         stage[(8 * (v >> 2) + 4 * hi + (v & 3)) * kPanelStagePitch + (lane & 31)] = E::from_float_sat(acc[r][tt][v] * sc + bs);
@@ -263,8 +266,8 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
         auto partial_rsrc = [&](int slot) {
             return gemm_buffer(g.partials + (size_t)slot * kPanelSlotFloats, (uint32_t)(kPanelSlotFloats * sizeof(float)));
         };
-        auto write_partial = [&]() {
-            const __amdgpu_buffer_rsrc_t rs = partial_rsrc(wg);
+        auto write_partial = [&](int slot) {
+            const __amdgpu_buffer_rsrc_t rs = partial_rsrc(slot);
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int r = i >> 3, tt = (i >> 2) & 1, j = i & 3;
@@ -277,27 +280,32 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
                 __builtin_amdgcn_raw_buffer_store_b128(v, rs, (uint32_t)lane * 16u, (uint32_t)(wave * 16 + i) * 1024u, kGemmCacheAgent);
             }
         };
-        auto add_partial = [&](int slot) {
-            const __amdgpu_buffer_rsrc_t rs = partial_rsrc(slot);
-            u32x4_t v[16];
+        // adds tile q = 2 r + tt (four 16-byte pieces per lane) of the partial tiles in slots sa and sb to this
+        // wavefront's accumulators; both sets of loads are in flight together (sb < 0: only sa)
+        auto add_partial_tile = [&](int q, int sa, int sb) {
+            const __amdgpu_buffer_rsrc_t ra = partial_rsrc(sa);
+            const __amdgpu_buffer_rsrc_t rb_ = partial_rsrc(sb < 0 ? sa : sb);
+            const uint32_t off_b = sb < 0 ? 0xFFFFFFF0u : (uint32_t)lane * 16u;     // past the end: reads zeros
+            u32x4_t va[4], vb[4];
 #pragma unroll
-            for (int i = 0; i < 16; ++i)
-                v[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, (uint32_t)lane * 16u, (uint32_t)(wave * 16 + i) * 1024u, kGemmCacheAgent);
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int r = i >> 3, tt = (i >> 2) & 1, j = i & 3;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const uint32_t bits = v[i][e];
-                    acc[r][tt][4 * j + e] += __builtin_bit_cast(float, bits);
-                }
+            for (int j = 0; j < 4; ++j) {
+                va[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, (uint32_t)lane * 16u, (uint32_t)(wave * 16 + q * 4 + j) * 1024u, kGemmCacheAgent);
+                vb[j] = __builtin_amdgcn_raw_buffer_load_b128(rb_, off_b, (uint32_t)(wave * 16 + q * 4 + j) * 1024u, kGemmCacheAgent);
             }
+#pragma unroll
+            for (int r = 0; r < 2; ++r)
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt) {
+                    if (2 * r + tt != q) continue;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint32_t xa = va[j][e], xb = vb[j][e];
+                            acc[r][tt][4 * j + e] += __builtin_bit_cast(float, xa) + __builtin_bit_cast(float, xb);
+                        }
+                }
         };
-
-        // Software pipeline over the units u of this workgroup: at the start of unit u the slab and the weight tiles
-        // of unit u + 1 are asked for (the slab straight into the LDS buffer that unit u - 1 has left), they arrive
-        // while the MFMAs of unit u run from the other buffer.  One barrier per unit.
-        if (u + 1 < u_end) advance(p1, rb1, tb1, kt1);
         // The loads of the next slab write LDS behind the compiler's back; it would make every LDS read that follows
         // them wait for them unless it can see that the two do not overlap.  The __restrict__ parameters say so: the
         // buffer the MFMAs read and the buffer the loads fill are different halves of the LDS allocation.
@@ -326,38 +334,83 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
             unit_body(panel_lds + cur * kPanelBufHalves, panel_lds + (cur ^ 1) * kPanelBufHalves, more);
             int stores = 0;       // store instructions of this wavefront issued behind the loads above
             if (last_kt || !more) {
-                if (seg_kt0 == 0) {
-                    if (!last_kt) {
-                        // owner of a panel whose later k tiles belong to the workgroups behind this one, up to the one
-                        // that holds the panel's last unit
-                        const long long panel_end = (long long)(u - kt) + kts;
-                        const int last = (int)((panel_end * G - 1) / U);
-                        bool ok = true;
-#pragma unroll 1
-                        for (int c = wg + 1; c <= last && ok; ++c) {
-                            if ((long long)c * U / G == (long long)(c + 1) * U / G) continue;   // a workgroup without units
-                            unsigned spins = 0;
-                            while (true) {
-                                unsigned f = 0;
-                                if (lane == 0) f = __hip_atomic_load(g.flags + (size_t)c * kPanelFlagStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                                f = (unsigned)__builtin_amdgcn_readfirstlane((int)f);
-                                if (f == gen) break;
-                                __builtin_amdgcn_s_sleep(4);
-                                if (++spins >= g.spin_limit) {       // bounded wait: report, finish with what is there
-                                    if (lane == 0) atomicOr(g.status, 1u);
-                                    ok = false;
-                                    break;
-                                }
-                            }
-                            if (ok) add_partial(c);
-                        }
-                    }
-                    epilogue(p, rb, tb);
+                if (seg_kt0 == 0 && last_kt) {
+                    epilogue(p, rb, tb, 0xFu);            // the whole k range of the panel was this workgroup's
                     stores = 8;
-                } else {
-                    write_partial();
+                } else if (last_kt) {
+                    // The last k tiles of a panel that began in earlier workgroups (always the first segment of a
+                    // range): hand the partial tile over and go on; the flag follows when the stores have arrived.
+                    write_partial(2 * wg);
                     flag_state = 1;
                     stores = 16;
+                } else {
+                    // The range ends inside the panel.  All workgroups in this position (the one with the panel's first
+                    // k tile and those that lie wholly inside it) finish the panel TOGETHER: each publishes its partial
+                    // tile, waits for everybody's, and sums and stores its share of the 32 output tiles (tile q of
+                    // wavefront w belongs to the workgroup with index (4 w + q) mod n among them), so that the time
+                    // of the reduction does not grow with the number of workgroups a long k range is shared by.
+                    // First raise the flag of this workgroup's earlier partial tile if that is still due: the
+                    // workgroups finishing THAT panel must not wait for what follows here.
+                    if (flag_state != 0) {
+                        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                        lds_barrier();
+                        if (tid == 0) __hip_atomic_store(g.flags + (size_t)(2 * wg) * kPanelFlagStride, gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        flag_state = 0;
+                    }
+                    auto has_units = [&](int c) { return (long long)c * U / G != (long long)(c + 1) * U / G; };
+                    const long long panel_first = (long long)(u - kt);
+                    const int w_first = (int)(((panel_first + 1) * G - 1) / U);
+                    const int w_last = (int)(((panel_first + kts) * G - 1) / U);      // holds the panel's last unit
+                    int n = 0, mine = 0;
+                    for (int c = w_first; c < w_last; ++c) {
+                        if (!has_units(c)) continue;
+                        if (c == wg) mine = n;
+                        ++n;
+                    }
+                    if (n > 1) {
+                        write_partial(2 * wg + 1);
+                        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                        lds_barrier();
+                        if (tid == 0) __hip_atomic_store(g.flags + (size_t)(2 * wg + 1) * kPanelFlagStride, gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    // everybody else's partial tile: the last workgroup's is the one of its first segment
+                    bool ok = true;
+#pragma unroll 1
+                    for (int c = w_first; c <= w_last && ok; ++c) {
+                        if (c == wg || !has_units(c)) continue;
+                        const unsigned* flag = g.flags + (size_t)(c == w_last ? 2 * c : 2 * c + 1) * kPanelFlagStride;
+                        unsigned spins = 0;
+                        while (true) {
+                            unsigned f = 0;
+                            if (lane == 0) f = __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            f = (unsigned)__builtin_amdgcn_readfirstlane((int)f);
+                            if (f == gen) break;
+                            __builtin_amdgcn_s_sleep(4);
+                            if (++spins >= g.spin_limit) {           // bounded wait: report, finish with what is there
+                                if (lane == 0) atomicOr(g.status, 1u);
+                                ok = false;
+                                break;
+                            }
+                        }
+                    }
+                    unsigned tile_mask = 0;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        if ((wave * 4 + q) % n != mine) continue;
+                        tile_mask |= 1u << q;
+                        if (!ok) continue;
+                        int held = -1;                    // a slot waiting for a partner to be loaded with
+#pragma unroll 1
+                        for (int c = w_first; c <= w_last; ++c) {
+                            if (c == wg || !has_units(c)) continue;
+                            const int slot = c == w_last ? 2 * c : 2 * c + 1;
+                            if (held < 0) { held = slot; continue; }
+                            add_partial_tile(q, held, slot);
+                            held = -1;
+                        }
+                        if (held >= 0) add_partial_tile(q, held, -1);
+                    }
+                    epilogue(p, rb, tb, tile_mask);
                 }
                 zero_acc();
                 seg_kt0 = 0;
@@ -372,7 +425,7 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
             w[0] = wn[0]; w[1] = wn[1];
             lds_barrier();
             if (flag_state == 2 && stores == 0) {
-                if (tid == 0) __hip_atomic_store(g.flags + (size_t)wg * kPanelFlagStride, gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (tid == 0) __hip_atomic_store(g.flags + (size_t)(2 * wg) * kPanelFlagStride, gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 flag_state = 0;
             }
             if (flag_state == 1) flag_state = 2;
@@ -384,7 +437,7 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
         if (flag_state != 0) {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             lds_barrier();
-            if (tid == 0) __hip_atomic_store(g.flags + (size_t)wg * kPanelFlagStride, gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (tid == 0) __hip_atomic_store(g.flags + (size_t)(2 * wg) * kPanelFlagStride, gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
     if (tid == 0) __hip_atomic_fetch_add(g.exit_count, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -405,8 +458,8 @@ static int panel_grid() {
 size_t panel_workspace_bytes() {
     const int G = panel_grid();
     if (G <= 0) return 0;
-    const size_t flags = ((size_t)G * kPanelFlagStride * sizeof(unsigned) + 255) / 256 * 256;
-    return kPanelHeadBytes + flags + (size_t)G * kPanelSlotFloats * sizeof(float);
+    const size_t flags = ((size_t)2 * G * kPanelFlagStride * sizeof(unsigned) + 255) / 256 * 256;
+    return kPanelHeadBytes + flags + (size_t)2 * G * kPanelSlotFloats * sizeof(float);
 }
 
 int panel_max_tokens() { return kPanelTok; }
@@ -470,7 +523,7 @@ hipError_t gemm_panel_group(int dtype, int count, const void* const* x, const ui
     a.total_units = (int)units;
     a.spin_limit = spin_limit ? spin_limit : (1u << 20);
     char* base = (char*)workspace;
-    const size_t flags = ((size_t)G * kPanelFlagStride * sizeof(unsigned) + 255) / 256 * 256;
+    const size_t flags = ((size_t)2 * G * kPanelFlagStride * sizeof(unsigned) + 255) / 256 * 256;
     a.exit_count = (unsigned long long*)base;
     a.status = (unsigned*)(base + 64);
     a.flags = (unsigned*)(base + kPanelHeadBytes);
