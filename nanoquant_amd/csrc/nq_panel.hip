@@ -105,6 +105,27 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
         }
 
         int p1 = p, rb1 = rb, tb1 = tb, kt1 = kt;     // unit u + 1 (where there is one)
+        // Fetching ahead: when this workgroup's range ends inside a panel that BEGINS in it and ends in the next
+        // workgroup (a short k range cut once), that workgroup's partial tile is usually there long before this one
+        // gets to the panel.  Its flag is looked at one unit ahead and, if set, the sixteen loads of the tile are issued
+        // in front of the last unit's MFMAs instead of behind them.  ahead_slot < 0: not that case.
+        int ahead_slot = -1;
+        if (u_end - u >= 2) {
+            const int lu = u_end - 1;
+            int lp = 0;
+#pragma unroll
+            for (int i = 1; i < kPanelMax; ++i) lp += lu >= g.p[i].first_unit ? 1 : 0;
+            const int lkts = g.p[lp].ktiles;
+            const int lkt = (lu - g.p[lp].first_unit) % lkts;
+            const long long lfirst = (long long)lu - lkt;
+            const int next = wg + 1;
+            if (lfirst >= u && lkt + 1 < lkts && next < G && (long long)next * U / G != (long long)(next + 1) * U / G &&
+                (int)(((lfirst + lkts) * G - 1) / U) == next)
+                ahead_slot = 2 * next;
+        }
+        unsigned ahead_flag = 0;
+        bool ahead_loaded = false;
+        u32x4_t ahead[8];             // the pieces of the tiles with r = 0; those with r = 1 follow behind the MFMAs
         float16_t acc[2][2];
         auto zero_acc = [&]() {
 #pragma unroll
@@ -331,6 +352,19 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
             const int kts = g.p[p].ktiles;
             const bool more = u + 1 < u_end;
             const bool last_kt = kt + 1 == kts;
+            if (ahead_slot >= 0) {
+                if (u + 2 == u_end) {
+                    if (lane == 0) ahead_flag = __hip_atomic_load(g.flags + (size_t)ahead_slot * kPanelFlagStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                } else if (u + 1 == u_end) {
+                    if ((unsigned)__builtin_amdgcn_readfirstlane((int)ahead_flag) == gen) {
+                        const __amdgpu_buffer_rsrc_t ra = partial_rsrc(ahead_slot);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i)
+                            ahead[i] = __builtin_amdgcn_raw_buffer_load_b128(ra, (uint32_t)lane * 16u, (uint32_t)(wave * 16 + i) * 1024u, kGemmCacheAgent);
+                        ahead_loaded = true;
+                    }
+                }
+            }
             unit_body(panel_lds + cur * kPanelBufHalves, panel_lds + (cur ^ 1) * kPanelBufHalves, more);
             int stores = 0;       // store instructions of this wavefront issued behind the loads above
             if (last_kt || !more) {
@@ -377,7 +411,7 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
                     bool ok = true;
 #pragma unroll 1
                     for (int c = w_first; c <= w_last && ok; ++c) {
-                        if (c == wg || !has_units(c)) continue;
+                        if (c == wg || !has_units(c) || ahead_loaded) continue;
                         const unsigned* flag = g.flags + (size_t)(c == w_last ? 2 * c : 2 * c + 1) * kPanelFlagStride;
                         unsigned spins = 0;
                         while (true) {
@@ -394,6 +428,44 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
                         }
                     }
                     unsigned tile_mask = 0;
+                    if (n == 1 && ahead_loaded) {
+                        const __amdgpu_buffer_rsrc_t rt_ = partial_rsrc(ahead_slot);
+                        u32x4_t v[8];
+#pragma unroll
+                        for (int i = 0; i < 8; ++i)
+                            v[i] = __builtin_amdgcn_raw_buffer_load_b128(rt_, (uint32_t)lane * 16u, (uint32_t)(wave * 16 + 8 + i) * 1024u, kGemmCacheAgent);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const uint32_t x = ahead[i][e];
+                                acc[0][(i >> 2) & 1][4 * (i & 3) + e] += __builtin_bit_cast(float, x);
+                            }
+#pragma unroll
+                        for (int i = 0; i < 8; ++i)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const uint32_t x = v[i][e];
+                                acc[1][(i >> 2) & 1][4 * (i & 3) + e] += __builtin_bit_cast(float, x);
+                            }
+                        tile_mask = 0xFu;
+                    } else if (n == 1 && ok) {
+                        // the common case of a short k range: this workgroup and the one behind it.  All four tiles
+                        // are this workgroup's, and their sixteen loads go out together.
+                        const __amdgpu_buffer_rsrc_t rt_ = partial_rsrc(2 * w_last);
+                        u32x4_t v[16];
+#pragma unroll
+                        for (int i = 0; i < 16; ++i)
+                            v[i] = __builtin_amdgcn_raw_buffer_load_b128(rt_, (uint32_t)lane * 16u, (uint32_t)(wave * 16 + i) * 1024u, kGemmCacheAgent);
+#pragma unroll
+                        for (int i = 0; i < 16; ++i)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const uint32_t x = v[i][e];
+                                acc[i >> 3][(i >> 2) & 1][4 * (i & 3) + e] += __builtin_bit_cast(float, x);
+                            }
+                        tile_mask = 0xFu;
+                    } else
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         if ((wave * 4 + q) % n != mine) continue;
@@ -464,17 +536,29 @@ size_t panel_workspace_bytes() {
 
 int panel_max_tokens() { return kPanelTok; }
 
-// Worth it when every compute unit gets at least a few k steps per stage; otherwise panels are cut into so many
-// pieces that the hand-over of partial tiles costs more than the shared slabs save.
+// Whether one stage of a group is better off as a panel launch than on the tiles of nq_gemm.hip (measured on
+// Llama-2-7B layers, per stage, 64 .. 4096 tokens).  Every compute unit must get a few k steps (otherwise panels are cut
+// into many pieces and the hand-over of partial tiles costs more than the shared slabs save); the longest k range
+// must not be shared by more than about four workgroups (the first stage of a 128-token layer, whose 43-tile down
+// projection is cut eight ways, is faster on the few-token tiles); token counts that fill their 128-token blocks
+// badly waste MFMAs, which only a stage with a long k makes up for (its block tiles need a k split and a finish
+// launch); and from about 1024 tokens on the block tiles are ahead.
 bool panel_applies(int count, int T, const int* K, const int* R) {
     const int G = panel_grid();
-    if (G <= 0 || count < 1 || count > kPanelMax || T < 96 || T > kPanelTok) return false;
+    if (G <= 0 || count < 1 || count > kPanelMax || T < 1 || T > 768) return false;
+    const int tblocks = (T + kPanelTok - 1) / kPanelTok;
     long long units = 0;
+    int longest = 0;
     for (int p = 0; p < count; ++p) {
         if (K[p] % kTileK != 0 || R[p] % 32 != 0) return false;
-        units += (long long)((R[p] + kPanelRows - 1) / kPanelRows) * (K[p] / kTileK);
+        units += (long long)((R[p] + kPanelRows - 1) / kPanelRows) * tblocks * (K[p] / kTileK);
+        longest = longest > K[p] / kTileK ? longest : K[p] / kTileK;
     }
-    return units >= 3ll * G;
+    const double per_wg = (double)units / G;
+    if (per_wg < 3.0) return false;
+    if (longest > 4.0 * per_wg) return false;
+    const double fill = (double)T / (tblocks * kPanelTok);
+    return fill >= 0.85 || longest > 16;
 }
 
 template <int DT, bool SCALED>
