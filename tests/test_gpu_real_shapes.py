@@ -201,9 +201,10 @@ def test_cfg4_q_o_8192_square(dev, batch):
         assert e < 1e-3, e
 
 
-def test_cfg4_full_stack_one_launch(dev):
+@pytest.mark.parametrize("batch", [1, 8])
+def test_cfg4_full_stack_one_launch(dev, batch):
     """The 560 linears of the Llama-3-70B-shaped stack (8.6 GB of random words generated on the device, as bench.py
-    does) in ONE run-list launch at batch 1.  No oracle fits this size; the property checked is that sampled linears
+    does) in ONE run-list launch at batch 1 and 8.  No oracle fits this size; the property checked is that sampled linears
     of the stack (first, middle, last layer; every shape) equal the per-linear operator on the same words, which the
     tests above and in test_gpu_configs.py hold against the oracle at these shapes."""
     shapes = ((8192, 8192), (1024, 8192), (1024, 8192), (8192, 8192), (28672, 8192), (28672, 8192), (8192, 28672))
@@ -211,8 +212,8 @@ def test_cfg4_full_stack_one_launch(dev):
     gen.manual_seed(70)
     i32 = torch.iinfo(torch.int32)
     sc = lambda k: (torch.randn(k, device=dev, generator=gen).abs() * 0.02 + 1e-3).to(torch.float16)
-    xs = {n: torch.randn(1, n, device=dev, generator=gen).to(torch.float16) for n in (8192, 28672)}
-    rl = DecodeRunList(1, torch.float16, dev)
+    xs = {n: torch.randn(batch, n, device=dev, generator=gen).to(torch.float16) for n in (8192, 28672)}
+    rl = DecodeRunList(batch, torch.float16, dev)
     keep = {}
     layers = 80
     for layer in range(layers):
@@ -228,7 +229,7 @@ def test_cfg4_full_stack_one_launch(dev):
                 keep[idx] = (xs[n], s_in, vt, s_mid, u, s_out)
             else:
                 del vt, u
-    print(f"cfg4 full stack: {layers * len(shapes)} linears in one launch", flush=True)
+    print(f"cfg4 full stack: {layers * len(shapes)} linears in one launch, batch {batch}", flush=True)
     ys = rl.run()
     torch.cuda.synchronize()
     assert rl.status() == 0
@@ -236,4 +237,6 @@ def test_cfg4_full_stack_one_launch(dev):
         y_op = torch.ops.binary_kernels.nanoquant_dyn_forward(x, s_in, vt, s_mid, u, s_out, 128, 128, 2, 2, 1, 1, 8, 8)
         torch.cuda.synchronize()
         scale = float(y_op.float().abs().max())
-        assert torch.allclose(ys[idx].float(), y_op.float(), rtol=2e-3, atol=2e-3 * scale), idx
+        # batch 8 runs on 16-bit operands in the run list (x * s_in and h rounded to fp16, as the operator does too)
+        tol = 2e-3 if batch == 1 else 4e-3
+        assert torch.allclose(ys[idx].float(), y_op.float(), rtol=tol, atol=tol * scale), (idx, batch)
