@@ -470,16 +470,39 @@ def main():
             ms_c = timed_launches(chained.run, 6, 2) / len(layers)
             if chained.status() != 0:
                 raise RuntimeError("run list reported an expired dependency wait")
+            # (c) the same four groups per layer without run lists: nq_gemv_forward_group, ordinary launches that need
+            #     neither a built list nor the GPU to themselves; two launches per group (all first stages, all second
+            #     stages), or one whose second stages wait inside the kernel
+            from nanoquant_amd import ops as nq_ops
+            ys_p = io_p[2]
+
+            def group_step(layer, one_launch):
+                for group in ((0, 1, 2), (3,), (4, 5), (6,)):
+                    nq_ops.gemv_group_forward([xs_p[j] for j in group],
+                                              [(layer[j].s_in, layer[j].vt_bits, layer[j].s_mid, layer[j].u_bits, layer[j].s_out)
+                                               for j in group], outs=[ys_p[j] for j in group], one_launch=one_launch)
+
+            ms_g = timed([(lambda layer=layer: group_step(layer, False)) for layer in layers], 4 * len(layers), len(layers))
+            ms_g1 = timed([(lambda layer=layer: group_step(layer, True)) for layer in layers], 4 * len(layers), len(layers))
+            if nq_ops.gemv_group_status(dev) != 0:
+                raise RuntimeError("a group launch reported an expired wait")
             lb = layer_bytes(b)
             extra[f"decoder_pattern_batch{b}"] = {
+                "four_groups_two_launches_each": {"us_per_layer": round(ms_g * 1e3, 3), "GBps": round(lb / (ms_g * 1e-3) / 1e9, 2),
+                                                  "frac_of_hbm_peak": round(lb / (ms_g * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+                "four_groups_one_launch_each": {"us_per_layer": round(ms_g1 * 1e3, 3), "GBps": round(lb / (ms_g1 * 1e-3) / 1e9, 2),
+                                                "frac_of_hbm_peak": round(lb / (ms_g1 * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
                 "four_launches_per_layer": {"us_per_layer": round(ms_p * 1e3, 3), "GBps": round(lb / (ms_p * 1e-3) / 1e9, 2),
                                             "frac_of_hbm_peak": round(lb / (ms_p * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
                 "chained_one_launch": {"us_per_layer": round(ms_c * 1e3, 3), "GBps": round(lb / (ms_c * 1e-3) / 1e9, 2),
                                        "frac_of_hbm_peak": round(lb / (ms_c * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                                        "phases": int(chained._plan.nphases)},
-                "note": "decoder-shaped issue patterns of the same 32 x 7 linears: (a) per layer the launches {q,k,v}, {o}, "
-                        "{gate,up}, {down} (128 launches in one HIP graph); (b) one launch for the stack with v -> o -> gate/up, "
-                        "gate -> down -> next layer's q/k/v linked through x_from"}
+                "note": "decoder-shaped issue patterns of the same 32 x 7 linears: per layer the launches {q,k,v}, {o}, "
+                        "{gate,up}, {down} in one HIP graph: as ordinary launches of nq_gemv_forward_group, two per group "
+                        "(four_groups_two_launches_each) or one per group whose second stages wait inside the kernel "
+                        "(four_groups_one_launch_each), and as run-list launches (four_launches_per_layer); "
+                        "chained_one_launch: one launch for the stack with v -> o -> gate/up, gate -> down -> next layer's "
+                        "q/k/v linked through x_from"}
             del chained
 
         # ---- cfg0: one 2048 x 2048 linear of rank 1024 at batch 1 (the reference's CPU-runnable case), GPU and CPU ----
@@ -508,7 +531,7 @@ def main():
         t_cpu0.sort()
         b0 = gemv_bytes(2048, 2048, 1024, 1)
         extra["cfg0_2048x2048_r1024_batch1"] = {
-            "gpu_us_operator_two_launches": round(us_op0, 2), "gpu_us_run_list_one_launch": round(us_rl0, 2),
+            "gpu_us_operator": round(us_op0, 2), "gpu_us_run_list_one_launch": round(us_rl0, 2),
             "GBps_operator": round(b0 / (us_op0 * 1e-6) / 1e9, 1), "cpu_us_dense_fp32": round(t_cpu0[len(t_cpu0) // 2] * 1e6, 1),
             "cpu_threads": torch.get_num_threads(), "max_rel_err_gpu_vs_dense_definition": float("%.3e" % err0),
             "note": "warm weights (0.5 MB, cache resident), graph replays; the CPU figure is the reference's dense path "
@@ -533,6 +556,7 @@ def main():
         mods = [[decode_module(lin) for lin in layer] for layer in layers]
         for layer in mods:
             for mod in layer:
+                mod.mfma_from_rows = 3         # opt in to the few-token MFMA tiles from 3 rows on
                 mod.prepare_mfma_route()       # set-up: otherwise the first call of 3 or more rows builds the tiles
         by_rows = {}
         with torch.no_grad():
@@ -542,8 +566,8 @@ def main():
                 by_rows[str(rows)] = round(timed(fns, 2 * len(layers), len(layers)) * 1e3, 1)
         extra["module_forward_us_per_layer_by_rows"] = dict(
             by_rows, note="NanoQuantLinear.forward of 7 modules prepared with kernel_type='gemv', graph replays over the "
-                          "rotating weight copies: two decode launches per linear up to 2 rows, the few-token MFMA tiles "
-                          "(built once from the decode words) from 3 rows on")
+                          "rotating weight copies: one decode launch per linear up to 2 rows, the few-token MFMA tiles "
+                          "(mfma_from_rows = 3, built once from the decode words) from 3 rows on")
         del mods
         # ---- prefill GEMM over the three distinct linear shapes of the layer ----
         # Timed as HIP graph replays: through Python the two-GEMM op costs more host time than GPU time.

@@ -167,6 +167,26 @@ int nq_runlist_status(const void* workspace, int* status_out, void* stream);
  * NQ_ERR_SHAPE for a batch size without a run-list kernel.  Sets bit 3 of plan->bound. */
 int nq_runlist_set_deterministic(nq_runlist_plan* plan, int on);
 
+/* Decode path for a group of independent linears: the q/k/v or gate/up projections of a decoder layer in two kernel
+ * launches per nq_gemv_group_max() linears (all first stages, then all second stages) instead of the two launches
+ * per linear of nq_gemv_forward and of the reference (kernel/cuda/gemv_kernel.cu:406-425), without a built run list:
+ * nothing to prepare, any pointers on every call, no requirement on what else the GPU runs.
+ *   linears: x_from = y_from = -1, no addend, out_f32 = 0, tiled = 0; h buffers distinct, fp32 [batch, r] each.
+ *   Pieces of 1, 2 and 4 batch rows are grouped; pieces of 8 and 16 rows take two launches per linear.
+ * one_launch = 1: ONE ordinary launch per group instead of two.  The workgroups of the second stages sit behind those
+ * of the first in the same grid, fetch their first sign words, and wait on flags until their linear's h is complete
+ * (workgroups start in the order of their ids, so whatever a workgroup waits for is running or done: no resident
+ * grid is needed).  On MI355X the signalling through device-coherent memory costs more than the launch boundary it
+ * replaces (a Llama-2-7B layer at batch 1 in four groups: 104 us with one launch per group, 53 us with two); the
+ * switch is kept for measurement and for callers that are charged per launch.  Its flags live in a device
+ * array inside the library (4.5 MiB per GPU, 256 slots dealt round robin, every launch puts its slot back to zero);
+ * the first call on each device looks up its address and should be made outside graph capture.  The wait is bounded
+ * (2^20 polls): if it expires the launch still ends, its outputs are invalid, and nq_gemv_group_status reports 1.
+ * nq_gemv_group_status copies the device's status word back (synchronises `stream`) and clears it. */
+int nq_gemv_group_max(void);
+int nq_gemv_forward_group(const nq_linear* linears, int count, int batch, int dtype, int one_launch, void* stream);
+int nq_gemv_group_status(int* status_out, void* stream);
+
 /* One matmul-free stage: out[b,row] = s_row[row] * sum_c sgn(bits[row,c]) * in[b,c] * s_col[c].
  * Replaces nanoquant_stage1_dyn_kernel / nanoquant_stage2_dyn_kernel launches
  * (kernel/cuda/gemv_kernel.cu:283-301).  in/out are `dtype`; s_col, s_row may be NULL. */

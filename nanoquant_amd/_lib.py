@@ -25,6 +25,9 @@ _SIGNATURES = {
     "nq_gemv_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "nq_gemv_forward_bias": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "nq_gemv_forward_noalloc": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "nq_gemv_group_max": (_i, []),
+    "nq_gemv_forward_group": (_i, [_vp, _i, _i, _i, _i, _vp]),
+    "nq_gemv_group_status": (_i, [ctypes.POINTER(_i), _vp]),
     "nq_gemv_mixture": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "nq_runlist_workspace_bytes": (_sz, [_vp, _i]),
     "nq_runlist_build": (_i, [_vp, _i, _i, _i, _i, _vp, _sz, _vp, _vp]),

@@ -41,7 +41,7 @@ const char* nq_status_string(int status) {
 
 int nq_last_hip_error(void) { return g_last_hip_error; }
 
-int nq_abi_version(void) { return 8; }
+int nq_abi_version(void) { return 9; }
 
 int nq_device_query(int attr, int* value) {
     if (!value) return NQ_ERR_NULL;
@@ -64,6 +64,59 @@ int nq_gemv_forward(const void* x, const void* s_in, const uint32_t* vt_bits, co
     return nq_gemv_forward_bias(x, s_in, vt_bits, s_mid, u_bits, s_out, nullptr, h_scratch, y, batch, n, r, m, dtype, stream);
 }
 
+// Both stages of every linear for `batch` rows.  Groups of independent linears in pieces of 1, 2 and 4 batch rows go
+// through nq::gemv_fused (two launches per nq::gemv_fused_max() linears, or one with `one_launch`); a single linear,
+// and pieces of 8 and 16 rows, take two launches per linear.
+static int forward_linears(const nq_linear* ls, int count, int batch, int dtype, bool one_launch, hipStream_t st) {
+    const int group = nq::gemv_fused_max();
+    int done = 0;
+    while (done < batch) {
+        int piece = 16;
+        while (piece > batch - done) piece >>= 1;
+        if (piece >= 8 || (count == 1 && !one_launch)) {
+            for (int i = 0; i < count; ++i) {
+                const nq_linear& l = ls[i];
+                if (l.m == 0) continue;
+                const char* x = (const char*)l.x + (size_t)done * l.n * 2;
+                float* h = l.h + (size_t)done * l.r;
+                char* y = (char*)l.y + (size_t)done * l.m * 2;
+                hipError_t e = nq::gemv_stage(dtype, true, l.vt_bits, x, l.s_in, l.s_mid, nullptr, h, true, piece, l.r,
+                                              words_of(l.n), l.n, l.n, l.r, st);
+                if (e != hipSuccess) return hip_status(e);
+                e = nq::gemv_stage(dtype, false, l.u_bits, h, nullptr, l.s_out, nullptr, y, false, piece, l.m,
+                                   words_of(l.r), l.r, l.r, l.m, st, l.bias);
+                if (e != hipSuccess) return hip_status(e);
+            }
+        } else {
+            for (int i0 = 0; i0 < count; i0 += group) {
+                const int c = count - i0 < group ? count - i0 : group;
+                const void *x[16], *s_in[16], *s_mid[16], *s_out[16], *bias[16];
+                const uint32_t *vt[16], *u[16];
+                float* h[16];
+                void* y[16];
+                int n[16], r[16], m[16];
+                int k = 0;
+                for (int i = i0; i < i0 + c; ++i) {
+                    const nq_linear& l = ls[i];
+                    if (l.m == 0) continue;
+                    x[k] = (const char*)l.x + (size_t)done * l.n * 2;
+                    h[k] = l.h + (size_t)done * l.r;
+                    y[k] = (char*)l.y + (size_t)done * l.m * 2;
+                    s_in[k] = l.s_in; s_mid[k] = l.s_mid; s_out[k] = l.s_out; bias[k] = l.bias;
+                    vt[k] = l.vt_bits; u[k] = l.u_bits;
+                    n[k] = l.n; r[k] = l.r; m[k] = l.m;
+                    ++k;
+                }
+                if (k == 0) continue;
+                hipError_t e = nq::gemv_fused(dtype, k, piece, x, s_in, vt, s_mid, u, s_out, bias, h, y, n, r, m, one_launch, st);
+                if (e != hipSuccess) return hip_status(e);
+            }
+        }
+        done += piece;
+    }
+    return NQ_OK;
+}
+
 int nq_gemv_forward_bias(const void* x, const void* s_in, const uint32_t* vt_bits, const void* s_mid,
                          const uint32_t* u_bits, const void* s_out, const void* bias, float* h_scratch, void* y,
                          int batch, int n, int r, int m, int dtype, void* stream) {
@@ -71,13 +124,38 @@ int nq_gemv_forward_bias(const void* x, const void* s_in, const uint32_t* vt_bit
     if (batch < 0 || n < 0 || r < 0 || m < 0) return NQ_ERR_SHAPE;
     if (batch == 0 || m == 0) return NQ_OK;
     if (!x || !s_in || !vt_bits || !u_bits || !s_out || !h_scratch || !y) return NQ_ERR_NULL;
-    hipStream_t st = (hipStream_t)stream;
-    hipError_t e = nq::gemv_stage(dtype, true, vt_bits, x, s_in, s_mid, nullptr, h_scratch, true, batch, r,
-                                  words_of(n), n, n, r, st);
+    nq_linear l{};
+    l.x = x; l.s_in = s_in; l.vt_bits = vt_bits; l.s_mid = s_mid; l.u_bits = u_bits; l.s_out = s_out;
+    l.h = h_scratch; l.y = y; l.bias = bias; l.n = n; l.r = r; l.m = m; l.x_from = -1; l.y_from = -1;
+    return forward_linears(&l, 1, batch, dtype, false, (hipStream_t)stream);
+}
+
+int nq_gemv_group_max(void) { return nq::gemv_fused_max(); }
+
+int nq_gemv_forward_group(const nq_linear* linears, int count, int batch, int dtype, int one_launch, void* stream) {
+    if (dtype != NQ_F16 && dtype != NQ_BF16) return NQ_ERR_DTYPE;
+    if (count < 0 || batch < 0 || (one_launch != 0 && one_launch != 1)) return NQ_ERR_SHAPE;
+    if (count == 0 || batch == 0) return NQ_OK;
+    if (!linears) return NQ_ERR_NULL;
+    for (int i = 0; i < count; ++i) {
+        const nq_linear& l = linears[i];
+        if (l.n < 0 || l.r < 0 || l.m < 0) return NQ_ERR_SHAPE;
+        if (l.x_from >= 0 || l.y_from >= 0 || l.addend || l.out_f32 || l.tiled) return NQ_ERR_SHAPE;   // independent plain linears only
+        if (l.m == 0) continue;
+        if (!l.x || !l.s_in || !l.vt_bits || !l.u_bits || !l.s_out || !l.h || !l.y) return NQ_ERR_NULL;
+        for (int j = 0; j < i; ++j)
+            if (linears[j].m && linears[j].h == l.h) return NQ_ERR_SHAPE;                               // every linear needs an h of its own
+    }
+    return forward_linears(linears, count, batch, dtype, one_launch != 0, (hipStream_t)stream);
+}
+
+int nq_gemv_group_status(int* status_out, void* stream) {
+    if (!status_out) return NQ_ERR_NULL;
+    unsigned v = 0;
+    hipError_t e = nq::gemv_fused_status(&v, (hipStream_t)stream);
     if (e != hipSuccess) return hip_status(e);
-    e = nq::gemv_stage(dtype, false, u_bits, h_scratch, nullptr, s_out, nullptr, y, false, batch, m,
-                       words_of(r), r, r, m, st, bias);
-    return hip_status(e);
+    *status_out = (int)v;
+    return NQ_OK;
 }
 
 // ---- the allocation-free variant of nq_gemv_forward_bias ---------------------------------------------

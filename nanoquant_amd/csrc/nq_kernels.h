@@ -13,6 +13,15 @@ hipError_t gemv_stage(int dtype, bool first, const uint32_t* bits, const void* i
                       int words, int K, int in_stride, int out_stride, hipStream_t stream,
                       const void* bias = nullptr);
 
+// Both stages of up to gemv_fused_max() independent linears (batch 1, 2 or 4) in two launches, or in one whose second
+// stages wait inside the kernel; see nq_gemv.hip.
+int gemv_fused_max();
+hipError_t gemv_fused(int dtype, int count, int batch, const void* const* x, const void* const* s_in,
+                      const uint32_t* const* vt_bits, const void* const* s_mid, const uint32_t* const* u_bits,
+                      const void* const* s_out, const void* const* bias, float* const* h, void* const* y,
+                      const int* n, const int* r, const int* m, bool one_launch, hipStream_t stream);
+hipError_t gemv_fused_status(unsigned* out, hipStream_t stream);
+
 // nq_stream.hip: one launch over a table of stages (see the file header).
 struct RunStage {
     const uint32_t* bits;   // [rows, words] packed signs, row-major "half2" order

@@ -47,13 +47,14 @@ class NanoQuantLinear(nn.Module):
         # scales and the bias) on a list built once per row count, instead of the two launches of the
         # reference's op (linear.py:121-130).  It bypasses the torch op, so leave it off under torch.compile.
         self.fused_launch = False
-        # A module prepared for decode ("gemv") sends calls of at least this many rows to the few-token MFMA tiles of
-        # the prefill path (0: never).  Their cost does not depend on the row count (109 us per Llama-2-7B layer of 7
-        # linears, weights from HBM), that of the decode kernels grows with every row: 75 / 94 / 164 / 131 / 220 / 195 us
-        # at 1 / 2 / 3 / 4 / 6 / 16 rows.  The prefill tiles are built once from the decode words on the first such
-        # call (or by `prepare_mfma_route()`), on the device, and kept beside them: a second copy of the packed
-        # factors.  Needs in_features % 256 == 0 and out_features % 32 == 0; other shapes stay on the decode kernels.
-        self.mfma_from_rows = 3
+        # Opt-in (0: never): a module prepared for decode ("gemv") sends calls of at least this many rows to the
+        # few-token MFMA tiles of the prefill path, whose cost does not grow with the row count while that of the
+        # decode kernels does; 3 is the break-even on a Llama-2-7B layer.  The price is a second copy of the packed
+        # factors (the prefill tiles, built once from the decode words on the device, on the first such call or by
+        # `prepare_mfma_route()`, and kept beside them), and results that differ in the last bits from the decode
+        # kernels' (other order of the fp32 additions, h rounded to 16 bits in between).  Needs
+        # in_features % 256 == 0 and out_features % 32 == 0; other shapes stay on the decode kernels.
+        self.mfma_from_rows = 0
         self._mfma_tiles = None
         self._fused_lists = {}
         self._fused_tiled = None
@@ -419,6 +420,46 @@ def prefill_group(modules: Sequence, x) -> list:
             bias_groups[i].append(b)
             group_x[i] = xf
         outs = ops.gemm_group_sum_forward(group_x, groups, bias_groups if any(b is not None for b in biases) else None)
+    for i, t in enumerate(xs_in):
+        y = outs[i]
+        if t.ndim == 3:
+            y = y.view(t.shape[0], t.shape[1], -1)
+        outs[i] = y.to(t.dtype) if y.dtype != t.dtype else y
+    return outs
+
+
+def decode_group(modules: Sequence, x) -> list:
+    """`[mod(x) for mod in modules]` for modules prepared with `_prepare_kernel("gemv")`, with the stages of all
+    modules sharing launches (`ops.gemv_group_forward`; pieces of 1, 2 and 4 rows, two launches per 8 modules): what a
+    decoder issues per layer at decode time is then eight launches, two each for {q,k,v}, {o}, {gate,up}, {down}, with
+    its attention, norms and activations between them, instead of the reference's two launches per module
+    (linear.py:121-130).  Nothing is prepared or kept: any activations on every call, no requirement on what else the
+    GPU runs.  `x` is one tensor for all modules or a list of one tensor per module, 2-D or 3-D as `forward` takes it."""
+    mods = list(modules)
+    if not mods:
+        return []
+    xs_in = [x] * len(mods) if isinstance(x, torch.Tensor) else list(x)
+    if len(xs_in) != len(mods):
+        raise ValueError("one input per module")
+    for mod in mods:
+        if not getattr(mod, "do_kernel_inference", False) or getattr(mod, "kernel_type", None) != "gemv":
+            raise ValueError("decode_group needs modules prepared with _prepare_kernel('gemv', dtype)")
+        if mod.dtype != mods[0].dtype:
+            raise ValueError("all modules of a group must be prepared for the same dtype")
+    flat, cache = [], {}
+    for t in xs_in:
+        if t.ndim not in (2, 3):
+            raise ValueError(f"Expected 2D or 3D input tensor, got {t.ndim}D")
+        if id(t) not in cache:                 # a shared input is converted once
+            v = t if t.dtype == mods[0].dtype else t.to(mods[0].dtype)
+            cache[id(t)] = v.contiguous().view(-1, v.size(-1))
+        flat.append(cache[id(t)])
+    biases = []
+    for mod in mods:
+        b = mod.bias if (mod.kernel_path_bias and mod.bias is not None) else None
+        biases.append(None if b is None else (b if b.dtype == mod.dtype else b.to(mod.dtype)))
+    outs = ops.gemv_group_forward(flat, [(m.scale_pre, m.V_int8, m.scale_mid, m.U_int8, m.scale_post) for m in mods],
+                                  biases if any(b is not None for b in biases) else None)
     for i, t in enumerate(xs_in):
         y = outs[i]
         if t.ndim == 3:

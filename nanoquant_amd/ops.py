@@ -328,6 +328,67 @@ def gemv_forward_with_bias(x, scale_g, Ubits, scale_l, Vbits, scale_h, bias):
     return _gemv_forward(x, scale_g, Ubits, scale_l, Vbits, scale_h, bias)
 
 
+def gemv_group_forward(xs, linears, biases=None, outs=None, one_launch=False):
+    """`[nanoquant_dyn_forward(x_i, *linears[i]) (+ biases[i])]` for independent linears in two launches per
+    `nq_gemv_group_max()` linears and piece of 1, 2 or 4 rows (`nq_gemv_forward_group`: all first stages, then all
+    second stages): the q/k/v or gate/up projections of a decoder layer at decode time, which the reference launches
+    one module and two kernels at a time (modules/linear.py:121-130).  `xs`: one tensor [rows, n] for all linears or
+    one per linear (same row count); `linears`: (scale_g, Ubits, scale_l, Vbits, scale_h) per linear, the operands of
+    the op in its order; `outs`: optional result tensors [rows, m_i] to write into; `one_launch`: a single launch per
+    group whose second stages wait inside the kernel (slower on MI355X, see include/nq_gfx950.h)."""
+    linears = list(linears)
+    if not linears:
+        return []
+    xs = [xs] * len(linears) if isinstance(xs, torch.Tensor) else list(xs)
+    if len(xs) != len(linears):
+        raise ValueError("one input per linear")
+    biases = [None] * len(linears) if biases is None else list(biases)
+    from .runlist import NqLinear
+    x0 = xs[0]
+    batch = x0.numel() // max(x0.size(-1), 1) if x0.dim() >= 1 else 0
+    dims, offsets, total = [], [], 0
+    for x, lin, b in zip(xs, linears, biases):
+        n, r, m = _check_gemv_args(x, *lin)
+        _check_bias(b, m, x)
+        if x.dtype != x0.dtype or x.device != x0.device:
+            raise RuntimeError("all inputs of a group must share dtype and device")
+        if x.numel() // max(n, 1) != batch:
+            raise RuntimeError("all inputs of a group must have the same number of rows")
+        dims.append((n, r, m))
+        offsets.append(total)
+        total += (batch * max(r, 1) + 63) // 64 * 64              # fp32: every h starts on a 256-byte boundary
+    if outs is None:
+        outs = [torch.empty((batch, m), dtype=x0.dtype, device=x0.device) for _, _, m in dims]
+    else:
+        outs = list(outs)
+        for y, (_, _, m) in zip(outs, dims):
+            _check_dev_cont(y, "out", x0.dtype, _FLOAT_WHAT[x0.dtype])
+            if tuple(y.shape) != (batch, m):
+                raise RuntimeError(f"out must be [{batch}, {m}], got {list(y.shape)}")
+    if batch == 0:
+        return outs
+    h = torch.empty(total, dtype=torch.float32, device=x0.device)
+    arr = (NqLinear * len(linears))()
+    p = lambda t: None if t is None else t.data_ptr()
+    for i, (x, (sg, ub, sl, vb, sh), b, y, (n, r, m)) in enumerate(zip(xs, linears, biases, outs, dims)):
+        arr[i] = NqLinear(p(x), p(sg), p(ub), p(sl), p(vb), p(sh), h.data_ptr() + 4 * offsets[i], p(y), None, n, r, m, -1, -1, 0,
+                          p(b), 0)
+    with torch.cuda.device(x0.device):
+        _lib.check(_lib.lib().nq_gemv_forward_group(arr, len(linears), batch, _dtype_id(x0), 1 if one_launch else 0,
+                                                     _stream(x0.device)))
+    return outs
+
+
+def gemv_group_status(device=None) -> int:
+    """Synchronises the current stream.  0, or 1 when a launch of `gemv_group_forward(one_launch=True)` on this device
+    ran into its bounded wait since the last call: the outputs of that launch are invalid.  Clears the flag."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    out = ctypes.c_int(0)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().nq_gemv_group_status(ctypes.byref(out), _stream(dev)))
+    return out.value
+
+
 def gemm_forward_with_bias(x, weight_u, weight_v, scale_g, scale_l, scale_h, workspace, bias):
     """marlin_nanoquant_forward + bias [m], added in the epilogue of the second GEMM."""
     return _gemm_nanoquant_forward(x, weight_u, weight_v, scale_g, scale_l, scale_h, workspace, bias)

@@ -37,7 +37,7 @@ def _stack(dev, kernel_type, dtype):
         f = lambda a: torch.from_numpy(a.astype(np.float32))
         mod = NanoQuantLinear.from_factors(f(vt), f(u), f(s_in), f(s_mid), f(s_out), dtype=dtype).to(dev)
         mod._prepare_kernel(kernel_type, dtype)
-        mod.mfma_from_rows = 0                                         # "gemv" means the decode op here, at 4 rows too
+        assert mod.mfma_from_rows == 0                                 # as built: "gemv" is the decode op at 4 rows too
         mods.append(mod)
         terms.append((vt, u, s_in, s_mid, s_out))
     return _Stack(mods).to(dev), terms

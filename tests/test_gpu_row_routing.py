@@ -1,5 +1,5 @@
-"""A module prepared for decode sends calls of 3 or more rows to the few-token MFMA tiles of the prefill path
-(the reference runs every batch size through its GEMV kernels, re-reading the weights per batch row:
+"""A module prepared for decode with `mfma_from_rows = 3` sends calls of 3 or more rows to the few-token MFMA tiles of
+the prefill path (opt-in; the reference runs every batch size through its GEMV kernels, re-reading the weights per batch row:
 kernel/cuda/gemv_kernel.cu:288-290).  Same interface, same result within the tolerance, tiles built from the decode
 words on the device."""
 import numpy as np
@@ -18,6 +18,8 @@ def _module(dev, m, n, r, seed, dtype):
     f = lambda a: torch.from_numpy(a.astype(np.float32))
     mod = NanoQuantLinear.from_factors(f(vt), f(u), f(s_in), f(s_mid), f(s_out), dtype=dtype).to(dev)
     mod._prepare_kernel("gemv", dtype)
+    assert mod.mfma_from_rows == 0                                     # the route is opt-in
+    mod.mfma_from_rows = 3
     return mod, (vt, u, s_in, s_mid, s_out)
 
 

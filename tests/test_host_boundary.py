@@ -252,10 +252,11 @@ def test_row_routing_and_run_list_options_need_no_gpu():
     vt, u, s_in, s_mid, s_out = oracle.synth_term(64, 256, 32, seed=9)
     f = lambda a: torch.from_numpy(a.astype(np.float32))
     mod = NanoQuantLinear.from_factors(f(vt), f(u), f(s_in), f(s_mid), f(s_out), dtype=torch.float32)
-    assert mod.mfma_from_rows == 3 and mod._mfma_tiles is None
+    assert mod.mfma_from_rows == 0 and mod._mfma_tiles is None
     with pytest.raises(RuntimeError, match="kernel_type='gemv'"):
         mod.prepare_mfma_route()                                       # not prepared for decode yet
     mod._prepare_kernel("gemv", torch.float16)
+    mod.mfma_from_rows = 3
     assert not mod._routes_to_mfma(torch.zeros(8, 256))                # CPU tensors never route (and never build tiles)
     assert mod._mfma_tiles is None
     mod.prepare_mfma_route()                                           # the packing pass itself runs on any device
