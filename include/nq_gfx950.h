@@ -155,6 +155,13 @@ int nq_runlist_run(const void* workspace, const nq_runlist_plan* plan, void* str
  * by x_from / y_from. */
 int nq_runlist_run_bound(const void* workspace, const nq_runlist_plan* plan, const void* x, void* y, void* stream);
 int nq_runlist_status(const void* workspace, int* status_out, void* stream);
+/* Workgroups of the run-list kernel that the current device keeps resident at once, for lists of this batch size and
+ * type whose longest input has `max_units` 16-byte units per row (plan.max_units).  variant -1: the smallest over all
+ * kernel variants a plan can be launched with (row-major or tile order, with or without reproducible sums, wavefronts
+ * owning row pairs), which is what nq_runlist_build sizes the grid with; 0..5: one variant (0 where it does not
+ * exist).  nq_runlist_run checks the grid against the variant it starts and returns NQ_ERR_HIP
+ * (hipErrorLaunchOutOfResources) instead of launching a grid that cannot be resident.  0 on error. */
+int nq_runlist_capacity(int batch, int dtype, int max_units, int variant);
 /* Reproducible sums for the launches of this plan, on (1) or off (0, as built).  The run-list kernel finishes a row
  * sum with additions from several wavefronts whose order differs from launch to launch, so outputs may differ in
  * the last bit between launches (the reference's reductions are ordered: kernel/cuda/gemv_kernel.cu:148-170,

@@ -35,6 +35,7 @@ _SIGNATURES = {
     "nq_runlist_run_bound": (_i, [_vp, _vp, _vp, _vp, _vp]),
     "nq_runlist_status": (_i, [_vp, ctypes.POINTER(_i), _vp]),
     "nq_runlist_set_deterministic": (_i, [_vp, _i]),
+    "nq_runlist_capacity": (_i, [_i, _i, _i, _i]),
     "nq_gemv_stage": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "nq_gemm_scratch_bytes": (_sz, [_i, _i, _i]),
     "nq_gemm_onebit": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),

@@ -625,6 +625,13 @@ int nq_runlist_run_bound(const void* workspace, const nq_runlist_plan* plan, con
                                       (plan->bound & 32) != 0));
 }
 
+int nq_runlist_capacity(int batch, int dtype, int max_units, int variant) {
+    if (dtype != NQ_F16 && dtype != NQ_BF16) return 0;
+    if (batch != 1 && batch != 2 && batch != 4 && batch != 8 && batch != 16) return 0;
+    if (max_units <= 0 || variant < -1 || variant > 5) return 0;
+    return nq::stream_capacity(dtype, batch, max_units, false, variant);
+}
+
 int nq_runlist_set_deterministic(nq_runlist_plan* plan, int on) {
     if (!plan) return NQ_ERR_NULL;
     if (plan->dtype != NQ_F16 && plan->dtype != NQ_BF16) return NQ_ERR_DTYPE;

@@ -64,7 +64,7 @@ size_t stream_counter_bytes(int nstages);
 // alt: the 16-bit arithmetic instead of the batch size's usual one, where stream_has_alt(dtype, batch);
 // own: the fp4 x fp8 kernel whose wavefronts own row pairs, where it exists (tile order, batch 2 and 4, no reproducible
 // sums, every input staged in one chunk; ignored otherwise)
-int stream_capacity(int dtype, int batch, int max_units, bool alt = false);
+int stream_capacity(int dtype, int batch, int max_units, bool alt = false, int variant = -1);
 int stream_chunk_cap(int dtype, int batch, int max_units, bool alt = false);
 int stream_row_granule(int dtype, int batch);
 hipError_t gemv_stream(int dtype, int batch, int nstages, const RunSlice* slices, unsigned long long* counters,

@@ -1139,19 +1139,65 @@ static hipError_t prepare_kernel(size_t lds) {
     return hipSuccess;
 }
 
-template <int DT, int BATCH, int ARITH>
-static int capacity_of(int max_units) {
-    using SK = StreamKernel<DT, BATCH, ARITH>;
-    int chunk_cap;
-    size_t lds;
-    stream_lds_plan(BATCH, ARITH, max_units, &chunk_cap, &lds);
-    if (prepare_kernel<DT, BATCH, ARITH>(lds) != hipSuccess) return 0;
-    int per_cu = 0, dev = 0, cus = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)SK::fn, SK::kThreads, lds) != hipSuccess)
-        return 0;
-    if (hipGetDevice(&dev) != hipSuccess) return 0;
+// Workgroups of `fn` (launched with `threads` lanes and `lds` bytes of dynamic LDS) that the current device keeps
+// resident at once; 0 on error.  The query is host time, so each calling thread keeps its last answers.
+static int resident_workgroups(const void* fn, int threads, size_t lds) {
+    struct Entry { const void* fn; size_t lds; int dev, cap; };
+    static thread_local Entry cache[16];
+    static thread_local int used = 0, next = 0;
+    const int dev = current_device();
+    if (dev < 0) return 0;
+    for (int i = 0; i < used; ++i)
+        if (cache[i].fn == fn && cache[i].lds == lds && cache[i].dev == dev) return cache[i].cap;
+    int per_cu = 0, cus = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, threads, lds) != hipSuccess) return 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cache[next] = Entry{fn, lds, dev, per_cu * cus};
+    next = (next + 1) % 16;
+    if (used < 16) ++used;
     return per_cu * cus;
+}
+
+// The instance that launch_stream starts for (tiled, det, own) and its LDS plan.  The kernel is only correct when its
+// whole grid is resident, so the builder sizes the grid from the smallest capacity over all variants that a plan may
+// be launched with (reproducible sums are switched on after the grid is fixed), and launch_stream checks the one
+// instance it is about to start.
+constexpr int kStreamVariants = 6;      // fn, fn_tiled, fn_det, fn_tiled_det, fn_tiled_own, fn_tiled_own_det
+template <int DT, int BATCH, int ARITH>
+static const void* stream_variant(int variant, int max_units, int* chunk_cap, size_t* lds) {
+    using SK = StreamKernel<DT, BATCH, ARITH>;
+    const bool det = variant == 2 || variant == 3 || variant == 5;
+    const bool own = variant >= 4;
+    if (own && !SK::kHasOwn) return nullptr;
+    stream_lds_plan(BATCH, SK::kArith, max_units, chunk_cap, lds, det, own);
+    if (own && max_units > *chunk_cap) return nullptr;     // such a list is launched on the row-block form instead
+    switch (variant) {
+        case 0: return (const void*)SK::fn;
+        case 1: return (const void*)SK::fn_tiled;
+        case 2: return (const void*)SK::fn_det;
+        case 3: return (const void*)SK::fn_tiled_det;
+        case 4: return (const void*)SK::fn_tiled_own;
+        default: return (const void*)SK::fn_tiled_own_det;
+    }
+}
+
+// variant < 0: the smallest capacity over all variants; else that of one variant (0: not available or error)
+template <int DT, int BATCH, int ARITH>
+static int capacity_of(int max_units, int variant = -1) {
+    using SK = StreamKernel<DT, BATCH, ARITH>;
+    int best = 0;
+    for (int v = 0; v < kStreamVariants; ++v) {
+        if (variant >= 0 && v != variant) continue;
+        int chunk_cap;
+        size_t lds;
+        const void* fn = stream_variant<DT, BATCH, ARITH>(v, max_units, &chunk_cap, &lds);
+        if (!fn) continue;
+        if (prepare_kernel<DT, BATCH, ARITH>(lds) != hipSuccess) return 0;
+        const int cap = resident_workgroups(fn, SK::kThreads, lds);
+        if (cap <= 0) return 0;
+        if (best == 0 || cap < best) best = cap;
+    }
+    return best;
 }
 
 template <int DT, int BATCH, int ARITH>
@@ -1173,18 +1219,15 @@ static hipError_t launch_stream(int nstages, const RunSlice* slices, unsigned lo
     if (!own) stream_lds_plan(BATCH, SK::kArith, max_units, &chunk_cap, &lds, det);
     hipError_t e = prepare_kernel<DT, BATCH, ARITH>(lds);
     if (e != hipSuccess) return e;
-    if (own)
-        hipLaunchKernelGGL((det ? SK::fn_tiled_own_det : SK::fn_tiled_own), dim3(nwg), dim3(SK::kThreads), lds, stream, nstages,
-                           slices, counters, status, spin_limit, chunk_cap, RunStage{}, 0, ext_in, ext_out);
-    else if (det)
-        hipLaunchKernelGGL((tiled ? SK::fn_tiled_det : SK::fn_det), dim3(nwg), dim3(SK::kThreads), lds, stream, nstages, slices,
-                           counters, status, spin_limit, chunk_cap, RunStage{}, 0, ext_in, ext_out);
-    else if (tiled && SK::kArith == 2)
-        hipLaunchKernelGGL((SK::fn_tiled), dim3(nwg), dim3(SK::kThreads), lds, stream, nstages, slices, counters, status,
-                           spin_limit, chunk_cap, RunStage{}, 0, ext_in, ext_out);
-    else
-        hipLaunchKernelGGL((SK::fn), dim3(nwg), dim3(SK::kThreads), lds, stream, nstages, slices, counters, status,
-                           spin_limit, chunk_cap, RunStage{}, 0, ext_in, ext_out);
+    const bool tiled_fn = tiled && SK::kArith == 2;
+    auto fn = own ? (det ? SK::fn_tiled_own_det : SK::fn_tiled_own)
+                  : det ? (tiled ? SK::fn_tiled_det : SK::fn_det) : tiled_fn ? SK::fn_tiled : SK::fn;
+    // a grid larger than what stays resident would wait for workgroups that never start
+    const int cap = resident_workgroups((const void*)fn, SK::kThreads, lds);
+    if (cap <= 0) return hipErrorInvalidValue;
+    if (nwg > cap) return hipErrorLaunchOutOfResources;
+    hipLaunchKernelGGL(fn, dim3(nwg), dim3(SK::kThreads), lds, stream, nstages, slices, counters, status, spin_limit, chunk_cap,
+                       RunStage{}, 0, ext_in, ext_out);
     return hipGetLastError();
 }
 
@@ -1246,9 +1289,10 @@ hipError_t gemv_stream_single(int dtype, int batch, const RunStage& st, hipStrea
         default: break;                                                                           \
     }
 
-// Number of workgroups the device keeps resident for this kernel variant (0 on error).
-int stream_capacity(int dtype, int batch, int max_units, bool alt) {
-#define NQ_CAP(D, B, A) capacity_of<D, B, A>(max_units)
+// Number of workgroups the device keeps resident for the run-list kernel of this batch size: the smallest over the
+// kernel variants a plan may be launched with (variant < 0), or that of one variant (0 on error or where it does not exist).
+int stream_capacity(int dtype, int batch, int max_units, bool alt, int variant) {
+#define NQ_CAP(D, B, A) capacity_of<D, B, A>(max_units, variant)
     NQ_STREAM_DISPATCH(NQ_CAP)
 #undef NQ_CAP
     return 0;

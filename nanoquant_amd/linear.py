@@ -47,6 +47,9 @@ class NanoQuantLinear(nn.Module):
         # scales and the bias) on a list built once per row count, instead of the two launches of the
         # reference's op (linear.py:121-130).  It bypasses the torch op, so leave it off under torch.compile.
         self.fused_launch = False
+        # With fused_launch: every so many launches of a list the status word is read back (one synchronisation) and an
+        # expired wait raises; the first launch of a list is always checked.  0: only `fused_status()` tells.
+        self.fused_status_every = 256
         # Opt-in (0: never): a module prepared for decode ("gemv") sends calls of at least this many rows to the
         # few-token MFMA tiles of the prefill path, whose cost does not grow with the row count while that of the
         # decode kernels does; 3 is the break-even on a Llama-2-7B layer.  The price is a second copy of the packed
@@ -218,6 +221,7 @@ class NanoQuantLinear(nn.Module):
             rl = DecodeRunList(rows, dtype=self.dtype, device=x.device)
             rl.add(None, self.scale_pre, V, scale_mid, U, self.scale_post, bias=bias, tiled=tiled, bind_y=True)
             rl.build()
+            rl.status_check_every = self.fused_status_every
             self._fused_lists[key] = rl
             # The first launch of a new list is checked (one synchronisation per list): the kernel needs its whole
             # grid resident at once, and a device shared with other work makes its bounded waits expire.

@@ -61,6 +61,10 @@ class DecodeRunList:
         self._entries: List[dict] = []
         self._keep: list = []          # tensors referenced by raw pointers stay alive here
         self._workspace: Optional[torch.Tensor] = None
+        # > 0: every so many launches `run` reads the status word (a synchronisation) and raises if a dependency wait
+        # expired since the last check; never while the stream is being captured.  0: the caller polls `status()`.
+        self.status_check_every = 0
+        self._runs = 0
 
     # ---- building -----------------------------------------------------------------------------
     def add(self, x: Optional[torch.Tensor], scale_pre: torch.Tensor, V_int8: torch.Tensor, scale_mid: Optional[torch.Tensor],
@@ -170,6 +174,12 @@ class DecodeRunList:
             stream = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
             _lib.check(_lib.lib().nq_runlist_run_bound(ctypes.c_void_p(self._workspace.data_ptr()),
                                                        ctypes.byref(self._plan), p(x), p(y), stream))
+        self._runs += 1
+        if self.status_check_every > 0 and self._runs % self.status_check_every == 0 \
+                and not torch.cuda.is_current_stream_capturing():
+            if self.status() != 0:
+                raise RuntimeError("a dependency wait of a run-list launch expired since the last check (is the GPU shared "
+                                   "with other kernels?): the outputs of that launch are invalid")
         return self.outputs
 
     def status(self) -> int:

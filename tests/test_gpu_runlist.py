@@ -563,6 +563,74 @@ def test_an_expired_wait_is_reported_and_the_list_stays_usable(dev):
         assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < 1e-2   # rank 40: the fp16-output budget
 
 
+def test_periodic_status_check_raises_after_an_expired_wait(dev):
+    """`status_check_every = k`: every k-th `run` reads the status word back and raises when a wait expired since the
+    last check, so that a caller who never polls `status()` cannot go on using invalid outputs for long."""
+    term, ops = _term(dev, 8192, 4096, 40, seed=860)
+    rl = DecodeRunList(1, torch.float16, dev)
+    rl.add(torch.from_numpy(oracle.synth_x(1, 4096, 861)).to(dev), *ops)
+    rl.status_check_every = 3
+    for _ in range(6):                                                 # two checks, both clean
+        rl.run()
+    rl.spin_limit = 1                                                  # the next launch gives up at its first unmet wait
+    rl.run()
+    rl.spin_limit = 0
+    rl.run()
+    with pytest.raises(RuntimeError, match="dependency wait"):
+        rl.run()                                                       # the ninth launch checks
+    torch.cuda.synchronize()
+    assert rl.status() == 0                                            # the check cleared the flag
+    for _ in range(3):
+        ys = rl.run()
+    ref = oracle.layer_forward(oracle.synth_x(1, 4096, 861).astype(np.float64), *term, dtype=np.float64)
+    assert oracle.max_rel_err(ys[0].float().cpu().numpy(), ref) < 1e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("batch", [1, 2, 4, 8, 16])
+def test_grid_fits_every_kernel_variant(dev, batch, dtype):
+    """The run-list kernel is only correct with its whole grid resident.  A plan can be launched on several kernel
+    variants (word order, reproducible sums, wavefronts owning row pairs) with LDS sizes of their own, and reproducible
+    sums are switched on after the grid is fixed: the grid must fit the smallest of them, and a launch whose grid does
+    not fit the variant it would start is refused instead of started."""
+    import ctypes
+    from nanoquant_amd import _lib
+    lib = _lib.lib()
+    dt = _lib.NQ_F16 if dtype == torch.float16 else _lib.NQ_BF16
+    for max_units in (8, 32, 86, 344, 1000):
+        caps = [lib.nq_runlist_capacity(batch, dt, max_units, v) for v in range(6)]
+        smallest = lib.nq_runlist_capacity(batch, dt, max_units, -1)
+        print(f"capacity batch={batch} {dtype} max_units={max_units}: {caps} -> {smallest}", flush=True)
+        assert all(c >= 0 for c in caps) and caps[0] > 0 and caps[2] > 0
+        assert smallest == min(c for c in caps if c > 0)
+    assert lib.nq_runlist_capacity(3, dt, 32, -1) == 0 and lib.nq_runlist_capacity(batch, dt, 32, 6) == 0
+    # a built list: the grid fits every variant, with and without reproducible sums, and both launch
+    term, ops_ = _term(dev, 512, 1024, 128, seed=850)
+    x = torch.from_numpy(oracle.synth_x(batch, 1024, 851)).to(dev, dtype)
+    rl = DecodeRunList(batch, dtype, dev)
+    rl.add(x, *[t if t is None or t.dtype == torch.int32 else t.to(dtype) for t in ops_])
+    rl.build()
+    plan = rl._plan
+    for v in range(6):
+        c = lib.nq_runlist_capacity(batch, dt, plan.max_units, v)
+        assert c == 0 or plan.workgroups <= c, (v, c, plan.workgroups)
+    y0 = rl.run()[0].clone()
+    assert lib.nq_runlist_set_deterministic(ctypes.byref(plan), 1) == 0     # after the grid was fixed
+    y1 = rl.run()[0].clone()
+    torch.cuda.synchronize()
+    assert rl.status() == 0
+    assert torch.allclose(y0.float(), y1.float(), rtol=2e-2, atol=2e-3 * float(y0.float().abs().max()))
+    # a plan whose grid was inflated behind the library's back is refused, nothing is launched
+    from nanoquant_amd.runlist import NqRunlistPlan
+    bad = NqRunlistPlan.from_buffer_copy(plan)
+    bad.workgroups = bad.index_words = 1 << 20
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    st = lib.nq_runlist_run(ctypes.c_void_p(rl._workspace.data_ptr()), ctypes.byref(bad), stream)
+    assert st == _lib.NQ_ERR_HIP
+    torch.cuda.synchronize()
+    assert rl.status() == 0
+
+
 @pytest.mark.parametrize("seed", range(16))
 def test_random_lists_match_the_oracle(dev, seed):
     """Seeded random lists: batch, type, word order, reproducible sums, 1 to 4 linears of ragged shapes, some fed by
