@@ -31,8 +31,9 @@ HBM_PEAK_GBS = 8000.0
 # copy kernel of known size (profiles/gemv_stream_llama2_7b_stack_b1.md); valid for the default workload only.
 MEASURED_TRAFFIC_BYTES = 843630592
 # The same for the two launches of the 128-token grouped layer (profiles/gemm_group_llama2_7b_layer_prefill.md):
-# (18776 + 27306) KiB x 2.000 fetched + (4352 + 10624) KiB written.
-MEASURED_PREFILL_TRAFFIC_BYTES = (18776 + 27306) * 2 * 1024 + (4352 + 10624) * 1024
+# (18786 + 25962) KiB x 2.000 fetched + (4352 + 48583) KiB written; 38.8 MB each way of the second launch are partial
+# tiles that its workgroups hand over through device-coherent memory.
+MEASURED_PREFILL_TRAFFIC_BYTES = (18786 + 25962) * 2 * 1024 + (4352 + 48583) * 1024
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 LLAMA2_7B_LAYER = (("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096),

@@ -238,6 +238,26 @@ class LinearStack:
         step.status = lambda: 0
         return step
 
+    def make_group_step(self, xs, one_launch: bool = False):
+        """What a decoder with attention between its projections can issue without a run list: per layer the groups
+        {q, k, v}, {o}, {gate, up}, {down} (one group per linear for other shapes), each group two launches
+        (`ops.gemv_group_forward`), or one with `one_launch`."""
+        from . import ops
+        torch = self.torch
+        nlin = len(self.layers[0])
+        groups = ((0, 1, 2), (3,), (4, 5), (6,)) if nlin == 7 else tuple((i,) for i in range(nlin))
+        batch = xs[0].shape[0]
+        outs = [torch.empty(batch, lin["m"], dtype=self.dtype, device=self.device) for lin in self.layers[0]]
+
+        def step():
+            for layer in self.layers:
+                for grp in groups:
+                    ops.gemv_group_forward([xs[j] for j in grp],
+                                           [(layer[j]["s_in"], layer[j]["vt"], layer[j]["s_mid"], layer[j]["u"], layer[j]["s_out"])
+                                            for j in grp], outs=[outs[j] for j in grp], one_launch=one_launch)
+        step.status = lambda: ops.gemv_group_status(self.device)
+        return step
+
     # -- prefill ---------------------------------------------------------------------------------
     def prefill(self, tokens: int, seed: int) -> float:
         """One pass of `tokens` rows through the prefill (GEMM) kernels of every linear; seconds.  The prefill
@@ -278,6 +298,8 @@ def run_config(stack: LinearStack, args, bs: int, pt: int, new: int, power: bool
         step = stack.make_runlist_step(bs, xs, per_layer=False, tiled=args.tiled)
     elif kind == "runlist-per-layer":
         step = stack.make_runlist_step(bs, xs, per_layer=True, tiled=args.tiled)
+    elif kind in ("gemv-group", "gemv-group-one-launch"):
+        step = stack.make_group_step(xs, one_launch=kind.endswith("one-launch"))
     else:
         step = stack.make_op_step(xs)
     graph = None
@@ -345,9 +367,11 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--model_shape", default="llama2-7b", choices=sorted(MODEL_SHAPES))
     p.add_argument("--layers", type=int, default=0, help="decoder layers (0: the model's own count)")
     p.add_argument("--bits", type=float, default=1.0, help="bits per weight of the factorisation")
-    p.add_argument("--quant_kernel_type", default="runlist", choices=["runlist", "runlist-per-layer", "gemv"],
+    p.add_argument("--quant_kernel_type", default="runlist",
+                   choices=["runlist", "runlist-per-layer", "gemv", "gemv-group", "gemv-group-one-launch"],
                    help="runlist: the whole stack in one launch per token; runlist-per-layer: one launch per layer; "
-                        "gemv: the reference's way, one operator call (two launches) per linear")
+                        "gemv: the reference's way, one operator call (two launches) per linear; gemv-group: per layer "
+                        "the groups {q,k,v}, {o}, {gate,up}, {down}, two launches each; gemv-group-one-launch: one each")
     p.add_argument("--batch_size", default="1", help="list, e.g. 1,4,16")
     p.add_argument("--prompt_tokens", default="128", help="list of prompt lengths for the prefill pass (0: none)")
     p.add_argument("--max_new_tokens", default="128", help="list")

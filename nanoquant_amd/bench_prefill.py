@@ -39,6 +39,9 @@ def run(argv=None) -> List[Dict[str, Any]]:
     ap.add_argument("--no_graph", action="store_true")
     ap.add_argument("--no_group", action="store_true")
     ap.add_argument("--no_single", action="store_true", help="skip the one-linear-after-the-other leg")
+    ap.add_argument("--panel", default="auto", choices=("auto", "always", "never"),
+                    help="grouped leg: persistent panel launches where the library's policy picks them (auto), for every "
+                         "stage (always), or the launches without a workspace only (never)")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args(argv)
 
@@ -102,13 +105,13 @@ def run(argv=None) -> List[Dict[str, Any]]:
         xs_by_n = {n: torch.randn(tokens, n, device=dev, generator=gen).to(dtype) for n in {n for (_, _, n) in shapes}}
         xs = [xs_by_n[n] for (_, _, n) in shapes]
         flops = sum(2.0 * tokens * packed_by_shape[(m, n)][1] * (m + n) for (_, m, n) in shapes)
-        row: Dict[str, Any] = {"model_shape": args.model_shape, "tokens": tokens, "dtype": args.dtype,
+        row: Dict[str, Any] = {"model_shape": args.model_shape, "tokens": tokens, "dtype": args.dtype, "panel": args.panel,
                                "linears": len(shapes), "GFLOP_per_layer": round(flops / 1e9, 2)}
         legs = []
         if not args.no_single:
             legs.append(("one_by_one", lambda: [op(x, *t) for x, t in zip(xs, terms)]))
         if not args.no_group:
-            legs.append(("grouped", lambda: ops.gemm_group_forward(xs, terms)))
+            legs.append(("grouped", lambda: ops.gemm_group_forward(xs, terms, panel=args.panel)))
         for name, fn in legs:
             us = timed(fn)
             tf = flops / (us * 1e-6) / 1e12

@@ -357,8 +357,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
     // ---- grid = what the device keeps resident; every workgroup gets an equal share of every phase ----
     // Which arithmetic: at batch 4 (fp16) a list with little work per workgroup (up to two Llama-2-7B layers on 256
     // workgroups: 14000 rows x 16-byte units each) runs on the 16-bit arithmetic of batch 8 and 16, whose staging costs a
-    // tenth of the quantising one; longer lists stream faster on the fp4 x fp8 arithmetic (crossover measured at 2.6
-    // layers: 24 against 31 us for one layer per launch, 9.6 against 6.3 us per layer for 16).
+    // tenth of the quantising one; longer lists stream faster on the fp4 x fp8 arithmetic (the two cross at 2.6 layers).
     bool alt = false;
     if (nq::stream_has_alt(dtype, batch)) {
         long long work = 0;
@@ -494,9 +493,8 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         // fill (never starting a slice that cannot hold a quarter of the fixed part in arithmetic) needs at most
         // the resident workgroups.
         {
-            // (the variant whose wavefronts own row pairs starts every slice without fetches in flight: 16000, from
-            // sweeps of the Llama-2-7B stack at batch 4 and 2: 5.8 against 5.95 and 5.3 against 5.45 us per layer;
-            // at batch 1 6000 / 10000 / 16000 / 24000 / 40000 give 6120 / 6149 / 6085 / 5990 / 5709 GB/s on that stack)
+            // (the variant whose wavefronts own row pairs starts every slice without fetches in flight, so a slice
+            // costs it more to start: 16000, and 10000 at batch 1, the best of sweeps on the Llama-2-7B stack)
             const long long fixed = own ? (batch == 1 ? 10000 : 16000) : wide ? 2200 : batch == 1 ? 8800 : batch == 2 ? 6600 : 4400;
             auto gran = [&](size_t k) { return table[ids[k]].tiled ? granule : 1; };
             // Batch 8 and 16: an input too long to be staged at once is staged again, chunk by chunk, for every 256 rows

@@ -448,22 +448,15 @@ static GemmPlan plan_gemm(int T, int K, int R) {
     p.kwave = false;
     // A long k (more than 16 tiles) needs a k-split with atomics and a finish launch on block tiles, while the
     // wavefronts of a few-token tile split k for free: those GEMMs stay on few-token tiles up to 1024 tokens
-    // (k 11008 -> 3072 rows: 512 tokens 51.3 vs 55.5 us, 1024 tokens 79.3 vs 94.7, 2048 tokens 148.8 vs 147.0).
+    // (the two kernels cross at 2048 tokens for k 11008 -> 3072 rows).
     if (T <= kKwaveMaxTokens || (K / kTileK > 16 && T <= 1024)) {
-        // 32x32 output tiles, wavefronts split k: no k-split scratch, one launch (4096x4096 at 128 tokens:
-        // 16.8 vs 22.7 us per linear with the block kernel).  The 7 linears of a Llama-2-7B layer one after the other,
-        // few-token vs block tiles: 144 tokens 191 vs 224 us, 160: 193 vs 231, 192: 220 vs 246, 256: 236 vs 252,
-        // 288: 287 vs 268, 384: 313 vs 300, 448: 349 vs 314.
+        // 32x32 output tiles, wavefronts split k: no k-split scratch, one launch.  For the linears of a Llama-2-7B
+        // layer one after the other these tiles are ahead of the block tiles up to 256 tokens, behind from 288 on.
         p.kwave = true;
         p.tt = 1; p.gy = (T + 31) / 32;
         // Every 32-row tile re-reads the 32-token activation slab, so wider workgroups save L2 traffic: with a
-        // long k the widest that still leaves workgroups for three quarters of the CUs.  Measured (us per GEMM, 1 / 2 / 4 row tiles):
-        // 128 tokens: 2048 rows k 4096: 8.3 / 9.8 / 13.6; 3072 rows k 4096: 10.9 / 9.9 / 13.5; 3072 rows k 11008:
-        // 23.3 / 20.1 / 27.5; 4096 rows k 3072: 8.9 / 8.7 / 11.9; 11008 rows k 3072: 21.8 / 18.5 / 18.9;
-        // 256 tokens: 2048 rows k 4096: 10.8 / 10.9 / 14.2; 3072 rows k 4096: 16.5 / 14.3 / 14.1; 3072 rows k 11008:
-        // 36.5 / 34.3 / 31.5; 4096 rows k 3072: 12.2 / 11.9 / 12.2.
-        // With a short k a workgroup is gone before its neighbours have started, and more of them do better: two
-        // per CU there (11008 rows k 3072 at 128 tokens: 688 workgroups of two row tiles, 2 us per linear faster than 344 of four).
+        // long k the widest that still leaves workgroups for three quarters of the CUs.  With a short k a workgroup
+        // is gone before its neighbours have started, and more of them do better: two per CU there.
         const int min_workgroups = K / kTileK >= 16 ? 192 : 512;
         p.rt = 1;
         for (int rt = 2; rt <= 4; rt *= 2)
@@ -478,9 +471,7 @@ static GemmPlan plan_gemm(int T, int K, int R) {
     p.tt = 2;
     {
         // Few tokens: 32-token blocks give twice the workgroups, which can spare the k-split and with it
-        // the atomics and the finish launch (4096x4096 at 256 tokens: 44 -> 27 us per linear; with the bound on
-        // 64-token workgroups raised from 256 to 512: 4096x4096 at 512 tokens 45.5 -> 33.6 us, at 1024 tokens
-        // 59.3 -> 49.5 us, 4096x11008 at 512 tokens 80.2 -> 71.0 us, the other shapes within 5 %).  Only when
+        // the atomics and the finish launch (4096x4096 at 256 tokens: 44 -> 27 us per linear).  Only when
         // k is short enough for one workgroup to walk it (<= 16 tiles).
         const int gx1 = (R + 127) / 128, gy1 = (T + 31) / 32;
         if (gx1 * ((T + 63) / 64) < 512 && gx1 * gy1 >= 128 && K / kTileK <= 16) {

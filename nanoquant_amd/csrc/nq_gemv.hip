@@ -335,9 +335,9 @@ static hipError_t launch_stage_batch(StageArgs a, int batch, hipStream_t stream)
 
 static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
-// Pieces of 8 and 16 batch rows go through the run-list kernel on this one stage (MFMA unit arithmetic, us per
-// Llama-2-7B layer: batch 8 157 vs 240, batch 16 225 vs 570); smaller pieces are as fast or faster on the lane-group
-// kernel below, whose launches carry less fixed cost (batch 4: 131 vs 133, batch 1: 80 vs 111).
+// Pieces of 8 and 16 batch rows go through the run-list kernel on this one stage (MFMA unit arithmetic: 1.5 and 2.5
+// times faster there); smaller pieces are as fast or faster on the lane-group kernel below, whose launches carry less
+// fixed cost.
 static bool use_stream_kernel(int piece) { return piece >= 8; }
 
 // One stage over `batch` input rows, any batch >= 1: split into power-of-two pieces of at most 16.

@@ -336,8 +336,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
             if constexpr (kQ8) {
                 // The packed words depend on nothing: the first three items of the slice are asked for before the
                 // dependency wait and the staging of the input (in tile order: unless the previous pass already did),
-                // and arrive while those run.  (Sending them out behind the first input loads of a slice that waits for
-                // nothing, so that the input does not queue behind them, gained 0.3 of 20 us per one-layer launch.)
+                // and arrive while those run.
                 if constexpr (OWN) {
                     // the first fetches are sent out after the staging
                 } else if constexpr (TILED) {
@@ -461,10 +460,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                 // on any order left to the hardware.  With an input of one chunk the wavefronts of a workgroup meet once
                 // per slice (after the staging) and the item fetches of a wavefront run on from group to group; with a
                 // longer input the chunks are staged again for every round and the accumulators are kept across the
-                // chunks of a round.  In the last round of a slice some wavefronts have no group.  (Sharing that round
-                // out item by item, with LDS float atomics into 20 KB of row sums and an epilogue by all lanes, measured
-                // the same on long lists and slower on short ones: 58 against 47 us per Llama-2-7B layer and launch at
-                // batch 16.)
+                // chunks of a round.  In the last round of a slice some wavefronts have no group.
                 const int lane = tid & 63, r16 = lane & 15, g = lane >> 4;
                 const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // scalar item arithmetic
                 constexpr int kAccs = Pow2<DT>::kClasses;
@@ -667,7 +663,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
                     const int nrows = seg.row_end - seg.row_begin;
                     const int npairs = (nrows + 31) >> 5;
                     const int ngroups = (cu_n + 3) >> 2;
-                    constexpr int kOwnDepth = 3;                       // item fetches in flight per wavefront (2 against 3: within +-1.5 % at batch 1, 2 and 4)
+                    constexpr int kOwnDepth = 3;                       // item fetches in flight per wavefront
                     const int positions = (ngroups + kOwnDepth - 1) / kOwnDepth * kOwnDepth;   // the register pairs keep their turns from pair to pair
                     // results that need only their row scale go out as buffer stores (see the end of a pair)
                     const size_t out_elems = (size_t)(BATCH - 1) * st.out_stride + st.rows;
@@ -1058,19 +1054,13 @@ static void stream_lds_plan(int batch, int arith, int max_units, int* chunk_cap_
     *lds_out = (size_t)racc_bytes + xs_bytes;
 }
 
-// Which arithmetic, by batch (measured on Llama-2-7B layers with row-major words: one launch per layer / 26 layers
-// per launch, us per layer):
-//                                          batch 1        batch 2        batch 4
-//   fp4 x fp8 pieces (ARITH 2), any type   20.2 /  6.9    24.1 /  7.4    31.4 / 10.9
-//   16-bit MFMA operands (ARITH 1), fp16   25.4 / 11.5    25.5 / 11.9    29.8 / 14.2
-//                                   bf16   36.4 / 21.1    31.1 / 17.1    32.3 / 18.4
-// The fp4 x fp8 arithmetic is three times cheaper per packed bit, but every workgroup quantises the whole input
-// vector of its stage (about 110 VALU instructions per 8 columns and batch row): at batch 4 that costs as much as
-// the arithmetic saves when a launch covers only one layer, and a third less time in long run lists (Llama-3-70B
-// stream at batch 4: 2.3 against 3.6 ms).  Its staging does not depend on the element type, so bf16 runs as fast
-// as fp16.  Batch 8 and 16 need more operand columns than one MFMA has.
+// Which arithmetic, by batch.  The fp4 x fp8 arithmetic (ARITH 2) is three times cheaper per packed bit than the
+// 16-bit MFMA operands (ARITH 1), but every workgroup quantises the whole input vector of its stage (about 110 lane
+// instructions per 8 columns and batch row): at batch 4 that costs as much as the arithmetic saves when a launch
+// covers only one layer, and a third less time in long run lists.  Its staging does not depend on the element type,
+// so bf16 runs as fast as fp16.  Batch 8 and 16 need more operand columns (batch rows x 3 pieces) than one MFMA has.
 // Every workgroup stages the whole input vector of its stage, so larger workgroups mean less staging work per
-// row: 1024 lanes everywhere (batch 16: 211 -> 80 us per layer going from 256 to 1024 lanes).
+// row: 1024 lanes everywhere.
 #ifndef NQ_STREAM_ARITH
 #define NQ_STREAM_ARITH(DT, BATCH) ((BATCH) <= 4 ? 2 : 1)
 #endif
@@ -1078,12 +1068,11 @@ static void stream_lds_plan(int batch, int arith, int max_units, int* chunk_cap_
 #define NQ_STREAM_THREADS(DT, BATCH) 1024
 #endif
 
-// Short lists at batch 4 run faster on the 16-bit arithmetic (one Llama-2-7B layer per launch: 24 against 31 us; its
-// staging is a tenth of the quantising one), long ones on the fp4 x fp8 arithmetic (16 layers per launch: 6.3 against
-// 9.6 us per layer): the builder picks per list (`alt`).  At batch 1 and 2 the fp4 x fp8 arithmetic wins or ties
-// everywhere (19 against 22, 22.5 against 22.3 us for one layer).  fp16 only: the 16-bit arithmetic rounds x * s_in and
-// the intermediate vector to the activation type, which costs bf16 lists a factor of eight in accuracy (2.3e-3 against
-// 3e-4 of the output maximum) where the fp4 x fp8 pieces are as exact for bf16 as for fp16.
+// Short lists at batch 4 run faster on the 16-bit arithmetic (its staging is a tenth of the quantising one), long
+// ones on the fp4 x fp8 arithmetic: the builder picks per list (`alt`).  At batch 1 and 2 the fp4 x fp8 arithmetic
+// wins or ties everywhere.  fp16 only: the 16-bit arithmetic rounds x * s_in and the intermediate vector to the
+// activation type, which costs bf16 lists a factor of eight in accuracy (2.3e-3 against 3e-4 of the output maximum)
+// where the fp4 x fp8 pieces are as exact for bf16 as for fp16.
 constexpr bool stream_alt_exists(int dtype, int batch) { return dtype == 0 && batch == 4; }
 
 template <int DT, int BATCH, int ARITH = NQ_STREAM_ARITH(DT, BATCH)>
@@ -1093,12 +1082,9 @@ struct StreamKernel {
     static constexpr auto fn = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, false>;
     static constexpr auto fn_tiled = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2>;
     // tile order, fp4 x fp8 arithmetic, wavefronts own row pairs: for lists whose longest input is staged in one chunk.
-    // Measured against the row-block form on Llama-2-7B stacks (us per layer, 1 / 2 / 4 / 8 / 32 layers per launch):
-    // batch 4  31.3 / 16.7 / 9.9 / 6.5 / 5.9 against 31.1 / 17.5 / 10.8 / 7.5 / 6.8 (no LDS atomics: four batch rows cost
-    // four times the flushes); batch 2  25.4 / 13.6 / 8.3 / 6.1 / 5.25 against 23.0 / 12.9 / 8.4 / 6.2 / 5.5 (a short
-    // slice has fewer row pairs than wavefronts); batch 1  32 layers 1.8 % slower, one layer 21.0 against 18.9 (the
-    // stores of a pair stop its fetches, and one batch row has little to flush): the builder asks for it at batch 4
-    // and, for long lists, at batch 2.
+    // It has no row sums in LDS and no LDS atomics, which pays at batch 4 (four batch rows cost four times the flushes)
+    // and in long lists at batch 1 and 2; a short slice has fewer row pairs than the workgroup has wavefronts, so the
+    // builder asks for it at batch 4 and, for long lists, at batch 1 and 2.
     static constexpr bool kHasOwn = kArith == 2 && BATCH <= 4;
     static constexpr auto fn_tiled_own = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2, false, kHasOwn>;
     static constexpr auto fn_tiled_own_det = gemv_stream_kernel<DT, BATCH, kArith, kThreads, false, kArith == 2, kHasOwn, kHasOwn>;

@@ -603,13 +603,26 @@ def gemv_stage_forward(inp: torch.Tensor, s_col: Optional[torch.Tensor], bits: t
 
 
 def tile_words_device(packed: torch.Tensor, inverse: bool, shape=None) -> torch.Tensor:
-    """Device pass of packing.tile_words / untile_words."""
+    """Device pass of packing.tile_words / untile_words.  The kernel trusts its sizes: what it is handed is checked
+    here (a GPU tensor of contiguous int32 words, exactly as many as the shape needs, 16-byte aligned on the tiled
+    side)."""
     lib = _lib.lib()
+    if not packed.is_cuda:
+        raise RuntimeError("packed words must be a CUDA tensor")
+    if packed.dtype != torch.int32 or not packed.is_contiguous():
+        raise RuntimeError("packed words must be a contiguous int32 tensor")
     if not inverse:
+        if packed.dim() != 2:
+            raise RuntimeError("row-major words must be a 2-D tensor [rows, words]")
         rows, words = packed.shape
         out = torch.empty(int(lib.nq_tiled_words(rows, words)), dtype=torch.int32, device=packed.device)
     else:
-        rows, words = shape
+        rows, words = (int(v) for v in shape)
+        if rows < 0 or words < 0 or packed.dim() != 1 or packed.numel() != int(lib.nq_tiled_words(rows, words)):
+            raise RuntimeError(f"tiled words of a [{rows}, {words}] matrix must be a flat tensor of "
+                               f"{int(lib.nq_tiled_words(rows, words))} words, got {list(packed.shape)}")
+        if packed.data_ptr() % 16 != 0:
+            raise RuntimeError("tiled words must be 16-byte aligned")
         out = torch.empty((rows, words), dtype=torch.int32, device=packed.device)
     if rows > 0 and words > 0:
         with torch.cuda.device(packed.device):

@@ -63,7 +63,7 @@ def test_parser_defaults_follow_the_reference_names():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("kind", ["runlist", "runlist-per-layer", "gemv"])
+@pytest.mark.parametrize("kind", ["runlist", "runlist-per-layer", "gemv", "gemv-group", "gemv-group-one-launch"])
 def test_tiny_sweep_writes_rows_and_aggregates(dev, tmp_path, kind):
     out = tmp_path / "sweep.csv"
     rc = bd.main(["--model_shape", "tiny", "--batch_size", "1,2", "--prompt_tokens", "32", "--max_new_tokens", "5",

@@ -236,6 +236,23 @@ def test_tile_order_on_the_device(dev, rows, words):
     assert np.array_equal(back.cpu().numpy(), a)
 
 
+def test_tile_order_pass_checks_what_it_is_handed(dev):
+    # the device pass trusts its sizes: tensors of another type, layout, size or alignment are refused on the host
+    from nanoquant_amd import ops
+    a = torch.zeros((70, 47), dtype=torch.int32, device=dev)
+    t = packing.tile_words(a)
+    for bad in (a.cpu(), a.to(torch.int64), a.t(), a.view(-1)):
+        with pytest.raises(RuntimeError):
+            ops.tile_words_device(bad, inverse=False)
+    for bad, shape in ((t[:-4], (70, 47)), (t, (70, 48 + 16)), (t.view(2, -1), (70, 47)), (t.to(torch.int64), (70, 47))):
+        with pytest.raises(RuntimeError):
+            ops.tile_words_device(bad, inverse=True, shape=shape)
+    longer = torch.zeros(t.numel() + 1, dtype=torch.int32, device=dev)
+    with pytest.raises(RuntimeError, match="aligned"):
+        ops.tile_words_device(longer[1:], inverse=True, shape=(70, 47))
+    assert torch.equal(packing.untile_words(t, (70, 47)), a)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("batch", [1, 2, 4, 16])
 def test_tiled_factors_give_the_same_layer(dev, batch, dtype):
