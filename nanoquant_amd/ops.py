@@ -84,8 +84,32 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else ctypes.c_void_p(t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(dev: torch.device):
+    """The current stream of `dev` as the C ABI takes it.  The raw-handle query costs a tenth of building a
+    `torch.cuda.Stream` object, which counts on a decode call that the GPU finishes in microseconds."""
+    if _raw_stream is not None and dev.index is not None:
+        return ctypes.c_void_p(_raw_stream(dev.index))
     return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+class _on_device:
+    """`torch.cuda.device(dev)` that does nothing when `dev` is already the current device (the usual case)."""
+    __slots__ = ("ctx",)
+
+    def __init__(self, dev: torch.device):
+        self.ctx = None if (dev.index is None or dev.index == torch.cuda.current_device()) else torch.cuda.device(dev)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+        return False
 
 
 # ---------------------------------------------------------------------------------------------
@@ -129,8 +153,8 @@ def _check_bias(bias, m, x):
         raise RuntimeError(f"bias must be [{m}], got {list(bias.shape)}")
 
 
-def _gemv_forward(x, scale_g, Ubits, scale_l, Vbits, scale_h, bias=None):
-    n, r, m = _check_gemv_args(x, scale_g, Ubits, scale_l, Vbits, scale_h)
+def _gemv_forward(x, scale_g, Ubits, scale_l, Vbits, scale_h, bias=None, dims=None):
+    n, r, m = dims if dims is not None else _check_gemv_args(x, scale_g, Ubits, scale_l, Vbits, scale_h)
     _check_bias(bias, m, x)
     lead = x.shape[:-1]
     batch = 1
@@ -139,7 +163,7 @@ def _gemv_forward(x, scale_g, Ubits, scale_l, Vbits, scale_h, bias=None):
     y = torch.empty((batch, m), dtype=x.dtype, device=x.device)
     if batch > 0 and m > 0:
         h = torch.empty((batch, max(r, 1)), dtype=torch.float32, device=x.device)
-        with torch.cuda.device(x.device):
+        with _on_device(x.device):
             _lib.check(_lib.lib().nq_gemv_forward_bias(_ptr(x), _ptr(scale_g), _ptr(Ubits), _ptr(scale_l), _ptr(Vbits),
                                                        _ptr(scale_h), _ptr(bias), _ptr(h), _ptr(y), batch, n, r, m,
                                                        _dtype_id(x), _stream(x.device)))
@@ -153,7 +177,7 @@ def nanoquant_dyn_forward(x, scale_g, Ubits, scale_l, Vbits, scale_h,
                           num_pipeline_stage1=2, num_pipeline_stage2=2):
     """y = scale_h * (Vbits (scale_l * (Ubits (scale_g * x)))): `Ubits` [r, n/32] is the FIRST stage,
     `Vbits` [m, r/32] the second (the reference's argument names, pybind.cpp:86-90)."""
-    _check_gemv_args(x, scale_g, Ubits, scale_l, Vbits, scale_h)
+    dims = _check_gemv_args(x, scale_g, Ubits, scale_l, Vbits, scale_h)
     _sweep("n_th1", num_thread_stage1)
     _sweep("n_rpw1", num_row_per_warp_stage1)
     _sweep("n_acc1", num_acc_stage1)
@@ -162,7 +186,7 @@ def nanoquant_dyn_forward(x, scale_g, Ubits, scale_l, Vbits, scale_h,
     _sweep("n_rpw2", num_row_per_warp_stage2)
     _sweep("n_acc2", num_acc_stage2)
     _sweep("n_pipe2", num_pipeline_stage2)
-    return _gemv_forward(x, scale_g, Ubits, scale_l, Vbits, scale_h)
+    return _gemv_forward(x, scale_g, Ubits, scale_l, Vbits, scale_h, dims=dims)
 
 
 def _nanoquant_dyn_forward_meta(x, scale_g, Ubits, scale_l, Vbits, scale_h, *hints, **kw):
@@ -373,7 +397,7 @@ def gemv_group_forward(xs, linears, biases=None, outs=None, one_launch=False):
     for i, (x, (sg, ub, sl, vb, sh), b, y, (n, r, m)) in enumerate(zip(xs, linears, biases, outs, dims)):
         arr[i] = NqLinear(p(x), p(sg), p(ub), p(sl), p(vb), p(sh), h.data_ptr() + 4 * offsets[i], p(y), None, n, r, m, -1, -1, 0,
                           p(b), 0)
-    with torch.cuda.device(x0.device):
+    with _on_device(x0.device):
         _lib.check(_lib.lib().nq_gemv_forward_group(arr, len(linears), batch, _dtype_id(x0), 1 if one_launch else 0,
                                                      _stream(x0.device)))
     return outs
