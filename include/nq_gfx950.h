@@ -193,6 +193,10 @@ int nq_runlist_set_deterministic(nq_runlist_plan* plan, int on);
 int nq_gemv_group_max(void);
 int nq_gemv_forward_group(const nq_linear* linears, int count, int batch, int dtype, int one_launch, void* stream);
 int nq_gemv_group_status(int* status_out, void* stream);
+/* Polls after which the wait of a one_launch group gives up (0 = the default of 2^20).  Process-wide.  Lowering it to 1
+ * makes a launch report an expiry at once, which is how a caller's handling of status 1 can be exercised from the
+ * host; every kernel still runs to its end. */
+int nq_gemv_group_set_spin_limit(unsigned polls);
 
 /* One matmul-free stage: out[b,row] = s_row[row] * sum_c sgn(bits[row,c]) * in[b,c] * s_col[c].
  * Replaces nanoquant_stage1_dyn_kernel / nanoquant_stage2_dyn_kernel launches
@@ -277,6 +281,9 @@ size_t nq_gemm_panel_workspace_bytes(void);
 int nq_gemm_nanoquant_group_ws(const nq_gemm_term* terms, int count, int tokens, int dtype, void* scratch,
                                size_t scratch_bytes, void* panel_ws, size_t panel_ws_bytes, int panel_mode, void* stream);
 int nq_gemm_panel_status(const void* panel_ws, int* status_out, void* stream);
+/* Polls after which a wait of a panel launch gives up (0 = the default of 2^20).  Process-wide; for exercising a
+ * caller's handling of status 1 from the host, as nq_gemv_group_set_spin_limit. */
+int nq_gemm_panel_set_spin_limit(unsigned polls);
 
 /* Word-order conversion on the device, in place allowed (dst == src): the checkpoint format
  * ("lsb_first", modules/linear.py:298) to the kernel format ("half2", modules/linear.py:171-172)

@@ -28,6 +28,7 @@ _SIGNATURES = {
     "nq_gemv_group_max": (_i, []),
     "nq_gemv_forward_group": (_i, [_vp, _i, _i, _i, _i, _vp]),
     "nq_gemv_group_status": (_i, [ctypes.POINTER(_i), _vp]),
+    "nq_gemv_group_set_spin_limit": (_i, [ctypes.c_uint]),
     "nq_gemv_mixture": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "nq_runlist_workspace_bytes": (_sz, [_vp, _i]),
     "nq_runlist_build": (_i, [_vp, _i, _i, _i, _i, _vp, _sz, _vp, _vp]),
@@ -48,6 +49,7 @@ _SIGNATURES = {
     "nq_gemm_panel_workspace_bytes": (_sz, []),
     "nq_gemm_nanoquant_group_ws": (_i, [_vp, _i, _i, _i, _vp, _sz, _vp, _sz, _i, _vp]),
     "nq_gemm_panel_status": (_i, [_vp, ctypes.POINTER(_i), _vp]),
+    "nq_gemm_panel_set_spin_limit": (_i, [ctypes.c_uint]),
     "nq_pack_gemm_tiles": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "nq_tiled_words": (_sz, [_i, _i]),
     "nq_tile_words": (_i, [_vp, _vp, _i, _i, _i, _vp]),

@@ -4,6 +4,7 @@
 #include "nq_kernels.h"
 
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -147,6 +148,11 @@ int nq_gemv_forward_group(const nq_linear* linears, int count, int batch, int dt
             if (linears[j].m && linears[j].h == l.h) return NQ_ERR_SHAPE;                               // every linear needs an h of its own
     }
     return forward_linears(linears, count, batch, dtype, one_launch != 0, (hipStream_t)stream);
+}
+
+int nq_gemv_group_set_spin_limit(unsigned polls) {
+    nq::gemv_fused_set_spin_limit(polls);
+    return NQ_OK;
 }
 
 int nq_gemv_group_status(int* status_out, void* stream) {
@@ -698,6 +704,14 @@ int nq_gemm_nanoquant_group(const nq_gemm_term* terms, int count, int tokens, in
     return nq_gemm_nanoquant_group_ws(terms, count, tokens, dtype, scratch, scratch_bytes, nullptr, 0, NQ_PANEL_NEVER, stream);
 }
 
+// Polls after which a wait of a panel launch gives up (0: the kernel's default).  Process-wide; meant for exercising
+// a caller's handling of an expired wait from the host.
+static std::atomic<unsigned> g_panel_spin_limit{0};
+int nq_gemm_panel_set_spin_limit(unsigned polls) {
+    g_panel_spin_limit.store(polls);
+    return NQ_OK;
+}
+
 size_t nq_gemm_panel_workspace_bytes(void) { return nq::panel_workspace_bytes(); }
 
 int nq_gemm_panel_status(const void* panel_ws, int* status_out, void* stream) {
@@ -759,7 +773,8 @@ int nq_gemm_nanoquant_group_ws(const nq_gemm_term* terms, int count, int tokens,
     // one stage: the panel launch where a workspace was given and the shapes make it the faster one
     auto stage = [&]() -> hipError_t {
         if (have_ws && (panel_mode == NQ_PANEL_ALWAYS || nq::panel_applies(count, tokens, K, R)))
-            return nq::gemm_panel_group(dtype, count, x, w, si, so, bs, out, tokens, K, R, panel_ws, 0u, (hipStream_t)stream);
+            return nq::gemm_panel_group(dtype, count, x, w, si, so, bs, out, tokens, K, R, panel_ws, g_panel_spin_limit.load(),
+                                        (hipStream_t)stream);
         return nq::gemm_onebit_group(dtype, count, x, w, si, so, bs, out, tokens, K, R, (hipStream_t)stream);
     };
     for (int i = 0; i < count; ++i) {

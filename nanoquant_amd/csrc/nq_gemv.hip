@@ -421,6 +421,9 @@ static hipError_t fused_pointers(unsigned** counters, unsigned** status) {
 
 int gemv_fused_max() { return kFusedMax; }
 
+static std::atomic<unsigned> g_fused_spin_limit{0};
+void gemv_fused_set_spin_limit(unsigned polls) { g_fused_spin_limit.store(polls); }
+
 hipError_t gemv_fused_status(unsigned* out, hipStream_t stream) {
     unsigned *c = nullptr, *st = nullptr;
     hipError_t e = fused_pointers(&c, &st);
@@ -532,7 +535,8 @@ hipError_t gemv_fused(int dtype, int count, int batch, const void* const* x, con
     if (e != hipSuccess) return e;
     f.slot = counters + (size_t)(g_fused_ticket.fetch_add(1u) % kFusedSlots) * kFusedSlotWords;
     f.status = status;
-    f.spin_limit = 1u << 20;
+    const unsigned spin = g_fused_spin_limit.load();
+    f.spin_limit = spin ? spin : (1u << 20);
     const size_t lds_bytes = lds_a > lds_b ? lds_a : lds_b;
     auto launch = [&](auto kern, PerDeviceFlag& attr_done) -> hipError_t {
         hipError_t err = raise_lds(kern, lds_bytes, attr_done);

@@ -21,6 +21,7 @@ hipError_t gemv_fused(int dtype, int count, int batch, const void* const* x, con
                       const void* const* s_out, const void* const* bias, float* const* h, void* const* y,
                       const int* n, const int* r, const int* m, bool one_launch, hipStream_t stream);
 hipError_t gemv_fused_status(unsigned* out, hipStream_t stream);
+void gemv_fused_set_spin_limit(unsigned polls);          // 0: the default
 
 // nq_stream.hip: one launch over a table of stages (see the file header).
 struct RunStage {

@@ -119,6 +119,36 @@ def test_panel_launches_repeat_and_replay(dev):
     assert ops.panel_status(dev) == 0
 
 
+def test_an_expired_wait_of_a_panel_launch_is_reported(dev):
+    """The workgroups that finish a shared panel wait a bounded number of polls for the others' partial tiles.  With
+    the bound lowered to one poll from the host, a launch whose panels are shared by many workgroups reports an expiry,
+    runs to its end, and the workspace serves the next launch (default bound) as before."""
+    lib = _lib.lib()
+    dtype, tokens = torch.float16, 128
+    shapes = [(512, 2816, 256), (256, 2816, 768)]                    # 11 k tiles over few rows: every panel is shared
+    terms = [_term(dev, m, n, r, 660 + i, dtype) for i, (m, n, r) in enumerate(shapes)]
+    xs = [_cast(oracle.synth_x(tokens, n, 760 + i), dtype).to(dev) for i, (m, n, r) in enumerate(shapes)]
+    packed = [p for p, _ in terms]
+    good = [y.clone() for y in ops.gemm_group_forward(xs, packed, panel="always")]
+    torch.cuda.synchronize()
+    assert ops.panel_status(dev) == 0
+    print("panel launch with waits of one poll", flush=True)
+    assert lib.nq_gemm_panel_set_spin_limit(1) == 0
+    try:
+        ops.gemm_group_forward(xs, packed, panel="always")
+        torch.cuda.synchronize()
+        assert ops.panel_status(dev) == 1                               # reported ...
+        assert ops.panel_status(dev) == 0                               # ... once
+    finally:
+        assert lib.nq_gemm_panel_set_spin_limit(0) == 0
+    again = ops.gemm_group_forward(xs, packed, panel="always")
+    torch.cuda.synchronize()
+    assert ops.panel_status(dev) == 0
+    for y, g0, (_, ref), x in zip(again, good, terms, xs):
+        assert torch.equal(y, g0)
+        assert oracle.max_rel_err(y.float().cpu().numpy(), ref(x.float().cpu().numpy())) < TOL[dtype]
+
+
 def test_panel_entry_point_argument_checks(dev):
     lib = _lib.lib()
     dtype, tokens, n = torch.float16, 128, 512

@@ -120,6 +120,33 @@ def test_group_launches_repeat_and_replay(dev, one_launch):
     assert ops.gemv_group_status(dev) == 0
 
 
+def test_an_expired_wait_of_a_one_launch_group_is_reported(dev):
+    """The second-stage workgroups of a one-launch group wait a bounded number of polls.  With the bound lowered to one
+    poll from the host they give up at once (the first stage has only just started), the launch still runs to its end
+    and the status word says so once; with the default bound back, the next launch is right again."""
+    lib = _lib.lib()
+    dtype, batch, n = torch.float16, 1, 4096
+    (args, ref) = _linear(dev, 4096, n, 1024, 470, dtype)
+    x = _cast(oracle.synth_x(batch, n, 79), dtype).to(dev)
+    good = ops.gemv_group_forward(x, [args], one_launch=True)[0].clone()
+    torch.cuda.synchronize()
+    assert ops.gemv_group_status(dev) == 0
+    print("one-launch group with a wait of one poll", flush=True)
+    assert lib.nq_gemv_group_set_spin_limit(1) == 0
+    try:
+        ops.gemv_group_forward(x, [args], one_launch=True)
+        torch.cuda.synchronize()
+        assert ops.gemv_group_status(dev) == 1                          # reported ...
+        assert ops.gemv_group_status(dev) == 0                          # ... once
+    finally:
+        assert lib.nq_gemv_group_set_spin_limit(0) == 0
+    again = ops.gemv_group_forward(x, [args], one_launch=True)[0]
+    torch.cuda.synchronize()
+    assert ops.gemv_group_status(dev) == 0
+    assert torch.equal(again, good)
+    assert oracle.max_rel_err(again.float().cpu().numpy(), ref(x.float().cpu().numpy())) < TOL[dtype]
+
+
 def test_decode_group_of_modules(dev):
     dtype = torch.float16
     rng = np.random.default_rng(3)
