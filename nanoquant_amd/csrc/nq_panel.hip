@@ -108,9 +108,11 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
         // Fetching ahead: when this workgroup's range ends inside a panel that BEGINS in it and ends in the next
         // workgroup (a short k range cut once), that workgroup's partial tile is usually there long before this one
         // gets to the panel.  Its flag is looked at one unit ahead and, if set, the sixteen loads of the tile are issued
-        // in front of the last unit's MFMAs instead of behind them.  ahead_slot < 0: not that case.
+        // in front of the last unit's MFMAs instead of behind them.  ahead_slot < 0: not that case.  Only for short
+        // ranges: the compiler carries the registers of `ahead` through two copies per unit (about 370 cycles), which a
+        // range of more than eight units pays more for than the loads hidden once are worth.
         int ahead_slot = -1;
-        if (u_end - u >= 2) {
+        if (u_end - u >= 2 && u_end - u <= 8) {
             const int lu = u_end - 1;
             int lp = 0;
 #pragma unroll
