@@ -1,4 +1,4 @@
-// Prefill at about 128 tokens: one persistent launch per GEMM stage of a group of linears.
+// Prefill at about 128 to 768 tokens: one persistent launch per GEMM stage of a group of linears.
 //
 //   C[t, j] = s_out[j] * sum_k (x[t, k] * s_in[k]) * sgn(W[j, k])       (same function as nq_gemm.hip)
 //
@@ -7,36 +7,41 @@
 // stripes that share an output tile).  At 128 tokens a whole decoder layer is 20 us of MFMA time, so what counts is
 // how much every byte staged and every sign word decoded is reused, and that no compute unit waits for another:
 //
-//  * A workgroup (8 wavefronts, one per compute unit) works on a PANEL of 128 tokens x 256 rows.  The activation
-//    slab [128 tokens][256 k] is staged once in LDS for all eight wavefronts (64 KiB of L2 traffic per 16.8 MFLOP;
-//    the few-token tiles of nq_gemm.hip stage 16 KiB per 2.1 MFLOP).  Two slabs in LDS: one barrier per k step.
+//  * A workgroup (4 wavefronts, two workgroups per compute unit) works on a PANEL of 64 tokens x 256 rows.  The
+//    activation slab [64 tokens][256 k] is staged once in LDS for all four wavefronts (32 KiB of L2 traffic per
+//    8.4 MFLOP; the few-token tiles of nq_gemm.hip stage 16 KiB per 2.1 MFLOP).  Two slabs in LDS: one barrier per
+//    k step.  Two workgroups share a compute unit so that one has MFMAs to issue while the other hands over a
+//    partial tile or stores a panel, and so that token counts are covered in blocks of 64.
 //  * A wavefront holds 64 tokens x 64 rows (four 32x32 accumulators): every sign fragment decoded in registers
 //    feeds two MFMAs and every activation fragment read from LDS feeds two (4 lane operations and half an LDS read
 //    per MFMA).
 //  * Units of work are (panel, k tile of 256); all units of the launch are numbered in one sequence and workgroup w
-//    takes the units [w U / G, (w + 1) U / G): every compute unit gets the same number of MFMAs whatever the shapes
-//    (stream-k).  A panel whose k range is cut by such a boundary is finished by the workgroup that holds its first
-//    k tile (the owner): the others write their partial 128 x 256 fp32 tile to a workspace slot and raise a flag, the
-//    owner adds the partial tiles to its own and stores.  Stores and loads of partial tiles are device-coherent; a
-//    flag is the number of the launch (derived from a counter of workgroup exits kept in the workspace, so nothing
-//    has to be cleared between launches or graph replays); waits are bounded and an expiry is reported in the
-//    workspace's status word.  A contributor never waits, and an owner only waits for workgroups with higher
-//    numbers, which the hardware starts in order: no cycle of waits can form.
+//    takes the units [w U / G, (w + 1) U / G): every workgroup gets the same number of MFMAs whatever the shapes
+//    (stream-k).  A panel whose k range is cut by such boundaries is finished together by the workgroups whose
+//    ranges end inside it: each writes its partial 64 x 256 fp32 tile to a workspace slot and raises a flag, and
+//    each adds the others' copies of its share of the output tiles and stores them; the workgroup that holds the
+//    panel's last unit only contributes.  Stores and loads of partial tiles are device-coherent; a flag is the
+//    number of the launch (derived from a counter of workgroup exits kept in the workspace, so nothing has to be
+//    cleared between launches or graph replays); waits are bounded and an expiry is reported in the workspace's
+//    status word.  A workgroup raises its own flags before it waits for anybody's, and the hardware starts
+//    workgroups in the order of their ids with all of them resident: no cycle of waits can form.
 #include "nq_common.h"
 #include "nq_kernels.h"
 #include "nq_mfma.h"
 
 namespace nq {
 
-constexpr int kPanelThreads = 512;
-constexpr int kPanelTok = 128;                              // tokens of a panel
+constexpr int kPanelThreads = 256;
+constexpr int kPanelWaves = kPanelThreads / 64;
+constexpr int kPanelTok = 64 * (kPanelWaves / 4);           // tokens of a panel: 64 per four wavefronts
 constexpr int kPanelRows = 256;                             // rows of a panel
-constexpr int kPanelBufHalves = kPanelTok * kTileK + kTileK;   // one slab [128 tokens][256 k] and its 256 input scales
+constexpr int kPanelBufHalves = kPanelTok * kTileK + kTileK;   // one slab [tokens][256 k] and its 256 input scales
 constexpr int kPanelStagePitch = 40;                        // 16-bit elements per token row of an epilogue staging tile
 constexpr int kPanelStageHalves = 32 * kPanelStagePitch;    // per wavefront: one 32 x 32 output tile on its way out
-constexpr size_t kPanelLdsBytes = (2 * (size_t)kPanelBufHalves + 8 * (size_t)kPanelStageHalves) * sizeof(uint16_t);
+constexpr size_t kPanelLdsBytes = (2 * (size_t)kPanelBufHalves + kPanelWaves * (size_t)kPanelStageHalves) * sizeof(uint16_t);
 constexpr int kPanelMax = 16;                               // problems per launch
-constexpr int kPanelSlotFloats = kPanelTok * kPanelRows;    // one partial tile: 128 KiB
+constexpr int kPanelPerCu = 2;                              // workgroups per compute unit: one computes while the other hands over
+constexpr int kPanelSlotFloats = kPanelTok * kPanelRows;    // one partial tile: 64 KiB
 constexpr int kPanelFlagStride = 16;                        // uint32 per flag (64 bytes: one flag per cache line)
 constexpr size_t kPanelHeadBytes = 256;                     // exit counter (u64 at 0), status word (u32 at 64)
 
@@ -69,7 +74,8 @@ struct SlabFetch {
 };
 
 template <int DT, bool SCALED>
-__global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) {
+// (second argument: wavefronts per SIMD, so that kPanelPerCu workgroups of four wavefronts fit a compute unit)
+__global__ __launch_bounds__(kPanelThreads, kPanelPerCu * kPanelWaves / 4) void gemm_panel_kernel(PanelArgs g) {
     using E = Elem<DT>;
     extern __shared__ __attribute__((aligned(16))) uint16_t panel_lds[];
     __shared__ unsigned s_gen;
@@ -158,7 +164,7 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
             f.voff = live ? (uint32_t)(ftb * kPanelTok + tk0) * row_bytes + (uint32_t)fkt * (kTileK * 2u) +
                                 (uint32_t)(((lane & 31) ^ (tk0 & 15)) * 16)
                           : 0xFFFFFFF0u;
-            f.pass_bytes = 16u * row_bytes;
+            f.pass_bytes = (uint32_t)(2 * kPanelWaves) * row_bytes;
             f.base = dst + wave * (2 * kTileK);
             if constexpr (SCALED) {
                 if (tid < 32 && live) {
@@ -169,10 +175,13 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
             }
             return f;
         };
-        // pass ps (0..7) of a slab: the two token rows 16 ps + 2 w, + 1 of wavefront w
+        // pass ps (0..7) of a slab: the two token rows 2 W ps + 2 w, + 1 of wavefront w (W wavefronts).  With four
+        // wavefronts a pass is 8 tokens, so bit 3 of the token, which is part of the chunk permutation, alternates
+        // with the pass: odd passes take the source chunk with bit 3 flipped (128 bytes further or nearer).
         auto slab_fetch_pass = [&](const SlabFetch& f, int ps) {
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(f.rs, (__attribute__((address_space(3))) void*)(f.base + ps * (16 * kTileK)), 16, f.voff,
-                                                     (uint32_t)ps * f.pass_bytes, 0, kGemmCacheDefault);
+            const uint32_t voff = (2 * kPanelWaves * ps) & 8 ? f.voff ^ 128u : f.voff;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(f.rs, (__attribute__((address_space(3))) void*)(f.base + ps * (2 * kPanelWaves * kTileK)), 16,
+                                                     voff, (uint32_t)ps * f.pass_bytes, 0, kGemmCacheDefault);
         };
         auto fetch_w = [&](int fp, int frb, int fkt, bool live) {
             const PanelProblem& P = g.p[fp];
@@ -518,6 +527,8 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel_kernel(PanelArgs g) 
 }
 
 // ---- host side --------------------------------------------------------------------------------
+// Workgroups of a launch: kPanelPerCu per compute unit, all resident at once (checked against the occupancy of the
+// kernel before the first launch on a device).
 static int panel_grid() {
     static PerDeviceFlag known;
     static int cus[64];
@@ -525,6 +536,7 @@ static int panel_grid() {
     if (dev >= 0 && dev < 64 && known.test(dev)) return cus[dev];
     int n = 0;
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev < 0 ? 0 : dev) != hipSuccess || n <= 0) return 0;
+    n *= kPanelPerCu;
     if (dev >= 0 && dev < 64) { cus[dev] = n; known.set(dev); }
     return n;
 }
@@ -539,12 +551,12 @@ size_t panel_workspace_bytes() {
 int panel_max_tokens() { return kPanelTok; }
 
 // Whether one stage of a group is better off as a panel launch than on the tiles of nq_gemm.hip (measured on
-// Llama-2-7B layers, per stage, 64 .. 4096 tokens).  Every compute unit must get a few k steps (otherwise panels are cut
+// Llama-2-7B layers, per stage, 64 .. 4096 tokens).  Every workgroup must get a few k steps (otherwise panels are cut
 // into many pieces and the hand-over of partial tiles costs more than the shared slabs save); the longest k range
-// must not be shared by more than about four workgroups (the first stage of a 128-token layer, whose 43-tile down
-// projection is cut eight ways, is faster on the few-token tiles); token counts that fill their 128-token blocks
-// badly waste MFMAs, which only a stage with a long k makes up for (its block tiles need a k split and a finish
-// launch); and from about 1024 tokens on the block tiles are ahead.
+// must not be shared by too many workgroups (the first stage of a 128-token layer, whose 43-tile down projection is
+// cut eight ways, is faster on the few-token tiles); token counts that fill their 64-token blocks badly waste MFMAs,
+// which only a stage with a long k makes up for (its block tiles need a k split and a finish launch); and from
+// about 1024 tokens on the block tiles are level.
 bool panel_applies(int count, int T, const int* K, const int* R) {
     const int G = panel_grid();
     if (G <= 0 || count < 1 || count > kPanelMax || T < 1 || T > 768) return false;
@@ -558,9 +570,11 @@ bool panel_applies(int count, int T, const int* K, const int* R) {
     }
     const double per_wg = (double)units / G;
     if (per_wg < 3.0) return false;
-    if (longest > 4.0 * per_wg) return false;
+    // up to two token blocks the few-token tiles are the alternative, and a strong one; beyond, panels win more easily
+    const bool few = T <= 2 * kPanelTok;
+    if (longest > (few ? 4.0 : 8.0) * per_wg) return false;
     const double fill = (double)T / (tblocks * kPanelTok);
-    return fill >= 0.85 || longest > 16;
+    return fill >= (few ? 0.85 : 0.70) || longest > 16;
 }
 
 template <int DT, bool SCALED>
@@ -574,7 +588,7 @@ static hipError_t launch_panel(const PanelArgs& a, int G, hipStream_t stream) {
         int per_cu = 0;
         e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kern, kPanelThreads, kPanelLdsBytes);
         if (e != hipSuccess) return e;
-        if (per_cu < 1) return hipErrorLaunchOutOfResources;
+        if (per_cu < kPanelPerCu) return hipErrorLaunchOutOfResources;
         attr_done.set(dev);
     }
     hipLaunchKernelGGL(kern, dim3(G), dim3(kPanelThreads), kPanelLdsBytes, stream, a);
