@@ -31,9 +31,9 @@ HBM_PEAK_GBS = 8000.0
 # copy kernel of known size (profiles/gemv_stream_llama2_7b_stack_b1.md); valid for the default workload only.
 MEASURED_TRAFFIC_BYTES = 843630592
 # The same for the two launches of the 128-token grouped layer (profiles/gemm_group_llama2_7b_layer_prefill.md):
-# (18786 + 25962) KiB x 2.000 fetched + (4352 + 48583) KiB written; 38.8 MB each way of the second launch are partial
+# (18756 + 26222) KiB x 2.000 fetched + (4352 + 48686) KiB written; 38.9 MB each way of the second launch are partial
 # tiles that its workgroups hand over through device-coherent memory.
-MEASURED_PREFILL_TRAFFIC_BYTES = (18786 + 25962) * 2 * 1024 + (4352 + 48583) * 1024
+MEASURED_PREFILL_TRAFFIC_BYTES = (18756 + 26222) * 2 * 1024 + (4352 + 48686) * 1024
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 LLAMA2_7B_LAYER = (("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096),
@@ -631,7 +631,7 @@ def main():
                 result["roofline_prefill"] = {
                     "bound": "mfma", "tokens": 128,
                     "kernel": "first GEMMs of the 7 linears: gemm_kwave_group_kernel<fp16> (few-token tiles); second GEMMs: "
-                              "gemm_panel_kernel<fp16> (persistent 128-token x 256-row panels); one launch each",
+                              "gemm_panel_kernel<fp16> (persistent 64-token x 256-row panels, two workgroups per CU); one launch each",
                     "achieved": round(tf, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "flops_per_layer": int(group_flops),
                     "us_per_layer": round(us, 2), "traffic": MEASURED_PREFILL_TRAFFIC_BYTES}

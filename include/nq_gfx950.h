@@ -261,11 +261,11 @@ int nq_gemm_group_max(void);
 int nq_gemm_nanoquant_group(const nq_gemm_term* terms, int count, int tokens, int dtype, void* scratch,
                             size_t scratch_bytes, void* stream);
 
-/* The same with a workspace for the panel launches.  Around 128 tokens (96..128) a group that gives every compute
- * unit a few k steps of work runs each of its two stages as ONE persistent launch over panels of 128 tokens x 256
- * rows whose k ranges are shared out evenly over the compute units (what the reference's stream-k stripes do,
- * kernel/cuda/gemm_kernel.cu:335-400, :594-640): panels cut by a share boundary hand their partial fp32 tiles to
- * the workgroup that finishes them through `panel_ws`.
+/* The same with a workspace for the panel launches.  From about 100 to 768 tokens a group that gives every
+ * workgroup a few k steps of work runs a stage as ONE persistent launch (two workgroups per compute unit) over panels
+ * of 64 tokens x 256 rows whose k ranges are shared out evenly over the workgroups (what the reference's stream-k
+ * stripes do, kernel/cuda/gemm_kernel.cu:335-400, :594-640): panels cut by a share boundary are finished together by
+ * the workgroups that end inside them, which exchange partial fp32 tiles through `panel_ws`.
  *   panel_ws: nq_gemm_panel_workspace_bytes() bytes of device memory, 256-byte aligned, ZERO when first used and
  *   left to these launches from then on (it holds partial tiles, hand-over flags and a count of finished
  *   workgroups from which every launch derives its own flag value, so nothing is cleared between launches or graph

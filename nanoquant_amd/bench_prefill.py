@@ -42,6 +42,9 @@ def run(argv=None) -> List[Dict[str, Any]]:
     ap.add_argument("--panel", default="auto", choices=("auto", "always", "never"),
                     help="grouped leg: persistent panel launches where the library's policy picks them (auto), for every "
                          "stage (always), or the launches without a workspace only (never)")
+    ap.add_argument("--constant_data", action="store_true",
+                    help="activations 0 and all signs +1 instead of random data: the same instructions with nothing "
+                         "toggling in the multipliers, to show how much of the time is the part's response to switching power")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args(argv)
 
@@ -66,6 +69,8 @@ def run(argv=None) -> List[Dict[str, Any]]:
         r = prefill_rank(m, n, args.bpw)
         v = torch.randint(0, 2, (n, r), device=dev, generator=gen, dtype=torch.int8) * 2 - 1
         u = torch.randint(0, 2, (r, m), device=dev, generator=gen, dtype=torch.int8) * 2 - 1
+        if args.constant_data:
+            v, u = torch.ones_like(v), torch.ones_like(u)
         sc = lambda k: (torch.randn(k, device=dev, generator=gen).abs() * 0.02 + 1e-3).to(dtype)
         packed_by_shape[(m, n)] = (packing.marlin_nanoquant_packer(v, u, sc(n), sc(r), sc(m)), r)
         del v, u
@@ -103,10 +108,12 @@ def run(argv=None) -> List[Dict[str, Any]]:
     rows = []
     for tokens in parse_int_list(args.tokens, "tokens"):
         xs_by_n = {n: torch.randn(tokens, n, device=dev, generator=gen).to(dtype) for n in {n for (_, _, n) in shapes}}
+        if args.constant_data:
+            xs_by_n = {n: torch.zeros_like(x) for n, x in xs_by_n.items()}
         xs = [xs_by_n[n] for (_, _, n) in shapes]
         flops = sum(2.0 * tokens * packed_by_shape[(m, n)][1] * (m + n) for (_, m, n) in shapes)
         row: Dict[str, Any] = {"model_shape": args.model_shape, "tokens": tokens, "dtype": args.dtype, "panel": args.panel,
-                               "linears": len(shapes), "GFLOP_per_layer": round(flops / 1e9, 2)}
+                               "data": "constant" if args.constant_data else "random", "linears": len(shapes), "GFLOP_per_layer": round(flops / 1e9, 2)}
         legs = []
         if not args.no_single:
             legs.append(("one_by_one", lambda: [op(x, *t) for x, t in zip(xs, terms)]))
