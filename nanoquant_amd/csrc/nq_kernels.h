@@ -93,10 +93,9 @@ hipError_t gemm_onebit_group(int dtype, int count, const void* const* x, const u
                              const void* const* s_in, const void* const* s_out, const void* const* bias, void* const* y,
                              int T, const int* K, const int* R, hipStream_t stream);
 
-// nq_panel.hip: the same GEMMs at about 128 tokens as one persistent launch over 128-token x 256-row panels
+// nq_panel.hip: the same GEMMs at about 128 to 768 tokens as one persistent launch over 64-token x 256-row panels
 // (see the file header).  workspace: panel_workspace_bytes() bytes, zero when first used.
 size_t panel_workspace_bytes();
-int panel_max_tokens();
 bool panel_applies(int count, int T, const int* K, const int* R);
 hipError_t gemm_panel_group(int dtype, int count, const void* const* x, const uint32_t* const* tiles,
                             const void* const* s_in, const void* const* s_out, const void* const* bias, void* const* y,

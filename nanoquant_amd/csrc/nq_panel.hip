@@ -548,8 +548,6 @@ size_t panel_workspace_bytes() {
     return kPanelHeadBytes + flags + (size_t)2 * G * kPanelSlotFloats * sizeof(float);
 }
 
-int panel_max_tokens() { return kPanelTok; }
-
 // Whether one stage of a group is better off as a panel launch than on the tiles of nq_gemm.hip (measured on
 // Llama-2-7B layers, per stage, 64 .. 4096 tokens).  Every workgroup must get a few k steps (otherwise panels are cut
 // into many pieces and the hand-over of partial tiles costs more than the shared slabs save); the longest k range
