@@ -273,6 +273,9 @@ int nq_gemm_nanoquant_group(const nq_gemm_term* terms, int count, int tokens, in
  *   panel_mode: NQ_PANEL_AUTO picks per stage (other token counts and small groups take the launches of
  *   nq_gemm_nanoquant_group), NQ_PANEL_ALWAYS forces the panel launch for any token count, NQ_PANEL_NEVER (or
  *   panel_ws NULL) never takes it.
+ * A panel launch keeps two workgroups per compute unit resident and its workgroups wait for each other's partial
+ * tiles: it may share the GPU with other kernels (its waits then last until those free their compute units), but a
+ * wait that outlasts its bound (2^20 polls, about a second) invalidates the launch's outputs.
  * The waits of a finishing workgroup are bounded; nq_gemm_panel_status copies the workspace's status word back
  * (synchronises) and clears it: 0 ok, 1 = a wait expired in some launch since the last call (that launch's outputs
  * are invalid; the workspace stays usable). */

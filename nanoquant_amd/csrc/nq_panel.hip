@@ -572,7 +572,7 @@ bool panel_applies(int count, int T, const int* K, const int* R) {
     const bool few = T <= 2 * kPanelTok;
     if (longest > (few ? 4.0 : 8.0) * per_wg) return false;
     const double fill = (double)T / (tblocks * kPanelTok);
-    return fill >= (few ? 0.85 : 0.70) || longest > 16;
+    return fill >= (few ? 0.78 : 0.70) || longest > 16;
 }
 
 template <int DT, bool SCALED>
