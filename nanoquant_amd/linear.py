@@ -462,8 +462,19 @@ def decode_group(modules: Sequence, x) -> list:
     for mod in mods:
         b = mod.bias if (mod.kernel_path_bias and mod.bias is not None) else None
         biases.append(None if b is None else (b if b.dtype == mod.dtype else b.to(mod.dtype)))
-    outs = ops.gemv_group_forward(flat, [(m.scale_pre, m.V_int8, m.scale_mid, m.U_int8, m.scale_post) for m in mods],
-                                  biases if any(b is not None for b in biases) else None)
+    # the operands are checked once per set of modules and tensors: a prepared group is kept while every operand is
+    # still the tensor it was built on
+    operands = [(m.scale_pre, m.V_int8, m.scale_mid, m.U_int8, m.scale_post) for m in mods]
+    cache = mods[0].__dict__.setdefault("_decode_groups", {})      # lives and dies with the first module of the group
+    key = tuple(id(m) for m in mods)
+    hit = cache.get(key)
+    if hit is None or len(hit[1]) != len(operands) or any(a is not b for old, new in zip(hit[1], operands) for a, b in zip(old, new)) \
+            or any(a is not b for a, b in zip(hit[2], biases)):
+        if len(cache) >= 16:
+            cache.clear()
+        hit = (ops.GemvGroup(operands, biases if any(b is not None for b in biases) else None), operands, list(biases))
+        cache[key] = hit
+    outs = hit[0](flat)
     for i, t in enumerate(xs_in):
         y = outs[i]
         if t.ndim == 3:

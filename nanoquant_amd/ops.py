@@ -403,6 +403,69 @@ def gemv_group_forward(xs, linears, biases=None, outs=None, one_launch=False):
     return outs
 
 
+class GemvGroup:
+    """A group of independent decode linears checked once, for callers that launch it again and again from Python
+    (`gemv_group_forward` checks every operand on every call, which costs more host time than the launches take on
+    the GPU).  `linears` and `biases` as `gemv_group_forward` takes them; the tensors are kept alive and must not be
+    resized.  `group(xs, outs=None, one_launch=False)` checks the inputs only."""
+
+    def __init__(self, linears, biases=None):
+        from .runlist import NqLinear
+        self.linears = [tuple(lin) for lin in linears]
+        if not self.linears:
+            raise ValueError("at least one linear")
+        self.biases = [None] * len(self.linears) if biases is None else list(biases)
+        if len(self.biases) != len(self.linears):
+            raise ValueError("one bias entry per linear")
+        sg0 = self.linears[0][0]
+        self.dtype, self.device = sg0.dtype, sg0.device
+        self.dims = []
+        for (sg, ub, sl, vb, sh), b in zip(self.linears, self.biases):
+            n = sg.numel()
+            probe = torch.empty((0, n), dtype=self.dtype, device=self.device)     # the operand checks of the op, without an input yet
+            self.dims.append(_check_gemv_args(probe, sg, ub, sl, vb, sh))
+            _check_bias(b, self.dims[-1][2], probe)
+        self._arr = (NqLinear * len(self.linears))()
+        p = lambda t: None if t is None else t.data_ptr()
+        for i, ((sg, ub, sl, vb, sh), b, (n, r, m)) in enumerate(zip(self.linears, self.biases, self.dims)):
+            self._arr[i] = NqLinear(None, p(sg), p(ub), p(sl), p(vb), p(sh), None, None, None, n, r, m, -1, -1, 0, p(b), 0)
+        self._dtype_id = _dtype_id(sg0)
+
+    def __call__(self, xs, outs=None, one_launch=False):
+        count = len(self.linears)
+        xs = [xs] * count if isinstance(xs, torch.Tensor) else list(xs)
+        if len(xs) != count:
+            raise ValueError("one input per linear")
+        x0 = xs[0]
+        batch = x0.numel() // self.dims[0][0] if x0.dim() >= 1 and self.dims[0][0] else 0
+        total, offsets = 0, []
+        for x, (n, r, m) in zip(xs, self.dims):
+            if not x.is_cuda or x.dtype != self.dtype or x.device != self.device or not x.is_contiguous():
+                raise RuntimeError("inputs of a group must be contiguous tensors of the group's dtype on its device")
+            if x.dim() < 1 or x.size(-1) != n or x.numel() != batch * n:
+                raise RuntimeError(f"input must be [{batch}, {n}], got {list(x.shape)}")
+            offsets.append(total)
+            total += (batch * max(r, 1) + 63) // 64 * 64
+        if outs is None:
+            outs = [torch.empty((batch, m), dtype=self.dtype, device=self.device) for _, _, m in self.dims]
+        else:
+            outs = list(outs)
+            for y, (_, _, m) in zip(outs, self.dims):
+                _check_dev_cont(y, "out", self.dtype, _FLOAT_WHAT[self.dtype])
+                if tuple(y.shape) != (batch, m):
+                    raise RuntimeError(f"out must be [{batch}, {m}], got {list(y.shape)}")
+        if batch == 0:
+            return outs
+        h = torch.empty(total, dtype=torch.float32, device=self.device)
+        hp, arr = h.data_ptr(), self._arr
+        for i in range(count):
+            arr[i].x, arr[i].h, arr[i].y = xs[i].data_ptr(), hp + 4 * offsets[i], outs[i].data_ptr()
+        with _on_device(self.device):
+            _lib.check(_lib.lib().nq_gemv_forward_group(arr, count, batch, self._dtype_id, 1 if one_launch else 0,
+                                                         _stream(self.device)))
+        return outs
+
+
 def gemv_group_status(device=None) -> int:
     """Synchronises the current stream.  0, or 1 when a launch of `gemv_group_forward(one_launch=True)` on this device
     ran into its bounded wait since the last call: the outputs of that launch are invalid.  Clears the flag."""

@@ -170,6 +170,38 @@ def test_decode_group_of_modules(dev):
             assert y.shape == want.shape and torch.equal(y, want)
     with pytest.raises(ValueError):
         nanoquant_amd.decode_group(mods, [x])
+    # the prepared group behind decode_group follows the modules: new factors for one of them are picked up
+    assert len(mods[0].__dict__["_decode_groups"]) == 1
+    vt, u, s_in, s_mid, s_out = oracle.synth_term(256, 512, 64, 99)
+    fresh = nanoquant_amd.NanoQuantLinear.from_factors(torch.from_numpy(vt).float(), torch.from_numpy(u).float(), torch.from_numpy(s_in),
+                                                       torch.from_numpy(s_mid), torch.from_numpy(s_out), dtype=torch.float32).to(dev)
+    fresh._prepare_kernel("gemv", dtype)
+    mods[2].V_int8, mods[2].U_int8 = fresh.V_int8, fresh.U_int8
+    mods[2].scale_pre, mods[2].scale_mid, mods[2].scale_post = fresh.scale_pre, fresh.scale_mid, fresh.scale_post
+    x = torch.from_numpy(oracle.synth_x(2, 512, 10)).to(dev, dtype)
+    ys = nanoquant_amd.decode_group(mods, x)
+    torch.cuda.synchronize()
+    assert torch.equal(ys[2], fresh(x)) and torch.equal(ys[0], mods[0](x))
+
+
+def test_prepared_group_checks_once_and_matches(dev):
+    dtype = torch.float16
+    lins = [_linear(dev, m, 1024, r, 480 + i, dtype) for i, (m, r) in enumerate([(512, 256), (128, 96)])]
+    bias = _cast(np.linspace(-1, 1, 512), dtype).to(dev)
+    group = ops.GemvGroup([a for a, _ in lins], [bias, None])
+    for batch in (1, 3, 8):
+        x = _cast(oracle.synth_x(batch, 1024, 490 + batch), dtype).to(dev)
+        ys = group(x)
+        want = ops.gemv_group_forward(x, [a for a, _ in lins], [bias, None])
+        torch.cuda.synchronize()
+        for y, w in zip(ys, want):
+            assert torch.equal(y, w)
+    with pytest.raises(RuntimeError):
+        group(torch.zeros(1, 1000, dtype=dtype, device=dev))            # wrong width
+    with pytest.raises(RuntimeError):
+        group(torch.zeros(1, 1024, dtype=torch.float32, device=dev))     # wrong type
+    with pytest.raises(RuntimeError):
+        ops.GemvGroup([(lins[0][0][0], lins[0][0][1], lins[0][0][2], lins[1][0][3], lins[0][0][4])])   # factors that do not fit
 
 
 def test_group_entry_point_argument_checks(dev):
