@@ -437,8 +437,9 @@ def decode_group(modules: Sequence, x) -> list:
     modules sharing launches (`ops.gemv_group_forward`; pieces of 1, 2 and 4 rows, two launches per 8 modules): what a
     decoder issues per layer at decode time is then eight launches, two each for {q,k,v}, {o}, {gate,up}, {down}, with
     its attention, norms and activations between them, instead of the reference's two launches per module
-    (linear.py:121-130).  Nothing is prepared or kept: any activations on every call, no requirement on what else the
-    GPU runs.  `x` is one tensor for all modules or a list of one tensor per module, 2-D or 3-D as `forward` takes it."""
+    (linear.py:121-130).  No run list is built: any activations on every call, no requirement on what else the GPU
+    runs; only the checked operand table of the group (`ops.GemvGroup`) is kept with the first module, and rebuilt
+    when a module's tensors are replaced.  `x` is one tensor for all modules or a list of one tensor per module, 2-D or 3-D as `forward` takes it."""
     mods = list(modules)
     if not mods:
         return []
