@@ -94,7 +94,9 @@ int nq_gemv_mixture(const void* x, const void* const* s_in, const uint32_t* cons
  * [batch, r] intermediate.  x_from >= 0 says that x is the y of that earlier entry of the list (the
  * kernel then orders the two); y_from >= 0 says that `addend` is the fp32 y of that earlier entry.
  * With out_f32 the result y is stored as fp32 (used for sums over terms); addend (fp32 [batch, m])
- * is added before the store.
+ * is added before the store.  Where the adding entry's own intermediate is ready in time, the builder cuts
+ * its second stage into the same rows on the same workgroups as the entry it adds onto, each slice right
+ * behind the one that writes its addend, and the two wait for nothing between them.
  *
  * nq_runlist_build writes the stage table into `workspace` (device memory of at least
  * nq_runlist_workspace_bytes(linears, nlinears) bytes, 256-byte aligned) -- it copies from host memory, so it

@@ -344,7 +344,19 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         b.vec_bits = (b.words % 4 == 0) && al16(l.u_bits);
         b.vec_in = al16(l.h) && ((size_t)l.r * 4) % 16 == 0;
         b.phase = a.phase + 1;
-        if (b.dep2 >= 0 && table[b.dep2].phase + 1 > b.phase) b.phase = table[b.dep2].phase + 1;
+        if (b.dep2 >= 0) {
+            // A term that adds onto the result of an earlier one: where its own input is ready in time, it runs in the
+            // phase of that stage, cut into the same rows on the same workgroups, each slice right behind the one that
+            // writes its addend -- nothing to wait for between the two.  Otherwise it runs a phase later and waits
+            // for the whole earlier stage.
+            const nq::RunStage& head = table[b.dep2];
+            if (a.phase + 1 <= head.phase && (head.tiled != 0) == (l.tiled != 0)) {
+                b.phase = head.phase;
+                b.addend_local = 1;
+            } else if (head.phase + 1 > b.phase) {
+                b.phase = head.phase + 1;
+            }
+        }
         // the kernel addresses the packed words of a stage with 32-bit byte offsets
         const size_t bytes_a = l.tiled ? nq::tiled_word_count(a.rows, a.words) * 4 : (size_t)a.rows * a.words * 4;
         const size_t bytes_b = l.tiled ? nq::tiled_word_count(b.rows, b.words) * 4 : (size_t)b.rows * b.words * 4;
@@ -386,8 +398,22 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
     int nwg = nq::stream_capacity(dtype, batch, max_units, alt);
     if (nwg <= 0) return NQ_ERR_HIP;
     if (nwg > kMaxResidentWorkgroups) nwg = kMaxResidentWorkgroups;
+    // A family: a stage and the stages that add onto its rows on the same workgroups (addend_local), in list order.
+    // The phases are cut family by family; a family costs the sum of its members.
+    std::vector<int> root((size_t)nstages);
+    std::vector<std::vector<int>> family((size_t)nstages);
+    for (int s = 0; s < nstages; ++s) {
+        root[(size_t)s] = table[(size_t)s].addend_local ? root[(size_t)table[(size_t)s].dep2] : s;
+        family[(size_t)root[(size_t)s]].push_back(s);
+    }
     std::vector<std::vector<int>> by_phase((size_t)nphases);
-    for (int s = 0; s < nstages; ++s) by_phase[table[s].phase].push_back(s);
+    for (int s = 0; s < nstages; ++s)
+        if (root[(size_t)s] == s) by_phase[table[s].phase].push_back(s);
+    auto family_units = [&](int head) {
+        long long u = 0;
+        for (int s : family[(size_t)head]) u += table[(size_t)s].units;
+        return u;
+    };
     // slices per phase and workgroup, in the order in which the workgroup works them off
     std::vector<std::vector<std::vector<nq::RunSegment>>> slice((size_t)nphases);
     for (int ph = 0; ph < nphases; ++ph) {
@@ -395,17 +421,8 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         const std::vector<int>& ids = by_phase[ph];
         std::vector<long long> prefix(ids.size() + 1, 0);
         for (size_t k = 0; k < ids.size(); ++k)
-            prefix[k + 1] = prefix[k] + (long long)table[ids[k]].rows * table[ids[k]].units;
+            prefix[k + 1] = prefix[k] + (long long)table[ids[k]].rows * family_units(ids[k]);
         const long long total = prefix.back();
-        // cut point -> (stage position, row): the same mapping is used for a slice's end and the next
-        // slice's begin, so the slices tile every stage exactly
-        auto locate = [&](long long c, size_t& k, int& row) {
-            k = 0;
-            while (k + 1 < ids.size() && prefix[k + 1] <= c) ++k;
-            if (c >= total) { k = ids.size() - 1; row = table[ids[k]].rows; return; }
-            row = (int)((c - prefix[k]) / table[ids[k]].units);
-            if (table[ids[k]].tiled) row &= ~(granule - 1);   // tile order: cut between the row groups of a wave-load
-        };
         if (ids.size() * 2 <= (size_t)nwg) {
             // Few stages, many workgroups: give every stage whole workgroups, so that no workgroup stages
             // two input vectors in one phase.  A slice costs units * rows + fixed: staging the input vector takes
@@ -418,16 +435,18 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
             const double overhead_rows = batch >= 16 ? 64.0 : wide ? 48.0 : 12.0;
             const double pass_cost = wide ? 700.0 : 0.0;
             const int chunk_cap = std::max(1, nq::stream_chunk_cap(dtype, batch, max_units, alt));
-            std::vector<double> fixed(ids.size(), 0.0);
-            for (size_t k = 0; k < ids.size(); ++k) {
-                const int u = table[ids[k]].units;
-                fixed[k] = u * overhead_rows + ((u + chunk_cap - 1) / chunk_cap - 1) * pass_cost;
-            }
+            std::vector<double> fixed(ids.size(), 0.0), width(ids.size(), 0.0);
+            for (size_t k = 0; k < ids.size(); ++k)
+                for (int s : family[(size_t)ids[k]]) {
+                    const int u = table[(size_t)s].units;
+                    fixed[k] += u * overhead_rows + ((u + chunk_cap - 1) / chunk_cap - 1) * pass_cost;
+                    width[k] += u;
+                }
             std::vector<int> share(ids.size(), 1);
             auto needed = [&](double t) {       // workgroups needed for every slice to cost at most t
                 long long sum = 0;
                 for (size_t k = 0; k < ids.size(); ++k) {
-                    const double u = table[ids[k]].units, r = table[ids[k]].rows;
+                    const double u = width[k], r = table[ids[k]].rows;
                     const double room = t - fixed[k];
                     if (room <= 0) return (long long)nwg + 1;
                     long long n = (long long)((u * r + room - 1e-9) / room);
@@ -439,7 +458,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
             };
             double lo = 0, hi = 0;
             for (size_t k = 0; k < ids.size(); ++k) {
-                const double t1 = (double)table[ids[k]].units * table[ids[k]].rows + fixed[k];
+                const double t1 = width[k] * table[ids[k]].rows + fixed[k];
                 if (t1 > hi) hi = t1;
             }
             for (int iter = 0; iter < 60; ++iter) {
@@ -448,7 +467,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
             }
             int used = 0;
             for (size_t k = 0; k < ids.size(); ++k) {
-                const double u = table[ids[k]].units, r = table[ids[k]].rows;
+                const double u = width[k], r = table[ids[k]].rows;
                 const double room = hi - fixed[k];
                 long long n = room > 0 ? (long long)((u * r + room - 1e-9) / room) : 1;
                 if (n < 1) n = 1;
@@ -462,7 +481,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
                 double worst = -1;
                 for (size_t k = 0; k < ids.size(); ++k) {
                     if (share[k] >= table[ids[k]].rows) continue;
-                    const double t = table[ids[k]].units * ((double)table[ids[k]].rows / share[k]) + fixed[k];
+                    const double t = width[k] * ((double)table[ids[k]].rows / share[k]) + fixed[k];
                     if (t > worst) { worst = t; best = k; }
                 }
                 if (best == ids.size()) break;
@@ -482,10 +501,11 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
                         rb = (int)std::min<long long>(rows, (long long)granule * ((long long)ntile * j / share[k]));
                         re = (int)std::min<long long>(rows, (long long)granule * ((long long)ntile * (j + 1) / share[k]));
                     }
-                    if (re > rb) {
-                        slice[ph][(size_t)w].push_back(nq::RunSegment{ids[k], rb, re, 0});
-                        table[ids[k]].seg_count += 1;
-                    }
+                    if (re > rb)
+                        for (int s : family[(size_t)ids[k]]) {
+                            slice[ph][(size_t)w].push_back(nq::RunSegment{s, rb, re, 0});
+                            table[(size_t)s].seg_count += 1;
+                        }
                 }
             }
             continue;
@@ -501,7 +521,7 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
         {
             // (the variant whose wavefronts own row pairs starts every slice without fetches in flight, so a slice
             // costs it more to start: 16000, and 10000 at batch 1, the best of sweeps on the Llama-2-7B stack)
-            const long long fixed = own ? (batch == 1 ? 10000 : 16000) : wide ? 2200 : batch == 1 ? 8800 : batch == 2 ? 6600 : 4400;
+            const long long fixed_one = own ? (batch == 1 ? 10000 : 16000) : wide ? 2200 : batch == 1 ? 8800 : batch == 2 ? 6600 : 4400;
             auto gran = [&](size_t k) { return table[ids[k]].tiled ? granule : 1; };
             // Batch 8 and 16: an input too long to be staged at once is staged again, chunk by chunk, for every 256 rows
             // of a slice (three barriers and a round trip to memory per chunk): charged as 10 more units per chunk and
@@ -519,7 +539,10 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
                 int row = 0;
                 while (k < ids.size()) {
                     const nq::RunStage& stg = table[ids[k]];
-                    const long long u = stg.units + restage(stg.units);
+                    const std::vector<int>& fam = family[(size_t)ids[k]];
+                    long long u = 0;
+                    for (int s : fam) u += table[(size_t)s].units + restage(table[(size_t)s].units);
+                    const long long fixed = fixed_one * (long long)fam.size();
                     const int left = stg.rows - row;
                     const int g = gran(k);
                     const long long least = fixed + u * std::min<long long>(left, std::max<long long>(g, fixed / (4 * u)));
@@ -532,17 +555,18 @@ int nq_runlist_build(const nq_linear* linears, int nlinears, int batch, int dtyp
                     long long fit = (budget - fixed) / u;
                     if (fit < left) fit = fit / g * g;                   // cut between the row groups of a wave-load
                     const int take = (int)std::min<long long>(left, fit);
-                    if (emit && w < nwg) {
-                        slice[ph][(size_t)w].push_back(nq::RunSegment{ids[k], row, row + take, 0});
-                        table[ids[k]].seg_count += 1;
-                    }
+                    if (emit && w < nwg)
+                        for (int s : fam) {
+                            slice[ph][(size_t)w].push_back(nq::RunSegment{s, row, row + take, 0});
+                            table[(size_t)s].seg_count += 1;
+                        }
                     budget -= fixed + u * take;
                     row += take;
                     if (row >= stg.rows) { ++k; row = 0; }
                 }
                 return w + 1;
             };
-            long long lo = total / nwg, hi = 2 * total + (long long)ids.size() * fixed + 1;   // restage() adds at most 10 to chunk_cap + 1 units
+            long long lo = total / nwg, hi = 2 * total + (long long)nstages * fixed_one + 1;   // restage() adds at most 10 to chunk_cap + 1 units
             while (lo < hi) {
                 const long long mid = lo + (hi - lo) / 2;
                 if (fill(mid, false) <= nwg) hi = mid; else lo = mid + 1;

@@ -46,7 +46,8 @@ struct RunStage {
     int tiled;              // `bits` is in the tile order of tile_words() instead of row-major
     int in_ext, out_ext;    // `in` / `out` are given with the launch instead (bound input / output of the list)
     int dep_segs, dep2_segs;  // seg_count of the stages `dep` / `dep2` (what a waiting slice compares the counter with)
-    int pad_;
+    int addend_local;       // the rows of `addend` that a slice reads were written by the slice before it on the same
+                            // workgroup (same rows of stage `dep2`): nothing to wait for
 };
 // One workgroup's share of one stage: rows [row_begin, row_end).
 struct RunSegment {

@@ -355,7 +355,7 @@ __global__ __launch_bounds__(THREADS) void gemv_stream_kernel(int nstages, const
 #pragma unroll 1
                     for (int which = 0; which < 2 && !bad; ++which) {
                         const int d = which ? st.dep2 : st.dep;
-                        if (d < 0) continue;
+                        if (d < 0 || (which && st.addend_local)) continue;
                         const unsigned long long want = (gen + 1) * (unsigned long long)(which ? st.dep2_segs : st.dep_segs);
                         while (true) {
                             unsigned long long c = 0;

@@ -554,13 +554,14 @@ def gemm_group_forward(xs, terms, biases=None, outs=None, panel="auto"):
     return outs
 
 
-def gemm_group_sum_forward(xs, term_groups, bias_groups=None):
+def gemm_group_sum_forward(xs, term_groups, bias_groups=None, panel="auto"):
     """`[sum_t marlin_nanoquant_forward(x_i, *term_groups[i][t]) for i]`: weights that are sums of several binary
     low-rank terms (mixture of ranks) on the grouped prefill launches.  All terms of all weights share the two
     launches of `gemm_group_forward`; the t-th terms of all weights write into one flat buffer per t, weights with
     more terms first, so that the sums over the terms are one in-place add per extra term index instead of one
     per weight.  `xs`: one tensor or one per weight; `bias_groups`: optional list (per weight) of lists (per term) of
-    bias tensors / None.  Returns one [tokens, m] tensor per weight (views of one buffer)."""
+    bias tensors / None; `panel` as in `gemm_group_forward`.  Returns one [tokens, m] tensor per weight (views of one
+    buffer)."""
     nw = len(term_groups)
     if nw == 0:
         return []
@@ -592,7 +593,8 @@ def gemm_group_sum_forward(xs, term_groups, bias_groups=None):
             flat_terms.append(term_groups[i][t])
             flat_bias.append(None if bias_groups is None or bias_groups[i] is None else bias_groups[i][t])
             flat_out.append(view)
-    gemm_group_forward(flat_x, flat_terms, flat_bias if any(b is not None for b in flat_bias) else None, outs=flat_out)
+    gemm_group_forward(flat_x, flat_terms, flat_bias if any(b is not None for b in flat_bias) else None, outs=flat_out,
+                       panel=panel)
     for t in range(1, depth):
         bufs[0][:sizes[t]].add_(bufs[t])
     return results

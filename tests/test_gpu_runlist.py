@@ -148,6 +148,114 @@ def test_mixture_through_addend(dev, dtype, tiled):
     assert oracle.max_rel_err(y.float().cpu().numpy(), ref) < (1e-2 if dtype == torch.bfloat16 else TIGHT)
 
 
+def _weight_of_terms(dev, rl, dtype, batch, m, n, ranks, seed, tiled, links=None, x=None, x_from=-1):
+    """Adds one weight = sum of len(ranks) terms to rl; term t adds onto the result of term links[t] (default: the one
+    before it).  Returns (index of the last term, [per-term fp64 references], x as fp64)."""
+    to = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev).to(dtype)
+    f64 = lambda t: t.float().cpu().numpy().astype(np.float64)
+    words = lambda w: packing.binary_packer(torch.from_numpy(w), "half2").to(dev)
+    order = (lambda w: packing.tile_words(w)) if tiled else (lambda w: w)
+    xt = to(oracle.synth_x(batch, n, seed)) if x is None else x
+    idx, refs = [], []
+    for t, r in enumerate(ranks):
+        vt, u, s_in, s_mid, s_out = oracle.synth_term(m, n, r, seed + 1 + t)
+        vt_p, u_p, mid_p = oracle.pad_rank(vt, u, s_mid, 32)
+        sc = (to(s_in), to(mid_p), to(s_out))
+        last = t == len(ranks) - 1
+        kw = dict(tiled=tiled, out_f32=not last)
+        if t == 0:
+            kw["x_from"] = x_from
+        else:
+            src = idx[t - 1 if links is None else links[t]]
+            kw.update(addend=rl.outputs[src], y_from=src)
+        idx.append(rl.add(xt, sc[0], order(words(vt_p)), sc[1], order(words(u_p)), sc[2], **kw))
+        refs.append(oracle.layer_forward(f64(xt), vt, u, f64(sc[0]), f64(to(s_mid)), f64(sc[2]), dtype=np.float64))
+    return idx, refs, f64(xt)
+
+
+@pytest.mark.parametrize("batch,dtype,tiled", [(1, torch.float16, True), (1, torch.float16, False), (4, torch.bfloat16, True),
+                                               (4, torch.float16, False), (16, torch.float16, True), (8, torch.bfloat16, False)])
+def test_terms_that_add_onto_the_same_rows(dev, batch, dtype, tiled):
+    # Three terms of one weight in a chain, and a weight whose third term adds onto the first one's result: all second
+    # stages share one phase, each workgroup runs the terms of its rows one behind the other.  A weight whose second
+    # term is fed by another linear of the list cannot do that (its input is ready too late) and waits for the whole
+    # first term instead.
+    rl = DecodeRunList(batch, dtype, dev)
+    ia, ra, _ = _weight_of_terms(dev, rl, dtype, batch, 1376, 1024, (320, 96, 64), 700, tiled)
+    ib, rb, _ = _weight_of_terms(dev, rl, dtype, batch, 512, 2048, (256, 128, 40), 710, tiled, links=[None, 0, 0])
+    ys = rl.run()
+    assert rl._plan.nphases == 2, rl._plan.nphases
+    torch.cuda.synchronize()
+    assert rl.status() == 0
+    tol = 1e-2 if dtype == torch.bfloat16 else 2e-3
+    print(f"families B={batch} {dtype} tiled={tiled}: plan flags {rl._plan.bound:#x}", flush=True)
+    for rep in range(3):
+        if rep:
+            for y in rl.outputs:
+                y.zero_()
+            ys = rl.run()
+            torch.cuda.synchronize()
+            assert rl.status() == 0
+        assert oracle.max_rel_err(ys[ia[2]].float().cpu().numpy(), ra[0] + ra[1] + ra[2]) < tol
+        assert oracle.max_rel_err(ys[ia[1]].cpu().numpy(), ra[0] + ra[1]) < tol          # fp32 partial sums
+        assert oracle.max_rel_err(ys[ib[1]].cpu().numpy(), rb[0] + rb[1]) < tol
+        assert oracle.max_rel_err(ys[ib[2]].float().cpu().numpy(), rb[0] + rb[2]) < tol   # onto the first term, not the second
+
+    # second term fed by an earlier linear's output: one phase later than the first term's second stage
+    rl2 = DecodeRunList(batch, dtype, dev)
+    i0, r0, _ = _weight_of_terms(dev, rl2, dtype, batch, 1024, 512, (128,), 720, tiled)
+    y0 = torch.from_numpy(r0[0]).to(dtype).to(dev)
+    to = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev).to(dtype)
+    f64 = lambda t: t.float().cpu().numpy().astype(np.float64)
+    words = lambda w: packing.binary_packer(torch.from_numpy(w), "half2").to(dev)
+    order = (lambda w: packing.tile_words(w)) if tiled else (lambda w: w)
+    xa = to(oracle.synth_x(batch, 1024, 730))
+    parts = []
+    for t, (r, xin, kw) in enumerate(((256, xa, dict(out_f32=True)),
+                                      (96, rl2.outputs[i0[0]], dict(x_from=i0[0])))):
+        vt, u, s_in, s_mid, s_out = oracle.synth_term(384, 1024, r, 731 + t)
+        sc = (to(s_in), to(s_mid), to(s_out))
+        if t == 1:
+            kw.update(addend=rl2.outputs[first], y_from=first)
+        k = rl2.add(xin, sc[0], order(words(vt)), sc[1], order(words(u)), sc[2], tiled=tiled, **kw)
+        if t == 0:
+            first = k
+        parts.append(oracle.layer_forward(f64(xa) if t == 0 else f64(y0), vt, u, f64(sc[0]), f64(sc[1]), f64(sc[2]),
+                                          dtype=np.float64))
+    ys2 = rl2.run()
+    torch.cuda.synchronize()
+    assert rl2.status() == 0
+    assert rl2._plan.nphases == 4, rl2._plan.nphases
+    assert oracle.max_rel_err(ys2[k].float().cpu().numpy(), parts[0] + parts[1]) < (2e-2 if dtype == torch.bfloat16 else 5e-3)
+
+
+@pytest.mark.parametrize("batch,dtype", [(1, torch.float16), (4, torch.float16), (16, torch.bfloat16)])
+def test_many_weights_of_two_and_three_terms(dev, batch, dtype):
+    # more families in the phase of the second stages than half the workgroups: the phase is cut by cost, a
+    # workgroup's share may begin and end inside a family, and every piece carries all terms of its rows
+    rng = np.random.default_rng(77 + batch)
+    rl = DecodeRunList(batch, dtype, dev)
+    want = []
+    for w in range(300):
+        m = int(rng.choice([64, 96, 160, 352]))
+        n = int(rng.choice([128, 256]))
+        ranks = tuple(int(v) for v in rng.choice([32, 64, 96], size=int(rng.integers(2, 4))))
+        idx, refs, _ = _weight_of_terms(dev, rl, dtype, batch, m, n, ranks, 9000 + 10 * w, True)
+        want.append((idx[-1], sum(refs)))
+    ys = rl.run()
+    torch.cuda.synchronize()
+    assert rl.status() == 0
+    assert rl._plan.nphases == 2
+    print(f"many families B={batch} {dtype}: workgroups {rl._plan.workgroups} plan flags {rl._plan.bound:#x}", flush=True)
+    for rep in range(2):
+        if rep:
+            ys = rl.run()
+            torch.cuda.synchronize()
+            assert rl.status() == 0
+        worst = max(oracle.max_rel_err(ys[i].float().cpu().numpy(), ref) for i, ref in want)
+        assert worst < (2e-2 if dtype == torch.bfloat16 else 1e-2), worst
+
+
 @pytest.mark.parametrize("batch", [1, 8, 16])
 def test_bf16_and_ragged_shapes(dev, batch):
     # ranks 70 and 2985 and 4100 columns: intermediate rows that allow no 16-byte loads (element-wise staging at every
