@@ -186,7 +186,7 @@ int nq_runlist_set_deterministic(nq_runlist_plan* plan, int on);
  * of the first in the same grid, fetch their first sign words, and wait on flags until their linear's h is complete
  * (workgroups start in the order of their ids, so whatever a workgroup waits for is running or done: no resident
  * grid is needed).  On MI355X the signalling through device-coherent memory costs more than the launch boundary it
- * replaces (a Llama-2-7B layer at batch 1 in four groups: 104 us with one launch per group, 53 us with two); the
+ * replaces (a Llama-2-7B layer at batch 1 in four groups: 82 us with one launch per group, 48 us with two); the
  * switch is kept for measurement and for callers that are charged per launch.  Its flags live in a device
  * array inside the library (4.5 MiB per GPU, 256 slots dealt round robin, every launch puts its slot back to zero);
  * the first call on each device looks up its address and should be made outside graph capture.  The wait is bounded

@@ -276,8 +276,9 @@ static int pick_group_log2(int units, int rows, int batch, double grid_cap = 153
         for (int gl = 0; gl <= 6; ++gl) {
             const int G = 1 << gl;
             const int passes = (units + G - 1) / G;
+            // more workgroups than stay resident run in rounds: beyond the cap a larger grid counts for less, not the same
             double grid = (double)rows / (4 * (kWave / G));
-            if (grid > grid_cap) grid = grid_cap;
+            if (grid > grid_cap) grid = grid_cap * (grid_cap / grid);
             const double score = (double)units / (double)(G * passes) * grid;
             if (score > best_score * 1.001) { best_score = score; best = gl; }
         }
@@ -457,6 +458,11 @@ static void fill_stage(StageArgs& a, bool first, const uint32_t* bits, const voi
     a.group_log2 = pick_group_log2(a.chunk_units, rows, batch, grid_cap);
 }
 
+// Workgroups that the lane-group choice of a group launch aims at, shared out by packed words (a single linear aims at
+// 1536): fewer, larger workgroups stage the input vectors less often (Llama-2-7B layer at batch 1 as {q,k,v} {o}
+// {gate,up} {down}: 53 us per layer at 1536, 48.5 at 512 .. 768, 50.7 at 384).
+constexpr double kGroupGridCap = 768.0;
+
 // y_i = s_out_i * (U_i (s_mid_i * (Vt_i (s_in_i * x_i)))) for `count` independent linears (<= gemv_fused_max());
 // batch 1, 2 or 4 rows; h_i: fp32 [batch, r_i] scratch of the caller.  Two launches (all first stages, then all second
 // stages), or with `one_launch` a single one whose second-stage workgroups wait inside the kernel.
@@ -476,8 +482,8 @@ hipError_t gemv_fused(int dtype, int count, int batch, const void* const* x, con
     }
     for (int i = 0; i < kFusedMax; ++i) {
         const int q = i < count ? i : count - 1;
-        const double cap_a = 1536.0 * ((double)r[q] * ((n[q] + 31) / 32)) / (words_a > 0 ? words_a : 1.0);
-        const double cap_b = 1536.0 * ((double)m[q] * ((r[q] + 31) / 32)) / (words_b > 0 ? words_b : 1.0);
+        const double cap_a = kGroupGridCap * ((double)r[q] * ((n[q] + 31) / 32)) / (words_a > 0 ? words_a : 1.0);
+        const double cap_b = kGroupGridCap * ((double)m[q] * ((r[q] + 31) / 32)) / (words_b > 0 ? words_b : 1.0);
         fill_stage(f.a[i], true, vt_bits[q], x[q], s_in[q], s_mid[q], h[q], nullptr, batch, r[q], (n[q] + 31) / 32, n[q], n[q], r[q],
                    cap_a < 64.0 ? 64.0 : cap_a);
         fill_stage(f.b[i], false, u_bits[q], h[q], nullptr, s_out[q], y[q], bias ? bias[q] : nullptr, batch, m[q], (r[q] + 31) / 32,
